@@ -1,0 +1,299 @@
+// Stand-alone Walsh-Hadamard transform over the last dimension (mi_fwht), gfx950.
+//
+// Bandwidth-bound: one 16-byte load and one 16-byte store per 8 (2-byte) or 4 (4-byte) elements,
+// everything in between on the matrix cores (tile_transform) plus a few fp32 butterflies.
+//
+//   n <= 512          : a wavefront transforms NT independent 512-element tiles (several rows
+//                       per tile; masked Hadamard operands).
+//   1024 <= n <= 4096 : one wavefront per row; n/512 tiles in registers, the tile-index bits by
+//                       fp32 butterflies between accumulators.
+//   n >= 8192         : one workgroup per row; each wavefront transforms 4096 contiguous
+//                       elements as above, then the remaining bits are gathered into registers
+//                       through one LDS exchange (write once, read once).
+//
+// Behaviour replaced: run_fht<dtype>() and its kernels, csrc/main.cu:12-122 and
+// HadaCore/hadamard_transform_cuda.cu:90-746 (normalised FWHT, n = 2..2^15).
+#include "fwht_device.hpp"
+
+namespace mi {
+namespace {
+
+// ---- element I/O -------------------------------------------------------------------------------
+// Each IO policy loads a lane's share of one tile into MFMA input form and stores two f32x4
+// accumulators back, both guarded against the end of the buffer (`total` elements).
+
+template <class T16_>
+struct Io16 {
+    using T16 = T16_;
+    using E = typename T16::E;
+    static constexpr int ESIZE = 2;
+    struct In {
+        typename T16::V8 a;
+    };
+
+    static __device__ __forceinline__ In load(const void* base, uint64_t tile, uint64_t total)
+    {
+        const E* p = static_cast<const E*>(base);
+        const uint64_t off = tile * 512u + 8u * (threadIdx.x & 63u);
+        In in;
+        if (off + 8u <= total) {
+            in.a = *reinterpret_cast<const typename T16::V8*>(p + off);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) in.a[j] = (off + j < total) ? p[off + j] : (E)0.0f;
+        }
+        return in;
+    }
+
+    static __device__ __forceinline__ void transform(const In& in, const TileOperands<T16>& ops,
+                                                     f32x4 (&acc)[2])
+    {
+        tile_transform<T16>(in.a, ops, acc);
+    }
+
+    static __device__ __forceinline__ void store(void* base, uint64_t tile, uint64_t total,
+                                                 const f32x4 (&acc)[2], float s)
+    {
+        E* p = static_cast<E*>(base);
+        const uint64_t off = tile * 512u + 8u * (threadIdx.x & 63u);
+        typename T16::V8 o;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[4 * t + r] = (E)(acc[t][r] * s);
+        if (off + 8u <= total) {
+            *reinterpret_cast<typename T16::V8*>(p + off) = o;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (off + j < total) p[off + j] = o[j];
+        }
+    }
+};
+
+struct Io32 {
+    using T16 = BF16;  // matrix-core type used for the three-piece products
+    static constexpr int ESIZE = 4;
+    struct In {
+        float v[8];
+    };
+
+    static __device__ __forceinline__ In load(const void* base, uint64_t tile, uint64_t total)
+    {
+        const float* p = static_cast<const float*>(base);
+        In in;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const uint64_t off = tile * 512u + 256u * t + 4u * (threadIdx.x & 63u);
+            if (off + 4u <= total) {
+                const f32x4 q = *reinterpret_cast<const f32x4*>(p + off);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) in.v[4 * t + r] = q[r];
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) in.v[4 * t + r] = (off + r < total) ? p[off + r] : 0.0f;
+            }
+        }
+        return in;
+    }
+
+    static __device__ __forceinline__ void transform(const In& in, const TileOperands<BF16>& ops,
+                                                     f32x4 (&acc)[2])
+    {
+        tile_transform_f32(in.v, ops, acc);
+    }
+
+    static __device__ __forceinline__ void store(void* base, uint64_t tile, uint64_t total,
+                                                 const f32x4 (&acc)[2], float s)
+    {
+        float* p = static_cast<float*>(base);
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const uint64_t off = tile * 512u + 256u * t + 4u * (threadIdx.x & 63u);
+            const f32x4 o = acc[t] * s;
+            if (off + 4u <= total) {
+                *reinterpret_cast<f32x4*>(p + off) = o;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (off + r < total) p[off + r] = o[r];
+            }
+        }
+    }
+};
+
+// ---- register kernel: NT tiles per wavefront, XB cross-tile bits ------------------------------
+template <class IO, int NT, int XB>
+__global__ void __launch_bounds__(256)
+fwht_reg_kernel(const void* in, void* out, uint64_t total, uint64_t num_waves, uint32_t p,
+                float fscale)
+{
+    // `in` may equal `out`: a wavefront reads all of its tiles before it writes any, and
+    // wavefronts own disjoint tiles, which is what makes in-place operation safe.
+    const uint64_t wave = (uint64_t)blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (wave >= num_waves) return;  // uniform per wavefront
+
+    TileOperands<typename IO::T16> ops;
+    make_tile_operands<typename IO::T16, IO::ESIZE>(p, ops);
+
+    typename IO::In tin[NT];
+#pragma unroll
+    for (int c = 0; c < NT; ++c) tin[c] = IO::load(in, wave * NT + c, total);
+
+    f32x4 acc[NT][2];
+#pragma unroll
+    for (int c = 0; c < NT; ++c) IO::transform(tin[c], ops, acc[c]);
+
+    cross_tile_butterflies<NT, XB>(acc);
+
+#pragma unroll
+    for (int c = 0; c < NT; ++c) IO::store(out, wave * NT + c, total, acc[c], fscale);
+}
+
+// ---- LDS kernel: one workgroup of W = 2^LW wavefronts per row of n = 4096 * W ----------------
+// Pass 1: wavefront w transforms elements [4096w, 4096w+4096) (12 bits).  Exchange: every
+// accumulator quad goes to LDS once; wavefront w then gathers, from all W sub-rows, the 8/W tiles
+// it owns, runs the LW remaining butterflies in registers and stores.
+template <class IO, int LW>
+__global__ void __launch_bounds__(64 << LW)
+fwht_lds_kernel(const void* in, void* out, uint64_t rows, float fscale)
+{
+    constexpr int W = 1 << LW;
+    constexpr int OWN = 8 / W;  // tiles per sub-row owned by a wavefront in pass 2
+    extern __shared__ f32x4 xch[];  // [W sub-rows][8 tiles][2 halves][64 lanes]
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t w = threadIdx.x >> 6;
+    const uint64_t row = blockIdx.x;
+    if (row >= rows) return;
+    const uint64_t total = rows << (12 + LW);
+    const uint64_t tile0 = row * (8u * W);
+
+    TileOperands<typename IO::T16> ops;
+    make_tile_operands<typename IO::T16, IO::ESIZE>(12 + LW, ops);
+
+    {
+        typename IO::In tin[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) tin[c] = IO::load(in, tile0 + w * 8u + c, total);
+        f32x4 acc[8][2];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) IO::transform(tin[c], ops, acc[c]);
+        cross_tile_butterflies<8, 3>(acc);
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+#pragma unroll
+            for (int t = 0; t < 2; ++t) xch[((w * 8u + c) * 2u + t) * 64u + lane] = acc[c][t];
+    }
+    __syncthreads();
+
+    f32x4 g[W * OWN][2];  // index s * OWN + c'
+#pragma unroll
+    for (int s = 0; s < W; ++s)
+#pragma unroll
+        for (int cc = 0; cc < OWN; ++cc)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+                g[s * OWN + cc][t] = xch[((s * 8u + w * OWN + cc) * 2u + t) * 64u + lane];
+
+    // butterflies over the sub-row index s (element bits 12 .. 12+LW-1)
+#pragma unroll
+    for (int b = 0; b < LW; ++b)
+#pragma unroll
+        for (int s = 0; s < W; ++s) {
+            if (s & (1 << b)) continue;
+#pragma unroll
+            for (int cc = 0; cc < OWN; ++cc)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const f32x4 x = g[s * OWN + cc][t], y = g[(s | (1 << b)) * OWN + cc][t];
+                    g[s * OWN + cc][t] = x + y;
+                    g[(s | (1 << b)) * OWN + cc][t] = x - y;
+                }
+        }
+
+#pragma unroll
+    for (int s = 0; s < W; ++s)
+#pragma unroll
+        for (int cc = 0; cc < OWN; ++cc)
+            IO::store(out, tile0 + s * 8u + w * OWN + cc, total, g[s * OWN + cc], fscale);
+}
+
+// ---- host dispatch --------------------------------------------------------------------------------
+template <class IO, int NT, int XB>
+int launch_reg(const void* in, void* out, uint64_t total, uint64_t num_waves, uint32_t p,
+               float fscale, hipStream_t s)
+{
+    const uint64_t blocks = (num_waves + 3u) / 4u;
+    if (blocks == 0) return MI_OK;
+    if (blocks > 0x7fffffffull) return MI_ERR_SHAPE;
+    hipLaunchKernelGGL((fwht_reg_kernel<IO, NT, XB>), dim3((uint32_t)blocks), dim3(256), 0, s, in,
+                       out, total, num_waves, p, fscale);
+    return launch_status();
+}
+
+template <class IO, int LW>
+int launch_lds(const void* in, void* out, uint64_t rows, float fscale, hipStream_t s)
+{
+    if (rows == 0) return MI_OK;
+    if (rows > 0x7fffffffull) return MI_ERR_SHAPE;
+    constexpr size_t lds = sizeof(f32x4) * 64u * 16u * (1u << LW);
+    auto kern = fwht_lds_kernel<IO, LW>;
+    if (lds > 64u * 1024u) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+            return MI_ERR_LAUNCH;
+    }
+    hipLaunchKernelGGL(kern, dim3((uint32_t)rows), dim3(64u << LW), lds, s, in, out, rows, fscale);
+    return launch_status();
+}
+
+template <class IO>
+int dispatch(const void* in, void* out, uint64_t rows, uint32_t n, float scale, hipStream_t s)
+{
+    const uint32_t p = ilog2(n);
+    const uint64_t total = rows * (uint64_t)n;
+    const int shift = tile_stage_shift<IO::ESIZE>(p);
+    const float fscale = (float)((double)scale * (double)(1u << shift));
+    if (p <= 9) {
+        const uint64_t tiles = (total + 511u) / 512u;
+        // several independent tiles per wavefront once there is enough work to fill the chip
+        if (tiles >= 4u * 16384u)
+            return launch_reg<IO, 4, 0>(in, out, total, (tiles + 3u) / 4u, p, fscale, s);
+        return launch_reg<IO, 1, 0>(in, out, total, tiles, p, fscale, s);
+    }
+    switch (p) {
+        case 10: return launch_reg<IO, 2, 1>(in, out, total, rows, p, fscale, s);
+        case 11: return launch_reg<IO, 4, 2>(in, out, total, rows, p, fscale, s);
+        case 12: return launch_reg<IO, 8, 3>(in, out, total, rows, p, fscale, s);
+        case 13: return launch_lds<IO, 1>(in, out, rows, fscale, s);
+        case 14: return launch_lds<IO, 2>(in, out, rows, fscale, s);
+        case 15: return launch_lds<IO, 3>(in, out, rows, fscale, s);
+        default: return MI_ERR_SIZE;
+    }
+}
+
+}  // namespace
+}  // namespace mi
+
+extern "C" int mi_fwht(const void* in, void* out, uint64_t rows, uint32_t n, int dtype, float scale,
+                       void* stream)
+{
+    using namespace mi;
+    if (!is_pow2(n) || n > 32768u) return MI_ERR_SIZE;
+    if (rows == 0) return MI_OK;
+    if (!in || !out) return MI_ERR_NULL;
+    if (!aligned16(in) || !aligned16(out)) return MI_ERR_ALIGN;
+    const size_t esize = dtype == MI_F32 ? 4 : 2;
+    if (in != out) {
+        const uintptr_t a = (uintptr_t)in, b = (uintptr_t)out;
+        const uint64_t bytes = rows * (uint64_t)n * esize;
+        if (a < b + bytes && b < a + bytes) return MI_ERR_ALIAS;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case MI_F32: return dispatch<Io32>(in, out, rows, n, scale, s);
+        case MI_BF16: return dispatch<Io16<BF16>>(in, out, rows, n, scale, s);
+        case MI_F16: return dispatch<Io16<F16>>(in, out, rows, n, scale, s);
+        default: return MI_ERR_DTYPE;
+    }
+}

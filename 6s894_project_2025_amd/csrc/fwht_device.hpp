@@ -1,0 +1,194 @@
+// Wave-level Hadamard building block for gfx950: transforms the 9 low index bits of a
+// 512-element tile on the matrix cores, with no cross-lane data movement.
+//
+// Role of the reference's device-callable seam
+//   HadamardTransform<dtype,N>::hadamard_transform_device(in, out, sm)   csrc/hada_handler.cuh:227-264
+// but built for 64-wide wavefronts and MFMA register layouts rather than mma.sync fragments.
+//
+// Layout algebra.  One wavefront holds a tile of 512 elements, 8 per lane.  Name the lane bits
+// lo = lane & 15, hi = lane >> 4 and the per-lane slot j = 0..7.  A *tile map* says which element
+// index bit each of those positions carries:
+//     2-byte elements:  j -> e0 e1 e2,   lo -> e3..e6,   hi -> e7 e8   (lane l holds e = 8l + j)
+//     4-byte elements:  j -> e0 e1 e8,   lo -> e2..e5,   hi -> e6 e7   (two 16-byte loads / lane)
+// Stage 1 is v_mfma_f32_16x16x32 with the data as the A operand (row = lo, K = 8*hi + j) and a
+// masked Hadamard matrix G1 as B.  It transforms the five K bits and, because the MFMA result
+// layout puts rows on (hi, r) and columns on lo, it leaves the untouched lo bits on (hi, r).
+// Stage 2 is v_mfma_f32_16x16x16 with the stage-1 result reused *as the A operand* (which reads
+// it transposed) against G2: it transforms those four bits and moves the stage-1 bits back to
+// (hi, r).  The column order of G1 is chosen so that after stage 2 lane l again holds
+// e = 8l + j (resp. the 4-byte map): the result layout equals the load layout, stores are
+// 16-byte and coalesced, and in-place operation is safe.
+//
+// Bits >= log2(n) are masked out of G1/G2 (identity), so one tile can hold several short rows.
+// Both stages carry a power-of-two factor (exact) that keeps 16-bit intermediates in range; the
+// caller folds the inverse into its final scale via tile_stage_gain().
+#pragma once
+
+#include "common.hpp"
+
+namespace mi {
+
+template <int ESIZE>
+struct TileMap;
+
+template <>
+struct TileMap<2> {
+    // element bit carried by canonical stage-1 bit q (q0..q2 = j bits, q3..q4 = hi bits)
+    static constexpr int qe[5] = {0, 1, 2, 7, 8};
+    static constexpr int lo_e0 = 3;  // lo bits carry e3..e6
+};
+
+template <>
+struct TileMap<4> {
+    static constexpr int qe[5] = {0, 1, 8, 6, 7};
+    static constexpr int lo_e0 = 2;  // lo bits carry e2..e5
+};
+
+// Masks of the stage-1 (5 canonical bits) and stage-2 (4 bits) index bits that lie inside a
+// transform of length 2^p.
+template <int ESIZE>
+__host__ __device__ inline void tile_masks(uint32_t p, uint32_t& mask1, uint32_t& mask2)
+{
+    constexpr int qe[5] = {TileMap<ESIZE>::qe[0], TileMap<ESIZE>::qe[1], TileMap<ESIZE>::qe[2],
+                           TileMap<ESIZE>::qe[3], TileMap<ESIZE>::qe[4]};
+    mask1 = 0;
+    for (int b = 0; b < 5; ++b)
+        if ((uint32_t)qe[b] < p) mask1 |= 1u << b;
+    mask2 = 0;
+    for (int b = 0; b < 4; ++b)
+        if ((uint32_t)(TileMap<ESIZE>::lo_e0 + b) < p) mask2 |= 1u << b;
+}
+
+// log2 of the (power-of-two) attenuation the two MFMA stages apply for a transform of length 2^p.
+template <int ESIZE>
+__host__ __device__ inline int tile_stage_shift(uint32_t p)
+{
+    uint32_t m1, m2;
+    tile_masks<ESIZE>(p, m1, m2);
+    return (__builtin_popcount(m1) >> 1) + (__builtin_popcount(m2) >> 1);
+}
+
+// Per-lane Hadamard operands for the two stages.
+template <class T16>
+struct TileOperands {
+    typename T16::V8 g1[2];  // stage-1 B operand for output halves t = 0, 1
+    typename T16::V4 g2;     // stage-2 B operand
+};
+
+template <class T16, int ESIZE>
+__device__ __forceinline__ void make_tile_operands(uint32_t p, TileOperands<T16>& ops)
+{
+    using E = typename T16::E;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t lo = lane & 15u, hi = lane >> 4;
+    uint32_t mask1, mask2;
+    tile_masks<ESIZE>(p, mask1, mask2);
+    const float c1 = __builtin_ldexpf(1.0f, -(__popc(mask1) >> 1));
+    const float c2 = __builtin_ldexpf(1.0f, -(__popc(mask2) >> 1));
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const uint32_t np = 16u * t + lo;  // stage-1 output column
+        // column -> canonical bits: n'0->q0, n'1->q1, n'2->q3, n'3->q4, n'4->q2
+        const uint32_t qn = (np & 3u) | (((np >> 2) & 1u) << 3) | (((np >> 3) & 1u) << 4) |
+                            (((np >> 4) & 1u) << 2);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t qk = 8u * hi + j;
+            ops.g1[t][j] = (E)masked_hadamard_entry(qk, qn, mask1, c1);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ops.g2[j] = (E)masked_hadamard_entry(4u * hi + j, lo, mask2, c2);
+}
+
+template <class T16>
+__device__ __forceinline__ typename T16::V4 narrow4(f32x4 v)
+{
+    using E = typename T16::E;
+    typename T16::V4 r;
+    r[0] = (E)v[0];
+    r[1] = (E)v[1];
+    r[2] = (E)v[2];
+    r[3] = (E)v[3];
+    return r;
+}
+
+// 16-bit tile: `a` = the lane's 8 elements.  Result acc[t][r] = element 8*lane + 4t + r.
+template <class T16>
+__device__ __forceinline__ void tile_transform(typename T16::V8 a, const TileOperands<T16>& ops,
+                                               f32x4 (&acc)[2])
+{
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        f32x4 d1 = T16::mfma32(a, ops.g1[t], zero);
+        acc[t] = T16::mfma16(narrow4<T16>(d1), ops.g2, zero);
+    }
+}
+
+// Exact three-way split of fp32 into bf16 pieces (8 + 8 + 8 significand bits): x = h + m + l.
+__device__ __forceinline__ void split3(float x, __bf16& h, __bf16& m, __bf16& l)
+{
+    h = (__bf16)x;
+    const float r = x - (float)h;
+    m = (__bf16)r;
+    l = (__bf16)(r - (float)m);
+}
+
+// fp32 tile on the bf16 matrix cores: every stage multiplies the three bf16 pieces of its input
+// by the +-2^-k Hadamard operand and accumulates in fp32, so each product is exact and the only
+// rounding is the fp32 accumulation.  v[j] = the lane's 8 elements under TileMap<4>.
+// Result acc[t][r] = element 256t + 4*lane + r.
+__device__ __forceinline__ void tile_transform_f32(const float (&v)[8],
+                                                   const TileOperands<BF16>& ops, f32x4 (&acc)[2])
+{
+    bf16x8 h, m, l;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        __bf16 a, b, c;
+        split3(v[j], a, b, c);
+        h[j] = a;
+        m[j] = b;
+        l[j] = c;
+    }
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        f32x4 d1 = BF16::mfma32(l, ops.g1[t], zero);
+        d1 = BF16::mfma32(m, ops.g1[t], d1);
+        d1 = BF16::mfma32(h, ops.g1[t], d1);
+        bf16x4 h2, m2, l2;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            __bf16 a, b, c;
+            split3(d1[r], a, b, c);
+            h2[r] = a;
+            m2[r] = b;
+            l2[r] = c;
+        }
+        f32x4 d2 = BF16::mfma16(l2, ops.g2, zero);
+        d2 = BF16::mfma16(m2, ops.g2, d2);
+        acc[t] = BF16::mfma16(h2, ops.g2, d2);
+    }
+}
+
+// In-register butterflies over XB tile-index bits (element bits 9 .. 9+XB-1) of NT tiles.
+template <int NT, int XB>
+__device__ __forceinline__ void cross_tile_butterflies(f32x4 (&acc)[NT][2])
+{
+#pragma unroll
+    for (int b = 0; b < XB; ++b) {
+#pragma unroll
+        for (int c = 0; c < NT; ++c) {
+            if (c & (1 << b)) continue;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const f32x4 x = acc[c][t], y = acc[c | (1 << b)][t];
+                acc[c][t] = x + y;
+                acc[c | (1 << b)][t] = x - y;
+            }
+        }
+    }
+}
+
+}  // namespace mi

@@ -1,0 +1,145 @@
+/*
+ * mi_hadamard.h -- C ABI of the MI355X (gfx950) fast Hadamard transform library.
+ *
+ * Plain pointers and sizes only; no torch or HIP types appear in the signatures (`stream` is a
+ * hipStream_t passed as void*, NULL = the null stream).  Every entry point
+ *   - enqueues its kernels on `stream` and returns without synchronising,
+ *   - allocates no device memory and keeps no mutable global state (safe from any host thread),
+ *   - returns MI_OK (0) or a negative mi_status; mi_status_string() turns it into text.
+ * All matrices are dense row-major with no padding between rows.
+ */
+#ifndef MI_HADAMARD_H
+#define MI_HADAMARD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum mi_dtype {
+    MI_F32 = 0,
+    MI_BF16 = 1,
+    MI_F16 = 2,
+} mi_dtype;
+
+typedef enum mi_status {
+    MI_OK = 0,
+    MI_ERR_DTYPE = -1,     /* dtype code not supported by this entry point            */
+    MI_ERR_SIZE = -2,      /* transform length not a power of two in the valid range  */
+    MI_ERR_ALIGN = -3,     /* a pointer is not 16-byte aligned                        */
+    MI_ERR_NULL = -4,      /* a required pointer is NULL                              */
+    MI_ERR_SHAPE = -5,     /* a dimension violates the entry point's tiling contract  */
+    MI_ERR_LAUNCH = -6,    /* hipGetLastError() reported a launch failure             */
+    MI_ERR_ALIAS = -7,     /* input/output overlap that the entry point cannot honour */
+} mi_status;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int mi_version(void);
+
+/* Text for a status code; never NULL. */
+const char* mi_status_string(int status);
+
+/*
+ * Walsh-Hadamard transform over the last dimension:  out[r, :] = scale * H_n * in[r, :]
+ * for r in [0, rows), H_n the Sylvester matrix H[i][j] = (-1)^popcount(i & j).
+ *
+ * Replaces the reference's internal seam
+ *     template<DType> void run_fht(void* a, void* out, uint32_t numel, uint32_t had_size,
+ *                                  cudaStream_t)                 csrc/main.cuh:5-6,
+ *                                                                HadaCore/hadamard_transform.cpp:8-9
+ * which its pybind op hadamard_transform(x, inplace) calls (csrc/hadamard_transform.cpp:49-59).
+ * Differences: `rows` is 64-bit (the reference's numel is u32); any row count is accepted (the
+ * reference pads numel to a multiple of 256 first, csrc/hadamard_transform.cpp:31-39); fp32 is
+ * accepted; `scale` is explicit (the reference hard-wires n^-1/2 in its kernel constants,
+ * HadaCore/hadamard_transform_cuda.cu:139-142).
+ *
+ *   in, out : device pointers, 16-byte aligned, rows*n elements; in == out is allowed
+ *             (in place); partial overlap is not.
+ *   n       : power of two, 1 <= n <= 32768.
+ *   dtype   : mi_dtype.  bf16/fp16 accumulate in fp32 on the matrix cores and round to the
+ *             storage type between MFMA stages and at the store; fp32 stays fp32 throughout.
+ */
+int mi_fwht(const void* in, void* out, uint64_t rows, uint32_t n, int dtype, float scale,
+            void* stream);
+
+/*
+ * Fused Hadamard + GEMV-batch:  Y[M,B] = W[M,N] * (scale * H_N * X[N,B]),
+ * the transform running down each column of X (dimension 0).
+ *
+ * Replaces  fused_hadamard_gemv_kernel(const float* W, const float* X, float* Y, int M, int N,
+ * int B)  and its _vec variant, fused_ht/fwht_gemv_fusion.cu:98-105,176-183, launched from
+ * benchmark_fused (:371-420).  Layouts are the ones that file indexes: X[i*B + b] (:50-51),
+ * W[row*N + k] (:146), Y[row*B + b] (:156).  scale = 1 reproduces the reference (raw +-1
+ * butterfly, :118-133).
+ *
+ *   dtype : MI_F32 only.   N : power of two, 2 <= N <= 4096.   M, B >= 1.
+ *   Y must not overlap W or X.
+ */
+int mi_fused_ht_gemv(const void* W, const void* X, void* Y, uint32_t M, uint32_t N, uint32_t B,
+                     int dtype, float scale, void* stream);
+
+/*
+ * Fused Hadamard -> GEMM:  C[M,N] = W[M,K] * (scale * H_K * X[K,N]),  X given as Xt[N,K]
+ * (each logical column of X contiguous).  The transformed operand never goes to HBM.
+ *
+ * Replaces  fused_ht_gemm_pipelined(const float* X, const float* W, float* C)  with compile-time
+ * KDIM/NDIM/MDIM, fused_ht/fusion_pipelined.cu:306-310, launched at :662-683.  Layouts:
+ * X[col*KDIM + k] (:164,612), W[row*KDIM + k] (:211,498), C[row*NDIM + col] (:220,558).
+ * scale = 1 reproduces the reference.
+ *
+ *   in_dtype  : MI_F32 (fp32 MFMA) or MI_BF16 / MI_F16 (16-bit MFMA, fp32 accumulate).
+ *   out_dtype : MI_F32, or the same 16-bit type as in_dtype.
+ *   K : power of two, 16 <= K <= 4096.   M, N >= 1 (edge tiles are masked).
+ */
+int mi_fused_ht_gemm(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
+                     int in_dtype, int out_dtype, float scale, void* stream);
+
+/*
+ * Randomized Hadamard + FP8 quantize:  y[t,:] = scale * H_n * (sign .* x[t,:]) rounded to bf16,
+ * then per row   amax = max|y|,  a = max(amax, 1e-30f),  row_scale[t] = a / 448,
+ * q[t,j] = e4m3fn_rne(clamp(y[t,j] * (448 / a), -448, 448))   (OCP E4M3FN; IEEE fp32 ops).
+ *
+ * No counterpart in the reference (it has no FP8 path); part of the build contract's hot path.
+ *
+ *   x         : bf16 [T,n];  n power of two, 16 <= n <= 4096... see mi_status on violation.
+ *   sign      : int8 [n], entries +1 / -1.
+ *   q         : uint8 [T,n] E4M3FN codes.      row_scale : fp32 [T] (dequantisation factors).
+ *   y_out     : optional bf16 [T,n] dump of the pre-quant values (NULL to skip).
+ */
+int mi_rht_quant_fp8(const void* x, const int8_t* sign, void* q, float* row_scale, void* y_out,
+                     uint64_t T, uint32_t n, float scale, void* stream);
+
+/*
+ * FP8 GEMM with per-row scales:  out[T,N] = bf16( (qa[T,K] . qb[N,K]^T) * sa[t] * sb[n] ),
+ * E4M3FN operands, fp32 accumulate.  No counterpart in the reference.
+ *   K multiple of 128;  T, N >= 1.
+ */
+int mi_fp8_gemm_rowscale(const void* qa, const float* sa, const void* qb, const float* sb,
+                         void* out, uint32_t T, uint32_t N, uint32_t K, void* stream);
+
+/*
+ * One-wavefront MFMA layout check:  D[16,16] = A[16,Kk] * B[Kk,16]  with exactly one matrix-core
+ * instruction, operands gathered under the register layout the kernels assume.
+ * Mirrors the reference's test hook  test_mma_m16_n8_k16(x, y)  (csrc/test_frag.cu:8-62,
+ * exported at csrc/hadamard_transform.cpp:83-89).
+ *   kind 0: v_mfma_f32_16x16x32_bf16 (Kk = 32)    kind 1: v_mfma_f32_16x16x16_bf16 (Kk = 16)
+ *   kind 2: v_mfma_f32_16x16x32_f16  (Kk = 32)    kind 3: v_mfma_f32_16x16x16_f16  (Kk = 16)
+ *   kind 4: v_mfma_f32_16x16x4_f32   (Kk = 4, A and B fp32)
+ *   A, B: row-major, element type per kind;  D: fp32 row-major.
+ */
+int mi_debug_mfma_16x16(int kind, const void* A, const void* B, float* D, void* stream);
+
+/*
+ * Element-wise narrowing conversions as the kernels perform them (hardware RNE), for unit tests
+ * (the reference's  test_bit_convert, csrc/test_bit.cu:8-42).
+ *   kind 0: fp32 -> bf16 bits (uint16)    kind 1: fp32 -> fp16 bits (uint16)
+ *   kind 2: fp32 -> E4M3FN code (uint8), input clamped to +-448 first
+ */
+int mi_debug_convert(int kind, const float* in, void* out, uint64_t count, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI_HADAMARD_H */

@@ -1,0 +1,185 @@
+"""GPU parity of the stand-alone transform against the fp64 oracle, through the C ABI.
+
+Tolerances (metric max|y - y64| / max|y64|): fp32 <= 1e-5, bf16/fp16 <= 2e-2 (build contract);
+plus the reference's own absolute bars against the matrix product in the tensor's dtype,
+allclose(atol=1e-2 fp16 / 5e-2 bf16, rtol=0), HadaCore/test.py:91,97."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+ATOL_REF = {torch.float16: 1e-2, torch.bfloat16: 5e-2}
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+ALL_N = [1 << p for p in range(0, 16)]
+
+
+def _check(pkg, oracle, x_cpu, scale=None, inplace=False):
+    x = x_cpu.cuda()
+    y = pkg.hadamard_transform(x, scale, inplace=inplace)
+    torch.cuda.synchronize()
+    y64 = oracle.fwht_f64(x_cpu.to(torch.float64).numpy(), scale)
+    err = oracle.rel_err(y.cpu().to(torch.float64).numpy(), y64)
+    assert err <= TOL[x_cpu.dtype], f"rel err {err} n={x_cpu.shape[-1]} {x_cpu.dtype}"
+    return y, err
+
+
+@pytest.mark.parametrize("kind,K,dt", [(0, 32, torch.bfloat16), (1, 16, torch.bfloat16),
+                                       (2, 32, torch.float16), (3, 16, torch.float16),
+                                       (4, 4, torch.float32)])
+def test_one_wave_mfma_layout(pkg, kind, K, dt):
+    # the analogue of test/test_mma.py:5-9: one matrix-core instruction == A @ B
+    from importlib import import_module
+    lib = import_module(pkg.__name__ + "._lib").load()
+    g = torch.Generator().manual_seed(kind)
+    A = torch.randn(16, K, generator=g).to(dt)
+    B = torch.randn(K, 16, generator=g).to(dt)
+    D = torch.zeros(16, 16, dtype=torch.float32, device="cuda")
+    Ad, Bd = A.cuda(), B.cuda()
+    st = lib.mi_debug_mfma_16x16(kind, Ad.data_ptr(), Bd.data_ptr(), D.data_ptr(), None)
+    assert st == 0
+    torch.cuda.synchronize()
+    want = A.double() @ B.double()
+    assert torch.allclose(D.cpu().double(), want, atol=1e-4, rtol=1e-5)
+
+
+def test_hardware_conversions_match_oracle(pkg, oracle):
+    from importlib import import_module
+    lib = import_module(pkg.__name__ + "._lib").load()
+    hi = np.arange(0, 1 << 16, dtype=np.uint32) << 16
+    lows = np.array([0, 1, 0x7FFF, 0x8000, 0x8001, 0xFFFF, 0x1000, 0xF000], dtype=np.uint32)
+    x = (hi[:, None] | lows[None, :]).reshape(-1).view(np.float32)
+    x = x[np.isfinite(x)]
+    xd = torch.from_numpy(x.copy()).cuda()
+    for kind, enc in [(0, oracle.f32_to_bf16), (1, oracle.f32_to_f16)]:
+        out = torch.empty(x.size, dtype=torch.int16, device="cuda")
+        assert lib.mi_debug_convert(kind, xd.data_ptr(), out.data_ptr(), x.size, None) == 0
+        torch.cuda.synchronize()
+        got = out.cpu().numpy().view(np.uint16)
+        want = enc(x)
+        # fp16 subnormal flushing is not expected: compare all bits
+        assert np.array_equal(got, want), f"kind {kind}: {(got != want).sum()} mismatches"
+    out = torch.empty(x.size, dtype=torch.uint8, device="cuda")
+    assert lib.mi_debug_convert(2, xd.data_ptr(), out.data_ptr(), x.size, None) == 0
+    torch.cuda.synchronize()
+    want = oracle.e4m3fn_encode(np.clip(x, -448.0, 448.0))
+    got = out.cpu().numpy()
+    assert np.array_equal(got, want), f"fp8: {(got != want).sum()} mismatches"
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=str)
+@pytest.mark.parametrize("n", ALL_N)
+def test_all_sizes_small_rows(pkg, oracle, n, dt):
+    rows = 7 if n <= 4096 else 3
+    x = oracle.inputs_fwht(rows, n, dt)
+    _check(pkg, oracle, x)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=str)
+@pytest.mark.parametrize("n,rows", [(16, 4099), (64, 1031), (256, 513), (512, 300), (1024, 130),
+                                    (4096, 67), (8192, 9), (32768, 5), (2, 3), (4, 1), (8, 5)])
+def test_ragged_row_counts(pkg, oracle, n, rows, dt):
+    # numel not a multiple of 256 / 512: the reference pads (csrc/hadamard_transform.cpp:31-39)
+    x = oracle.inputs_fwht(rows, n, dt)
+    _check(pkg, oracle, x)
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=str)
+@pytest.mark.parametrize("n", [2, 16, 256, 4096, 32768])
+def test_reference_absolute_tolerance(pkg, oracle, n, dt):
+    # HadaCore/test.py:80-97: randn fp32 -> dtype, op in place, vs a @ H.to(dtype)
+    rows = max(1, (1 << 15) // n)
+    x = oracle.inputs_fwht(rows, n, dt)
+    xd = x.cuda()
+    out = pkg.hadamard_transform(xd, inplace=True)
+    assert out.data_ptr() == xd.data_ptr()
+    torch.cuda.synchronize()
+    truth = oracle.hadamard_matrix_ref(x.to(torch.float32)).to(dt)
+    assert torch.allclose(truth.float(), xd.cpu().float(), atol=ATOL_REF[dt], rtol=0)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=str)
+def test_scale_argument_and_unnormalised(pkg, oracle, dt):
+    x = oracle.inputs_fwht(33, 256, dt)
+    _check(pkg, oracle, x, scale=1.0)
+    _check(pkg, oracle, x, scale=0.37)
+    _check(pkg, oracle, x, scale=None)
+
+
+def test_binding_semantics(pkg, oracle):
+    x = oracle.inputs_fwht(6 * 5, 128, torch.bfloat16).reshape(6, 5, 128).cuda()
+    y = pkg.hadamard_transform(x)
+    assert y.shape == x.shape and y.data_ptr() != x.data_ptr()
+    x0 = x.clone()
+    z = pkg.hadamard_transform(x, inplace=True)
+    assert z is x
+    assert torch.equal(z, y)
+    # non-contiguous input: transposed view, last dim strided
+    base = oracle.inputs_fwht(64, 48, torch.float32).cuda()
+    v = base.t()  # [48, 64], stride (1, 48)
+    assert not v.is_contiguous()
+    want = pkg.hadamard_transform(v.contiguous())
+    got = pkg.hadamard_transform(v)
+    assert torch.equal(got, want)
+    v2 = base.clone().t()
+    pkg.hadamard_transform(v2, inplace=True)
+    assert torch.equal(v2, want)
+    # row-strided slice (dense last dim, padded rows) and a misaligned view
+    wide = oracle.inputs_fwht(10, 64, torch.float16).cuda()
+    sl = wide[:, :32]
+    assert torch.equal(pkg.hadamard_transform(sl), pkg.hadamard_transform(sl.contiguous()))
+    mis = wide.reshape(-1)[4:4 + 128].reshape(4, 32)
+    assert mis.data_ptr() % 16 != 0
+    assert torch.equal(pkg.hadamard_transform(mis), pkg.hadamard_transform(mis.clone()))
+    mis_before = mis.clone()
+    pkg.hadamard_transform(mis, inplace=True)
+    assert torch.equal(mis, pkg.hadamard_transform(mis_before))
+    # empty
+    e = torch.empty(0, 64, dtype=torch.bfloat16, device="cuda")
+    assert pkg.hadamard_transform(e).shape == (0, 64)
+    del x0
+
+
+def test_errors(pkg):
+    with pytest.raises(RuntimeError, match="supported"):
+        pkg.hadamard_transform(torch.zeros(4, 8, dtype=torch.float64, device="cuda"))
+    with pytest.raises(RuntimeError):
+        pkg.hadamard_transform(torch.zeros(4, 8, dtype=torch.bfloat16))  # CPU tensor
+    with pytest.raises(RuntimeError, match="power of two"):
+        pkg.hadamard_transform(torch.zeros(4, 24, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(RuntimeError, match="power of two"):
+        pkg.hadamard_transform(torch.zeros(1, 1 << 16, dtype=torch.bfloat16, device="cuda"))
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=str)
+def test_involution_at_full_size(pkg, dt):
+    # BASELINE config 2 shape: [16384, 4096]; the normalised transform is its own inverse and
+    # preserves the row norms (size-independent properties, checked on the device)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(16384, 4096, generator=g, dtype=torch.float32).to(dt).cuda()
+    y = pkg.hadamard_transform(x)
+    z = pkg.hadamard_transform(y)
+    tol = 1e-5 if dt == torch.float32 else 2e-2
+    num = (z.float() - x.float()).abs().max().item()
+    den = x.float().abs().max().item()
+    assert num / den <= tol
+    nx = x.float().norm(dim=1)
+    ny = y.float().norm(dim=1)
+    assert ((ny - nx).abs() / nx).max().item() <= (1e-5 if dt == torch.float32 else 5e-3)
+    # first 64 rows against the oracle would need /root/reference-free fp64 math: done on device
+    H = None
+    del H
+
+
+def test_full_size_rows_against_oracle(pkg, oracle):
+    # a slice of the full-size bf16 problem against the fp64 oracle
+    x = oracle.inputs_fwht(16384, 4096, torch.bfloat16)
+    xd = x.cuda()
+    pkg.hadamard_transform(xd, inplace=True)
+    torch.cuda.synchronize()
+    idx = [0, 1, 2, 3, 4095, 8191, 8192, 16383]
+    y64 = oracle.fwht_f64(x[idx].to(torch.float64).numpy())
+    assert oracle.rel_err(xd[idx].cpu().to(torch.float64).numpy(), y64) <= 2e-2
