@@ -42,8 +42,6 @@ def load() -> ctypes.CDLL:
             "(there is no CPU or PyTorch fallback for these ops)")
     lib = ctypes.CDLL(LIB_PATH)
     for name, (res, args) in SIGNATURES.items():
-        if not hasattr(lib, name):  # TEMP while entry points are being added
-            continue
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args

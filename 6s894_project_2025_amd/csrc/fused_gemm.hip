@@ -1,0 +1,281 @@
+// Fused Hadamard -> GEMM (mi_fused_ht_gemm), gfx950:  C[M,N] = W[M,K] * (scale * H_K * X[K,N]),
+// X given as Xt[N,K].  The transformed operand lives only in LDS.
+//
+// Structure ("X-stationary"): a workgroup owns BN columns of X for the whole K extent.
+//   prologue : its wavefronts transform those BN rows of Xt on the matrix cores (tile_transform,
+//              the stand-alone kernel's building block), round to the 16-bit type and park
+//              them in LDS as Y[BN][K] (16-byte chunks XOR-swizzled so that both the prologue's
+//              writes and the main loop's fragment reads are bank-conflict free);
+//   main loop: each wavefront takes 64-row blocks of W inside the workgroup's M range, streams
+//              them from global memory straight into MFMA operand registers (8 contiguous K per
+//              lane) and contracts against Y fragments read from LDS with
+//              v_mfma_f32_16x16x32; Y is the A operand and W the B operand, so a lane ends up
+//              with 16 consecutive output columns of one row of C and stores them as 16-byte
+//              vectors.
+// The M range is split over gridDim.y workgroups so that the chip is filled.
+//
+// Behaviour replaced: fused_ht_gemm_pipelined, fused_ht/fusion_pipelined.cu:306-563 (cp.async
+// double-buffered X tile + in-smem butterfly + scalar-FMA GEMM; fp32 only, compile-time dims).
+#include "fwht_device.hpp"
+
+namespace mi {
+namespace {
+
+constexpr int kGemmThreads = 512;
+constexpr int kGemmWaves = kGemmThreads / 64;
+
+template <class T16>
+struct OutStore {
+    // 16 consecutive columns of one row, fp32 accumulators -> `out_f32 ? float : T16::E`
+    static __device__ __forceinline__ void row16(void* C, bool out_f32, uint64_t row, uint32_t ldc,
+                                                 uint32_t col0, uint32_t ncols, const float (&v)[16])
+    {
+        using E = typename T16::E;
+        if (out_f32) {
+            float* p = static_cast<float*>(C) + row * ldc + col0;
+            if (ncols >= 16 && (ldc & 3u) == 0) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    f32x4 o = {v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
+                    *reinterpret_cast<f32x4*>(p + 4 * q) = o;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    if ((uint32_t)i < ncols) p[i] = v[i];
+            }
+        } else {
+            E* p = static_cast<E*>(C) + row * ldc + col0;
+            if (ncols >= 16 && (ldc & 7u) == 0) {
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    typename T16::V8 o;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) o[i] = (E)v[8 * q + i];
+                    *reinterpret_cast<typename T16::V8*>(p + 8 * q) = o;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    if ((uint32_t)i < ncols) p[i] = (E)v[i];
+            }
+        }
+    }
+};
+
+// Byte offset of 16-byte chunk q of column n in the swizzled Y[BN][K] LDS image.
+// `col_bytes` = bytes per column, LOG_NB = log2(16-column fragments per block): the fragment
+// read of lane `lo` touches column NB*lo + nb, so the swizzle key is n / NB.
+template <int LOG_NB>
+__device__ __forceinline__ uint32_t y_chunk_offset(uint32_t n, uint32_t q, uint32_t col_bytes,
+                                                   uint32_t swz_mask)
+{
+    return n * col_bytes + ((q ^ ((n >> LOG_NB) & swz_mask)) << 4);
+}
+
+// XB = log2(max(K,512)/512): tiles per column that need cross-tile butterflies.
+template <class T16, int BN, int XB>
+__global__ void __launch_bounds__(kGemmThreads)
+fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16::E* __restrict__ Xt,
+                       void* __restrict__ C, uint32_t M, uint32_t N, uint32_t K, uint32_t logK,
+                       uint32_t m_per_block, int out_f32, float fscale)
+{
+    using E = typename T16::E;
+    using V8 = typename T16::V8;
+    constexpr int NB = BN / 16;  // 16-column fragments of Y (A-operand blocks)
+    constexpr int LOG_NB = NB == 4 ? 2 : (NB == 2 ? 1 : 0);
+    extern __shared__ __attribute__((aligned(16))) unsigned char ylds[];
+
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t lo = lane & 15u, hi = lane >> 4;
+    const uint32_t n0 = blockIdx.x * BN;
+    const uint32_t chunks_per_col = K >> 3;
+    const uint32_t swz_mask = (chunks_per_col >= 16u ? 16u : chunks_per_col) - 1u;
+
+    // ---- prologue: Y = bf16(scale * H_K * X[:, n0:n0+BN]) into LDS -------------------------------
+    {
+        TileOperands<T16> ops;
+        make_tile_operands<T16, 2>(logK, ops);
+        constexpr int NT = 1 << XB;                       // tiles per wavefront step
+        const uint32_t block_tiles = (BN * K) >> 9;       // 512-element tiles in this block
+        const uint64_t total = (uint64_t)N * K;           // elements in Xt
+        const uint64_t tile_base = ((uint64_t)n0 * K) >> 9;
+        for (uint32_t t0 = wave * NT; t0 < block_tiles; t0 += kGemmWaves * NT) {
+            V8 in[NT];
+#pragma unroll
+            for (int c = 0; c < NT; ++c) {
+                const uint64_t off = (tile_base + t0 + c) * 512u + 8u * lane;
+                if (off + 8u <= total) {
+                    in[c] = *reinterpret_cast<const V8*>(Xt + off);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) in[c][j] = (E)0.0f;  // columns past N
+                }
+            }
+            f32x4 acc[NT][2];
+#pragma unroll
+            for (int c = 0; c < NT; ++c) tile_transform<T16>(in[c], ops, acc[c]);
+            cross_tile_butterflies<NT, XB>(acc);
+#pragma unroll
+            for (int c = 0; c < NT; ++c) {
+                V8 o;
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) o[4 * t + r] = (E)(acc[c][t][r] * fscale);
+                const uint32_t e = (t0 + c) * 512u + 8u * lane;  // element offset in the block
+                const uint32_t n = e >> logK, q = (e & (K - 1u)) >> 3;
+                *reinterpret_cast<V8*>(ylds + y_chunk_offset<LOG_NB>(n, q, K * 2u, swz_mask)) = o;
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- main loop ------------------------------------------------------------------------------
+    const uint32_t m_begin = blockIdx.y * m_per_block;
+    const uint32_t m_end = min(M, m_begin + m_per_block);
+    const uint32_t ksteps = K >> 5;
+
+    for (uint32_t mb = m_begin + wave * 64u; mb < m_end; mb += kGemmWaves * 64u) {
+        f32x4 acc[NB][4];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi) acc[nb][mi] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+        const E* wrow[4];
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) {
+            const uint32_t m = min(mb + 16u * mi + lo, M - 1u);  // clamp: masked at the store
+            wrow[mi] = W + (uint64_t)m * K + 8u * hi;
+        }
+        V8 bcur[4], bnext[4];
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) bcur[mi] = *reinterpret_cast<const V8*>(wrow[mi]);
+
+        for (uint32_t ks = 0; ks < ksteps; ++ks) {
+            if (ks + 1 < ksteps) {
+#pragma unroll
+                for (int mi = 0; mi < 4; ++mi)
+                    bnext[mi] = *reinterpret_cast<const V8*>(wrow[mi] + 32u * (ks + 1));
+            }
+            V8 a[NB];
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+                a[nb] = *reinterpret_cast<const V8*>(
+                    ylds + y_chunk_offset<LOG_NB>(NB * lo + nb, 4u * ks + hi, K * 2u, swz_mask));
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int mi = 0; mi < 4; ++mi)
+                    acc[nb][mi] = T16::mfma32(a[nb], bcur[mi], acc[nb][mi]);
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi) bcur[mi] = bnext[mi];
+        }
+
+        // D[m'][n']: n' = lo is the row of W; m' = 4*hi + r is the A-operand lane, which carried
+        // column NB*m' + nb.  So this lane owns the contiguous run of 4*NB columns starting at
+        // 4*NB*hi, in the order v[NB*r + nb].
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) {
+            const uint32_t m = mb + 16u * mi + lo;
+            if (m >= m_end) continue;
+            float v[16];
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) v[NB * r + nb] = acc[nb][mi][r];
+            const uint32_t col0 = n0 + (4u * NB) * hi;
+            if (col0 < N) {
+                const uint32_t ncols = min((uint32_t)(4 * NB), N - col0);
+                if constexpr (NB == 4) {
+                    OutStore<T16>::row16(C, out_f32 != 0, m, N, col0, ncols, v);
+                } else {
+                    // narrower blocks: element-wise store
+#pragma unroll
+                    for (int i = 0; i < 4 * NB; ++i) {
+                        if ((uint32_t)i >= ncols) break;
+                        if (out_f32)
+                            static_cast<float*>(C)[(uint64_t)m * N + col0 + i] = v[i];
+                        else
+                            static_cast<E*>(C)[(uint64_t)m * N + col0 + i] = (E)v[i];
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <class T16, int BN, int XB>
+int launch_gemm16(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
+                  int out_f32, float scale, hipStream_t s)
+{
+    const uint32_t logK = ilog2(K);
+    const int shift = tile_stage_shift<2>(logK);
+    const float fscale = (float)((double)scale * (double)(1u << shift));
+    const uint32_t n_tiles = (N + BN - 1) / BN;
+    // split M so that about two workgroups per compute unit exist; each covers a multiple of
+    // 512 rows (8 wavefronts x 64 rows)
+    const uint32_t row_blocks = (M + 511u) / 512u;
+    uint32_t msplit = (512u + n_tiles - 1u) / n_tiles;
+    if (msplit < 1u) msplit = 1u;
+    if (msplit > row_blocks) msplit = row_blocks;
+    const uint32_t m_per_block = ((row_blocks + msplit - 1u) / msplit) * 512u;
+    msplit = (M + m_per_block - 1u) / m_per_block;
+    const size_t lds = (size_t)BN * K * 2u;
+    auto kern = fused_ht_gemm16_kernel<T16, BN, XB>;
+    if (lds > 64u * 1024u) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+            return MI_ERR_LAUNCH;
+    }
+    hipLaunchKernelGGL(kern, dim3(n_tiles, msplit), dim3(kGemmThreads), lds, s,
+                       static_cast<const typename T16::E*>(W),
+                       static_cast<const typename T16::E*>(Xt), C, M, N, K, logK, m_per_block,
+                       out_f32, fscale);
+    return launch_status();
+}
+
+template <class T16>
+int dispatch_gemm16(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
+                    int out_f32, float scale, hipStream_t s)
+{
+    switch (K) {
+        case 32:
+        case 64:
+        case 128:
+        case 256:
+        case 512: return launch_gemm16<T16, 64, 0>(W, Xt, C, M, N, K, out_f32, scale, s);
+        case 1024: return launch_gemm16<T16, 64, 1>(W, Xt, C, M, N, K, out_f32, scale, s);
+        case 2048: return launch_gemm16<T16, 32, 2>(W, Xt, C, M, N, K, out_f32, scale, s);
+        case 4096: return launch_gemm16<T16, 16, 3>(W, Xt, C, M, N, K, out_f32, scale, s);
+        default: return MI_ERR_SIZE;
+    }
+}
+
+}  // namespace
+
+int fused_gemm_f32(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, uint32_t K,
+                   float scale, hipStream_t s);  // fused_gemm_f32.hip
+
+}  // namespace mi
+
+extern "C" int mi_fused_ht_gemm(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N,
+                                uint32_t K, int in_dtype, int out_dtype, float scale, void* stream)
+{
+    using namespace mi;
+    if (!is_pow2(K) || K < 32u || K > 4096u) return MI_ERR_SIZE;
+    if (M == 0 || N == 0) return MI_OK;
+    if (!W || !Xt || !C) return MI_ERR_NULL;
+    if (!aligned16(W) || !aligned16(Xt) || !aligned16(C)) return MI_ERR_ALIGN;
+    if (out_dtype != MI_F32 && out_dtype != in_dtype) return MI_ERR_DTYPE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (in_dtype) {
+        case MI_F32:
+            return fused_gemm_f32(static_cast<const float*>(W), static_cast<const float*>(Xt),
+                                  static_cast<float*>(C), M, N, K, scale, s);
+        case MI_BF16: return dispatch_gemm16<BF16>(W, Xt, C, M, N, K, out_dtype == MI_F32, scale, s);
+        case MI_F16: return dispatch_gemm16<F16>(W, Xt, C, M, N, K, out_dtype == MI_F32, scale, s);
+        default: return MI_ERR_DTYPE;
+    }
+}

@@ -1,0 +1,180 @@
+// fp32 variant of the fused Hadamard -> GEMM (see fused_gemm.hip for the structure).
+//
+// The transformed tile Y[BN][K] is kept in LDS as fp32; the prologue runs the fp32 transform on
+// the bf16 matrix cores with exact three-piece operands (tile_transform_f32), and the
+// contraction uses the fp32 matrix-core instruction v_mfma_f32_16x16x4_f32, so every product
+// and sum is fp32 (there is no reduced-precision shortcut on this hardware).
+// One 16-byte load per lane supplies four consecutive K for four MFMAs: lane (lo, hi) of K-step
+// kk holds k = 16*kk + 4*hi + s, s = 0..3, for both operands.
+#include "fwht_device.hpp"
+
+namespace mi {
+namespace {
+
+constexpr int kThreads = 512;
+constexpr int kWaves = kThreads / 64;
+
+template <int LOG_NB>
+__device__ __forceinline__ uint32_t y_off(uint32_t n, uint32_t q, uint32_t col_bytes,
+                                          uint32_t swz_mask)
+{
+    return n * col_bytes + ((q ^ ((n >> LOG_NB) & swz_mask)) << 4);
+}
+
+template <int BN, int XB>
+__global__ void __launch_bounds__(kThreads)
+fused_ht_gemm_f32_kernel(const float* __restrict__ W, const float* __restrict__ Xt,
+                         float* __restrict__ C, uint32_t M, uint32_t N, uint32_t K, uint32_t logK,
+                         uint32_t m_per_block, float fscale)
+{
+    constexpr int NB = BN / 16;
+    constexpr int LOG_NB = NB == 4 ? 2 : (NB == 2 ? 1 : 0);
+    extern __shared__ __attribute__((aligned(16))) unsigned char ylds[];
+
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t lo = lane & 15u, hi = lane >> 4;
+    const uint32_t n0 = blockIdx.x * BN;
+    const uint32_t chunks_per_col = K >> 2;
+    const uint32_t swz_mask = (chunks_per_col >= 16u ? 16u : chunks_per_col) - 1u;
+    const uint32_t col_bytes = K * 4u;
+
+    {
+        TileOperands<BF16> ops;
+        make_tile_operands<BF16, 4>(logK, ops);
+        constexpr int NT = 1 << XB;
+        const uint32_t block_tiles = (BN * K) >> 9;
+        const uint64_t total = (uint64_t)N * K;
+        const uint64_t tile_base = ((uint64_t)n0 * K) >> 9;
+        for (uint32_t t0 = wave * NT; t0 < block_tiles; t0 += kWaves * NT) {
+            float in[NT][8];
+#pragma unroll
+            for (int c = 0; c < NT; ++c)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const uint64_t off = (tile_base + t0 + c) * 512u + 256u * t + 4u * lane;
+                    f32x4 q = {0.f, 0.f, 0.f, 0.f};
+                    if (off + 4u <= total) q = *reinterpret_cast<const f32x4*>(Xt + off);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) in[c][4 * t + r] = q[r];
+                }
+            f32x4 acc[NT][2];
+#pragma unroll
+            for (int c = 0; c < NT; ++c) tile_transform_f32(in[c], ops, acc[c]);
+            cross_tile_butterflies<NT, XB>(acc);
+#pragma unroll
+            for (int c = 0; c < NT; ++c)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const uint32_t e = (t0 + c) * 512u + 256u * t + 4u * lane;
+                    const uint32_t n = e >> logK, q = (e & (K - 1u)) >> 2;
+                    *reinterpret_cast<f32x4*>(ylds + y_off<LOG_NB>(n, q, col_bytes, swz_mask)) =
+                        acc[c][t] * fscale;
+                }
+        }
+    }
+    __syncthreads();
+
+    const uint32_t m_begin = blockIdx.y * m_per_block;
+    const uint32_t m_end = min(M, m_begin + m_per_block);
+    const uint32_t ksteps = K >> 4;
+
+    for (uint32_t mb = m_begin + wave * 64u; mb < m_end; mb += kWaves * 64u) {
+        f32x4 acc[NB][4];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi) acc[nb][mi] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const float* wrow[4];
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) {
+            const uint32_t m = min(mb + 16u * mi + lo, M - 1u);
+            wrow[mi] = W + (uint64_t)m * K + 4u * hi;
+        }
+        f32x4 bcur[4], bnext[4];
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) bcur[mi] = *reinterpret_cast<const f32x4*>(wrow[mi]);
+
+        for (uint32_t kk = 0; kk < ksteps; ++kk) {
+            if (kk + 1 < ksteps) {
+#pragma unroll
+                for (int mi = 0; mi < 4; ++mi)
+                    bnext[mi] = *reinterpret_cast<const f32x4*>(wrow[mi] + 16u * (kk + 1));
+            }
+            f32x4 a[NB];
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+                a[nb] = *reinterpret_cast<const f32x4*>(
+                    ylds + y_off<LOG_NB>(NB * lo + nb, 4u * kk + hi, col_bytes, swz_mask));
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                    for (int mi = 0; mi < 4; ++mi)
+                        acc[nb][mi] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[nb][s], bcur[mi][s],
+                                                                           acc[nb][mi], 0, 0, 0);
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi) bcur[mi] = bnext[mi];
+        }
+
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) {
+            const uint32_t m = mb + 16u * mi + lo;
+            if (m >= m_end) continue;
+            const uint32_t col0 = n0 + (4u * NB) * hi;
+            if (col0 >= N) continue;
+            const uint32_t ncols = min((uint32_t)(4 * NB), N - col0);
+            float* p = C + (uint64_t)m * N + col0;
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+                    if ((uint32_t)(NB * r + nb) < ncols) p[NB * r + nb] = acc[nb][mi][r];
+        }
+    }
+}
+
+template <int BN, int XB>
+int launch(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, uint32_t K,
+           float scale, hipStream_t s)
+{
+    const uint32_t logK = ilog2(K);
+    const int shift = tile_stage_shift<4>(logK);
+    const float fscale = (float)((double)scale * (double)(1u << shift));
+    const uint32_t n_tiles = (N + BN - 1) / BN;
+    const uint32_t row_blocks = (M + 511u) / 512u;
+    uint32_t msplit = (512u + n_tiles - 1u) / n_tiles;
+    if (msplit < 1u) msplit = 1u;
+    if (msplit > row_blocks) msplit = row_blocks;
+    const uint32_t m_per_block = ((row_blocks + msplit - 1u) / msplit) * 512u;
+    msplit = (M + m_per_block - 1u) / m_per_block;
+    const size_t lds = (size_t)BN * K * 4u;
+    auto kern = fused_ht_gemm_f32_kernel<BN, XB>;
+    if (lds > 64u * 1024u) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+            return MI_ERR_LAUNCH;
+    }
+    hipLaunchKernelGGL(kern, dim3(n_tiles, msplit), dim3(kThreads), lds, s, W, Xt, C, M, N, K, logK,
+                       m_per_block, fscale);
+    return launch_status();
+}
+
+}  // namespace
+
+int fused_gemm_f32(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, uint32_t K,
+                   float scale, hipStream_t s)
+{
+    switch (K) {
+        case 32:
+        case 64:
+        case 128:
+        case 256:
+        case 512: return launch<32, 0>(W, Xt, C, M, N, K, scale, s);
+        case 1024: return launch<32, 1>(W, Xt, C, M, N, K, scale, s);
+        case 2048: return launch<16, 2>(W, Xt, C, M, N, K, scale, s);
+        default: return MI_ERR_SIZE;  // fp32 tile of K = 4096 does not fit in LDS
+    }
+}
+
+}  // namespace mi

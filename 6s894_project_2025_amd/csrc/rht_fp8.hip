@@ -1,0 +1,239 @@
+// Randomized Hadamard + FP8 (OCP E4M3FN) quantize epilogue (mi_rht_quant_fp8) and the FP8 GEMM
+// with per-row scales (mi_fp8_gemm_rowscale), gfx950.  The reference has no FP8 path; the
+// arithmetic convention is the one stated in include/mi_hadamard.h.
+//
+// Quantize kernel: same skeleton as the stand-alone transform (one 16-byte load per 8 elements,
+// two MFMA stages per 512-element tile, fp32 butterflies across tiles), with
+//   - the +-1 diagonal folded into the load as a sign-bit XOR (exact),
+//   - the result rounded to bf16 exactly as mi_fwht would store it (so the codes equal
+//     quantising mi_fwht's output), the row amax taken over those bf16 values by a lane
+//     reduction over the lanes that share a row,
+//   - v_cvt_pk_fp8_f32 for the narrowing (hardware RNE to E4M3FN), 8 codes = one 8-byte store.
+// Bandwidth-bound: 2 bytes in, 1 byte (+ 4 bytes per row) out per element.
+#include "fwht_device.hpp"
+
+namespace mi {
+namespace {
+
+constexpr float kFp8Max = 448.0f;
+constexpr float kAmaxFloor = 1e-30f;
+
+// NT tiles per wavefront; XB cross-tile bits (n = 512 << XB when XB > 0, else n <= 512 and the
+// NT tiles are independent).
+template <int NT, int XB>
+__global__ void __launch_bounds__(256)
+rht_quant_fp8_kernel(const __bf16* __restrict__ x, const int8_t* __restrict__ sign,
+                     uint8_t* __restrict__ q, float* __restrict__ row_scale,
+                     __bf16* __restrict__ y_out, uint64_t total, uint64_t num_waves, uint32_t p,
+                     float fscale)
+{
+    const uint64_t wave = (uint64_t)blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (wave >= num_waves) return;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t n = 1u << p;
+
+    TileOperands<BF16> ops;
+    make_tile_operands<BF16, 2>(p, ops);
+
+    // load + sign flip
+    bf16x8 in[NT];
+#pragma unroll
+    for (int c = 0; c < NT; ++c) {
+        const uint64_t off = (wave * NT + c) * 512u + 8u * lane;
+        u32x4 bits = {0u, 0u, 0u, 0u};
+        if (off + 8u <= total) bits = *reinterpret_cast<const u32x4*>(x + off);
+        const uint32_t col = (uint32_t)(off & (uint64_t)(n - 1u));
+        const u32x2 sg = *reinterpret_cast<const u32x2*>(sign + col);  // 8 int8, +1 / -1
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const uint32_t s2 = (w < 2 ? sg[0] : sg[1]) >> (16 * (w & 1));
+            // byte 0 -> element 2w, byte 1 -> element 2w+1; -1 = 0xff has bit 7 set
+            const uint32_t flip = ((s2 & 0x80u) << 8) | ((s2 & 0x8000u) << 16);
+            bits[w] ^= flip;
+        }
+        in[c] = __builtin_bit_cast(bf16x8, bits);
+    }
+
+    f32x4 acc[NT][2];
+#pragma unroll
+    for (int c = 0; c < NT; ++c) tile_transform<BF16>(in[c], ops, acc[c]);
+    cross_tile_butterflies<NT, XB>(acc);
+
+    // round to bf16 (the pre-quant values), amax per row
+    bf16x8 y[NT];
+    float amax[NT];
+#pragma unroll
+    for (int c = 0; c < NT; ++c) {
+        float m = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const __bf16 b = (__bf16)(acc[c][t][r] * fscale);
+                y[c][4 * t + r] = b;
+                m = fmaxf(m, fabsf((float)b));
+            }
+        amax[c] = m;
+    }
+    // lanes that share a row: lane bit i carries element bit 3 + i, so the low min(6, p - 3)
+    // lane bits index inside a row
+    const uint32_t row_lane_bits = p >= 9u ? 6u : p - 3u;
+#pragma unroll
+    for (int c = 0; c < NT; ++c) {
+        float m = amax[c];
+        for (uint32_t b = 0; b < row_lane_bits; ++b) m = fmaxf(m, __shfl_xor(m, 1 << b, 64));
+        amax[c] = m;
+    }
+    if (XB > 0) {  // one row spans all NT tiles
+        float m = amax[0];
+#pragma unroll
+        for (int c = 1; c < NT; ++c) m = fmaxf(m, amax[c]);
+#pragma unroll
+        for (int c = 0; c < NT; ++c) amax[c] = m;
+    }
+
+#pragma unroll
+    for (int c = 0; c < NT; ++c) {
+        const uint64_t off = (wave * NT + c) * 512u + 8u * lane;
+        if (off + 8u > total) continue;
+        const float a = fmaxf(amax[c], kAmaxFloor);
+        const float inv = kFp8Max / a;
+        // first lane of each row writes the dequantisation factor
+        const bool row_head = XB > 0 ? (c == 0 && lane == 0) : ((off & (uint64_t)(n - 1u)) == 0);
+        if (row_head) row_scale[off >> p] = a / kFp8Max;
+        u32x2 codes;
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                v[i] = __builtin_amdgcn_fmed3f((float)y[c][4 * w + i] * inv, -kFp8Max, kFp8Max);
+            int pk = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
+            pk = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], pk, true);
+            codes[w] = (uint32_t)pk;
+        }
+        *reinterpret_cast<u32x2*>(q + off) = codes;
+        if (y_out) *reinterpret_cast<bf16x8*>(y_out + off) = y[c];
+    }
+}
+
+template <int NT, int XB>
+int launch_quant(const void* x, const int8_t* sign, void* q, float* rs, void* y_out, uint64_t total,
+                 uint64_t num_waves, uint32_t p, float fscale, hipStream_t s)
+{
+    const uint64_t blocks = (num_waves + 3u) / 4u;
+    if (blocks > 0x7fffffffull) return MI_ERR_SHAPE;
+    hipLaunchKernelGGL((rht_quant_fp8_kernel<NT, XB>), dim3((uint32_t)blocks), dim3(256), 0, s,
+                       static_cast<const __bf16*>(x), sign, static_cast<uint8_t*>(q), rs,
+                       static_cast<__bf16*>(y_out), total, num_waves, p, fscale);
+    return launch_status();
+}
+
+// ---- FP8 GEMM, per-row scales -----------------------------------------------------------------------
+// out[t][n] = bf16( sum_k a[t][k] * b[n][k] * sa[t] * sb[n] ).  Workgroup tile 128 x 128, four
+// wavefronts of 64 x 64, operands read K-contiguously (8 codes per lane per MFMA) with
+// v_mfma_f32_16x16x32_fp8_fp8; qb rows play the A operand so that a lane owns consecutive
+// output columns.
+__global__ void __launch_bounds__(256)
+fp8_gemm_rowscale_kernel(const uint8_t* __restrict__ qa, const float* __restrict__ sa,
+                         const uint8_t* __restrict__ qb, const float* __restrict__ sb,
+                         __bf16* __restrict__ out, uint32_t T, uint32_t N, uint32_t K)
+{
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t lo = lane & 15u, hi = lane >> 4;
+    const uint32_t t0 = blockIdx.y * 128u + (wave >> 1) * 64u;
+    const uint32_t n0 = blockIdx.x * 128u + (wave & 1u) * 64u;
+    if (t0 >= T || n0 >= N) return;
+
+    // A operand: qb rows (columns of out), lane `lo` carries column n0 + 4*lo + nb
+    // B operand: qa rows, lane `lo` carries row t0 + 16*ti + lo
+    const uint8_t* prow_b[4];
+    const uint8_t* prow_a[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+        prow_b[nb] = qb + (uint64_t)min(n0 + 4u * lo + nb, N - 1u) * K + 8u * hi;
+#pragma unroll
+    for (int ti = 0; ti < 4; ++ti)
+        prow_a[ti] = qa + (uint64_t)min(t0 + 16u * ti + lo, T - 1u) * K + 8u * hi;
+
+    f32x4 acc[4][4];
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+        for (int ti = 0; ti < 4; ++ti) acc[nb][ti] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    for (uint32_t k = 0; k < K; k += 32u) {
+        long a[4], b[4];
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) a[nb] = *reinterpret_cast<const long*>(prow_b[nb] + k);
+#pragma unroll
+        for (int ti = 0; ti < 4; ++ti) b[ti] = *reinterpret_cast<const long*>(prow_a[ti] + k);
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+            for (int ti = 0; ti < 4; ++ti)
+                acc[nb][ti] =
+                    __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[nb], b[ti], acc[nb][ti], 0, 0, 0);
+    }
+
+    // D[m'][n']: n' = lo -> row t;  m' = 4*hi + r -> column n0 + 4*m' + nb = n0 + 16*hi + 4*r + nb
+#pragma unroll
+    for (int ti = 0; ti < 4; ++ti) {
+        const uint32_t t = t0 + 16u * ti + lo;
+        if (t >= T) continue;
+        const float st = sa[t];
+        const uint32_t col0 = n0 + 16u * hi;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb) {
+                const uint32_t col = col0 + 4u * r + nb;
+                if (col < N) out[(uint64_t)t * N + col] = (__bf16)(acc[nb][ti][r] * st * sb[col]);
+            }
+    }
+}
+
+}  // namespace
+}  // namespace mi
+
+extern "C" int mi_rht_quant_fp8(const void* x, const int8_t* sign, void* q, float* row_scale,
+                                void* y_out, uint64_t T, uint32_t n, float scale, void* stream)
+{
+    using namespace mi;
+    if (!is_pow2(n) || n < 16u || n > 4096u) return MI_ERR_SIZE;
+    if (T == 0) return MI_OK;
+    if (!x || !sign || !q || !row_scale) return MI_ERR_NULL;
+    if (!aligned16(x) || !aligned16(q) || (y_out && !aligned16(y_out)) ||
+        (reinterpret_cast<uintptr_t>(sign) & 7u))
+        return MI_ERR_ALIGN;
+    const uint32_t p = ilog2(n);
+    const uint64_t total = T * (uint64_t)n;
+    const int shift = tile_stage_shift<2>(p);
+    const float fscale = (float)((double)scale * (double)(1u << shift));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (p <= 9) {
+        const uint64_t tiles = (total + 511u) / 512u;
+        return launch_quant<1, 0>(x, sign, q, row_scale, y_out, total, tiles, p, fscale, s);
+    }
+    switch (p) {
+        case 10: return launch_quant<2, 1>(x, sign, q, row_scale, y_out, total, T, p, fscale, s);
+        case 11: return launch_quant<4, 2>(x, sign, q, row_scale, y_out, total, T, p, fscale, s);
+        default: return launch_quant<8, 3>(x, sign, q, row_scale, y_out, total, T, p, fscale, s);
+    }
+}
+
+extern "C" int mi_fp8_gemm_rowscale(const void* qa, const float* sa, const void* qb,
+                                    const float* sb, void* out, uint32_t T, uint32_t N, uint32_t K,
+                                    void* stream)
+{
+    using namespace mi;
+    if (K == 0 || (K & 127u)) return MI_ERR_SHAPE;
+    if (T == 0 || N == 0) return MI_OK;
+    if (!qa || !sa || !qb || !sb || !out) return MI_ERR_NULL;
+    if (!aligned16(qa) || !aligned16(qb) || !aligned16(out)) return MI_ERR_ALIGN;
+    const dim3 grid((N + 127u) / 128u, (T + 127u) / 128u);
+    hipLaunchKernelGGL(fp8_gemm_rowscale_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint8_t*>(qa), sa, static_cast<const uint8_t*>(qb), sb,
+                       static_cast<__bf16*>(out), T, N, K);
+    return launch_status();
+}
