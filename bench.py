@@ -1,0 +1,241 @@
+#!/usr/bin/env python3
+"""Benchmark of the Hadamard hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep] [--no-cpu]
+
+A *step* is one pass of the stand-alone transform over one batch: the in-place normalised FWHT of
+a bf16 X[16384, 4096] (BASELINE config 2), inputs resident in HBM before timing starts.  The
+protocol is the reference's (bench/bench.py:112-127): warm-up launches, then K back-to-back
+launches on the same buffer inside one event window on the launch stream.  One JSON line is
+printed; besides the headline it carries
+  roofline      - the transform kernel against the 8 TB/s HBM peak,
+  cpu_baseline  - the reference's truth path (x @ Sylvester matrix in torch, on the host cores)
+                  on a bounded row sample of the same workload,
+  fused_ht_gemm - C = W.H(X) at K=1024, M=N=4096 in bf16 against the dense bf16 MFMA peak,
+  others        - the remaining configurations (fp32 fused GEMM, HT+GEMV, RHT+FP8 quantize,
+                  FP8 GEMM), and with --sweep the n = 2^4..2^15 transform sweep.
+"""
+from __future__ import annotations
+
+import argparse
+import importlib
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+PEAK_TFLOPS = {"bf16": 2516.6, "f16": 2516.6, "f32": 157.3, "fp8": 5033.2}
+
+
+def _events_ms(torch, fn, steps, warmup):
+    """Average milliseconds per call: `warmup` untimed calls, then `steps` back-to-back calls
+    bracketed by events on the current stream and full synchronisation on both sides."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = torch.cuda.Event(enable_timing=True)
+    t1 = torch.cuda.Event(enable_timing=True)
+    w0 = time.perf_counter()
+    t0.record()
+    for _ in range(steps):
+        fn()
+    t1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - w0) * 1e3
+    return t0.elapsed_time(t1) / steps, wall_ms / steps
+
+
+def _load_traffic():
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), recorded in
+    profiles/hbm_traffic.json by hand from the committed summaries; None when absent."""
+    p = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(p):
+        with open(p) as f:
+            return json.load(f)
+    return {}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--sweep", action="store_true", help="also time n = 2^4..2^15 (128 MiB each)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only-fwht", action="store_true", help="headline kernel only (profiling)")
+    ap.add_argument("--only-gemm", action="store_true", help="fused GEMM only (profiling)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.stderr.write("bench.py: this build runs on exactly one GPU; --gpus must be 1 "
+                         "(rows shard across GPUs with no exchange, see DESIGN.md)\n")
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.stderr.write("bench.py: no GPU visible\n")
+        return 2
+    hada = importlib.import_module("6s894_project_2025_amd")
+    dev = torch.device("cuda:0")
+    traffic = _load_traffic()
+    steps, warmup = args.steps, args.warmup
+
+    # ---- headline: config 2 ---------------------------------------------------------------------
+    rows, n = 16384, 4096
+    g = torch.Generator().manual_seed(0)
+    x_cpu = torch.randn(rows, n, generator=g, dtype=torch.float32).to(torch.bfloat16)
+    result = {}
+    if not args.only_gemm:
+        x = x_cpu.to(dev)
+        ms, wall_ms = _events_ms(torch, lambda: hada.hadamard_transform(x, inplace=True), steps, warmup)
+        alg_bytes = 2 * rows * n * 2
+        gbs = alg_bytes / ms / 1e6
+        # size-independent sanity on the timed buffer: an even number of normalised transforms
+        # returns the input (up to bf16 rounding drift)
+        if (steps + warmup) % 2 == 1:
+            hada.hadamard_transform(x, inplace=True)
+        drift = (x.float() - x_cpu.to(dev).float()).abs().max().item()
+        add_ms, _ = _events_ms(torch, lambda: x.add_(1), min(steps, 50), 3)
+        result = {
+            "metric": "standalone FWHT HBM GB/s (bf16 [16384,4096], in place; half of the reference's "
+                      "compound metric, the fused HT+GEMM TFLOP/s half is under fused_ht_gemm)",
+            "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": round(ms, 6), "wall_ms_per_step": round(wall_ms, 6),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "BASELINE configs[1]: in-place normalised FWHT over the last dim, "
+                                   "bf16 X[16384,4096] iid N(0,1) seed 0, scale 1/64",
+                       "rows": rows, "n": n, "algorithmic_bytes_per_step": alg_bytes},
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                         "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                         "traffic": traffic.get("fwht_bf16_16384x4096"),
+                         "kernel": "fwht_reg_kernel<Io16<BF16>,8,3>",
+                         "add_one_proxy_gbs": round(alg_bytes / add_ms / 1e6, 1)},
+            "checks": {"max_abs_drift_after_even_number_of_transforms": drift},
+        }
+        del x
+        if args.only_fwht:
+            print(json.dumps(result))
+            return 0
+
+    # ---- fused HT -> GEMM, config 4 -----------------------------------------------------------------
+    M = N = 4096
+    K = 1024
+    gsteps = max(10, min(steps, 100))
+    others = {}
+    for name, dt in (("bf16", torch.bfloat16), ("f32", torch.float32)):
+        W = torch.randn(M, K, generator=torch.Generator().manual_seed(1)).to(dt).to(dev)
+        Xt = torch.randn(N, K, generator=torch.Generator().manual_seed(0)).to(dt).to(dev)
+        C = hada.fused_ht_gemm(W, Xt)
+        ms, _ = _events_ms(torch, lambda: hada.fused_ht_gemm(W, Xt), gsteps, 3)
+        flops = 2 * M * N * K
+        tf = flops / ms / 1e9
+        entry = {"metric": f"fused HT+GEMM TFLOP/s (K=1024, M=N=4096, {name}, fp32 accumulate, "
+                           f"C in {name})",
+                 "value": round(tf, 1), "unit": "TFLOP/s", "ms_per_step": round(ms, 6), "steps": gsteps,
+                 "algorithmic_flops_per_step": flops,
+                 "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_TFLOPS[name],
+                              "unit": "TFLOP/s", "frac": round(tf / PEAK_TFLOPS[name], 4),
+                              "traffic": traffic.get(f"fused_ht_gemm_{name}")}}
+        if name == "bf16":
+            mm_ms, _ = _events_ms(torch, lambda: torch.matmul(W, Xt.t()), gsteps, 3)
+            entry["library_gemm_without_transform_tflops"] = round(flops / mm_ms / 1e9, 1)
+            result["fused_ht_gemm"] = entry
+            if args.only_gemm:
+                print(json.dumps(entry))
+                return 0
+        else:
+            others["fused_ht_gemm_f32"] = entry
+        del W, Xt, C
+
+    # ---- remaining configurations --------------------------------------------------------------------
+    for (m, nn, b) in ((256, 256, 512), (1024, 1024, 8), (1024, 1024, 64), (1024, 1024, 512)):
+        W = torch.randn(m, nn, device=dev) / math.sqrt(nn)
+        X = torch.randn(nn, b, device=dev)
+        ms, _ = _events_ms(torch, lambda: hada.fused_ht_gemv(W, X), 50, 3)
+        others[f"fused_ht_gemv_M{m}_N{nn}_B{b}"] = {
+            "us": round(ms * 1e3, 2),
+            "algorithmic_bytes": 4 * (m * nn + nn * b + m * b),
+            "algorithmic_flops": 2 * m * nn * b + int(nn * math.log2(nn) * b),
+            "GB/s": round(4 * (m * nn + nn * b + m * b) / ms / 1e6, 1),
+            "TFLOP/s": round((2 * m * nn * b + nn * math.log2(nn) * b) / ms / 1e9, 3)}
+    T, nq, Nw = 8192, 4096, 14336
+    xa = torch.randn(T, nq, device=dev).to(torch.bfloat16)
+    sign = (1 - 2 * torch.randint(0, 2, (nq,), generator=torch.Generator().manual_seed(2))).to(torch.int8).to(dev)
+    ms, _ = _events_ms(torch, lambda: hada.rht_quant_fp8(xa, sign), 50, 3)
+    qbytes = T * nq * 3 + T * 4
+    others["rht_quant_fp8_8192x4096"] = {
+        "us": round(ms * 1e3, 2), "algorithmic_bytes": qbytes, "GB/s": round(qbytes / ms / 1e6, 1),
+        "roofline": {"bound": "hbm", "achieved": round(qbytes / ms / 1e6, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(qbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                     "traffic": traffic.get("rht_quant_fp8_8192x4096")}}
+    qx, sx = hada.rht_quant_fp8(xa, sign)
+    w = (torch.randn(Nw, nq, device=dev) * 0.02).to(torch.bfloat16)
+    qw, sw = hada.rht_quant_fp8(w, sign)
+    ms, _ = _events_ms(torch, lambda: hada.fp8_gemm_rowscale(qx, sx, qw, sw), 5, 1)
+    fl = 2 * T * Nw * nq
+    others["fp8_gemm_8192x14336x4096"] = {
+        "us": round(ms * 1e3, 1), "algorithmic_flops": fl, "TFLOP/s": round(fl / ms / 1e9, 1),
+        "roofline": {"bound": "mfma", "achieved": round(fl / ms / 1e9, 1), "peak": PEAK_TFLOPS["fp8"],
+                     "unit": "TFLOP/s", "frac": round(fl / ms / 1e9 / PEAK_TFLOPS["fp8"], 4),
+                     "traffic": None}}
+    del xa, w, qx, qw
+
+    if args.sweep:
+        sweep = {}
+        for dname, dt, es in (("bf16", torch.bfloat16, 2), ("f16", torch.float16, 2), ("f32", torch.float32, 4)):
+            for p in range(4, 16):
+                nn = 1 << p
+                numel = (128 << 20) // es
+                t = torch.randn(numel // nn, nn, device=dev).to(dt)
+                ms, _ = _events_ms(torch, lambda: hada.hadamard_transform(t, inplace=True), 50, 3)
+                sweep[f"{dname}_n{nn}"] = {"us": round(ms * 1e3, 2),
+                                           "GB/s": round(2 * numel * es / ms / 1e6, 1)}
+                del t
+        others["fwht_sweep_128MiB"] = sweep
+    result["others"] = others
+
+    # ---- CPU baseline: the reference's truth path on the host cores ---------------------------------
+    if not args.no_cpu:
+        import oracle  # CPU restatement: only this leg uses it
+
+        nthreads = torch.get_num_threads()
+        sample = 64
+        xs = x_cpu[:sample].clone()
+        oracle.hadamard_matrix_ref(xs)  # builds the matrix, warms the thread pool
+        t0 = time.perf_counter()
+        oracle.hadamard_matrix_ref(xs)
+        est = time.perf_counter() - t0
+        # grow the sample so that the timed region is roughly 10 s of host work
+        sample = int(max(64, min(rows, 64 * (10.0 / max(est, 1e-3)) / 4)))
+        xs = x_cpu[:sample].clone()
+        import scipy.linalg
+
+        H = (torch.tensor(scipy.linalg.hadamard(n), dtype=torch.float32) / math.sqrt(n)).to(torch.bfloat16)
+        for _ in range(1):
+            xs @ H
+        reps = 3
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            xs @ H
+        dt_s = (time.perf_counter() - t0) / reps
+        result["cpu_baseline"] = {
+            "value": round(2 * sample * n * 2 / dt_s / 1e9, 4), "unit": "GB/s", "cores": nthreads,
+            "kind": "port",
+            "sample": f"torch CPU x @ (hadamard(4096)/64).to(bf16) on the first {sample} of 16384 rows "
+                      f"(matrix built once, untimed), mean of {reps} calls; os.cpu_count()={os.cpu_count()}",
+            "ms_for_sample": round(dt_s * 1e3, 3),
+            "ms_extrapolated_full_batch": round(dt_s * 1e3 * rows / sample, 1)}
+
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
