@@ -6,12 +6,17 @@
 //              the stand-alone kernel's building block), round to the 16-bit type and park
 //              them in LDS as Y[BN][K] (16-byte chunks XOR-swizzled so that both the prologue's
 //              writes and the main loop's fragment reads are bank-conflict free);
-//   main loop: each wavefront takes 64-row blocks of W inside the workgroup's M range, streams
-//              them from global memory straight into MFMA operand registers (8 contiguous K per
-//              lane) and contracts against Y fragments read from LDS with
-//              v_mfma_f32_16x16x32; Y is the A operand and W the B operand, so a lane ends up
-//              with 16 consecutive output columns of one row of C and stores them as 16-byte
-//              vectors.
+//   main loop: each wavefront takes 64-row blocks of W inside the workgroup's M range.  W is
+//              read from global memory with four adjacent lanes covering 64 contiguous bytes of
+//              a row (the pattern the L1 coalesces; one lane per row runs at a quarter of the
+//              rate), prefetched several K steps ahead into registers, and turned into MFMA
+//              operand order (lane = row) through a 4 KB wavefront-private LDS staging area
+//              (ds_write_b128 / ds_read_b128, both conflict-free under an XOR swizzle;
+//              ds_bpermute moves only 4 bytes per lane and measured 3x slower).  It is contracted
+//              against Y fragments read from LDS with v_mfma_f32_16x16x32; Y is the A operand and
+//              W the B operand, so a lane ends up with 16 consecutive output columns of one row.
+//   epilogue : the 64 x BN result block goes through the same staging area so that eight adjacent
+//              lanes store 128 contiguous bytes of a row of C.
 // The M range is split over gridDim.y workgroups so that the chip is filled.
 //
 // Behaviour replaced: fused_ht_gemm_pipelined, fused_ht/fusion_pipelined.cu:306-563 (cp.async
@@ -23,6 +28,9 @@ namespace {
 
 constexpr int kGemmThreads = 512;
 constexpr int kGemmWaves = kGemmThreads / 64;
+constexpr int kWaveRows = 64;   // rows of W per wavefront block
+constexpr int kMI = kWaveRows / 16;
+constexpr int kStageBytes = 4096;  // per-wavefront LDS staging: 64 rows x 32 K x 2 B
 
 template <class T16>
 struct OutStore {
@@ -78,7 +86,7 @@ template <class T16, int BN, int XB>
 __global__ void __launch_bounds__(kGemmThreads)
 fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16::E* __restrict__ Xt,
                        void* __restrict__ C, uint32_t M, uint32_t N, uint32_t K, uint32_t logK,
-                       uint32_t m_per_block, int out_f32, float fscale)
+                       uint32_t m_per_block, uint32_t msplit, int out_f32, float fscale)
 {
     using E = typename T16::E;
     using V8 = typename T16::V8;
@@ -88,7 +96,10 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
 
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t lo = lane & 15u, hi = lane >> 4;
-    const uint32_t n0 = blockIdx.x * BN;
+    // 1-D grid, M-slice index fastest: consecutive workgroup ids go to different XCDs, so every
+    // XCD keeps working on the same few M slices of W and that slice stays in its L2.
+    const uint32_t n0 = (blockIdx.x / msplit) * BN;
+    const uint32_t m_begin = (blockIdx.x % msplit) * m_per_block;
     const uint32_t chunks_per_col = K >> 3;
     const uint32_t swz_mask = (chunks_per_col >= 16u ? 16u : chunks_per_col) - 1u;
 
@@ -96,88 +107,141 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
     {
         TileOperands<T16> ops;
         make_tile_operands<T16, 2>(logK, ops);
-        constexpr int NT = 1 << XB;                       // tiles per wavefront step
+        constexpr int NT = 1 << XB;                       // tiles per column (or 1)
+        constexpr int BATCH = 16;                         // tiles in flight per wavefront
+        static_assert(BATCH % NT == 0, "batch must hold whole columns");
         const uint32_t block_tiles = (BN * K) >> 9;       // 512-element tiles in this block
         const uint64_t total = (uint64_t)N * K;           // elements in Xt
         const uint64_t tile_base = ((uint64_t)n0 * K) >> 9;
-        for (uint32_t t0 = wave * NT; t0 < block_tiles; t0 += kGemmWaves * NT) {
-            V8 in[NT];
+        for (uint32_t t0 = wave * BATCH; t0 < block_tiles; t0 += kGemmWaves * BATCH) {
+            V8 in[BATCH];
 #pragma unroll
-            for (int c = 0; c < NT; ++c) {
+            for (int c = 0; c < BATCH; ++c) {
                 const uint64_t off = (tile_base + t0 + c) * 512u + 8u * lane;
-                if (off + 8u <= total) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) in[c][j] = (E)0.0f;  // columns past N, tiles past the block
+                if (t0 + c < block_tiles && off + 8u <= total)
                     in[c] = *reinterpret_cast<const V8*>(Xt + off);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) in[c][j] = (E)0.0f;  // columns past N
-                }
             }
-            f32x4 acc[NT][2];
 #pragma unroll
-            for (int c = 0; c < NT; ++c) tile_transform<T16>(in[c], ops, acc[c]);
-            cross_tile_butterflies<NT, XB>(acc);
+            for (int g = 0; g < BATCH / NT; ++g) {
+                f32x4 acc[NT][2];
 #pragma unroll
-            for (int c = 0; c < NT; ++c) {
-                V8 o;
+                for (int c = 0; c < NT; ++c) tile_transform<T16>(in[g * NT + c], ops, acc[c]);
+                cross_tile_butterflies<NT, XB>(acc);
 #pragma unroll
-                for (int t = 0; t < 2; ++t)
+                for (int c = 0; c < NT; ++c) {
+                    if (t0 + g * NT + c >= block_tiles) continue;
+                    V8 o;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) o[4 * t + r] = (E)(acc[c][t][r] * fscale);
-                const uint32_t e = (t0 + c) * 512u + 8u * lane;  // element offset in the block
-                const uint32_t n = e >> logK, q = (e & (K - 1u)) >> 3;
-                *reinterpret_cast<V8*>(ylds + y_chunk_offset<LOG_NB>(n, q, K * 2u, swz_mask)) = o;
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) o[4 * t + r] = (E)(acc[c][t][r] * fscale);
+                    const uint32_t e = (t0 + g * NT + c) * 512u + 8u * lane;  // offset in the block
+                    const uint32_t n = e >> logK, q = (e & (K - 1u)) >> 3;
+                    *reinterpret_cast<V8*>(ylds + y_chunk_offset<LOG_NB>(n, q, K * 2u, swz_mask)) = o;
+                }
             }
         }
     }
     __syncthreads();
 
     // ---- main loop ------------------------------------------------------------------------------
-    const uint32_t m_begin = blockIdx.y * m_per_block;
     const uint32_t m_end = min(M, m_begin + m_per_block);
-    const uint32_t ksteps = K >> 5;
+    unsigned char* stage = ylds + (size_t)BN * K * 2u + wave * kStageBytes;
+    // staging layout for a 64-row x 32-K sub-step: row r (64 bytes), 16-byte chunk c stored at
+    // position c ^ ((r >> 2) & 3).  Writer lane l holds row 16*mi + l/4, chunk l%4; reader lane
+    // (hi, lo) takes row 16*mi + lo, chunk hi.
+    const uint32_t wr_off = (lane >> 2) * 64u + (((lane & 3u) ^ ((lane >> 4) & 3u)) << 4);
+    const uint32_t rd_off = lo * 64u + ((hi ^ ((lo >> 2) & 3u)) << 4);
 
-    for (uint32_t mb = m_begin + wave * 64u; mb < m_end; mb += kGemmWaves * 64u) {
-        f32x4 acc[NB][4];
+    for (uint32_t mb = m_begin + wave * kWaveRows; mb < m_end; mb += kGemmWaves * kWaveRows) {
+        f32x4 acc[NB][kMI];
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-            for (int mi = 0; mi < 4; ++mi) acc[nb][mi] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int mi = 0; mi < kMI; ++mi) acc[nb][mi] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-        const E* wrow[4];
+        if (K >= 64u) {
+            const E* wld[kMI];
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) {
-            const uint32_t m = min(mb + 16u * mi + lo, M - 1u);  // clamp: masked at the store
-            wrow[mi] = W + (uint64_t)m * K + 8u * hi;
-        }
-        V8 bcur[4], bnext[4];
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) bcur[mi] = *reinterpret_cast<const V8*>(wrow[mi]);
-
-        for (uint32_t ks = 0; ks < ksteps; ++ks) {
-            if (ks + 1 < ksteps) {
-#pragma unroll
-                for (int mi = 0; mi < 4; ++mi)
-                    bnext[mi] = *reinterpret_cast<const V8*>(wrow[mi] + 32u * (ks + 1));
+            for (int mi = 0; mi < kMI; ++mi) {
+                const uint32_t m = min(mb + 16u * mi + (lane >> 2), M - 1u);  // masked at the store
+                wld[mi] = W + (uint64_t)m * K + 8u * (lane & 3u);
             }
+            constexpr int kDepth = 3;  // K64 steps in flight
+            const uint32_t ksteps = K >> 6;
+            u32x4 wraw[kDepth][kMI][2];
+#pragma unroll
+            for (int d = 0; d < kDepth; ++d)
+                if ((uint32_t)d < ksteps) {
+#pragma unroll
+                    for (int mi = 0; mi < kMI; ++mi)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h)
+                            wraw[d][mi][h] =
+                                *reinterpret_cast<const u32x4*>(wld[mi] + 64u * d + 32u * h);
+                }
+            for (uint32_t ks0 = 0; ks0 < ksteps; ks0 += kDepth) {
+#pragma unroll
+                for (int d = 0; d < kDepth; ++d) {
+                    const uint32_t ks = ks0 + d;
+                    if (ks < ksteps) {
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                            for (int mi = 0; mi < kMI; ++mi)
+                                *reinterpret_cast<u32x4*>(stage + mi * 1024u + wr_off) =
+                                    wraw[d][mi][h];
+                            V8 a[NB];
+#pragma unroll
+                            for (int nb = 0; nb < NB; ++nb)
+                                a[nb] = *reinterpret_cast<const V8*>(
+                                    ylds + y_chunk_offset<LOG_NB>(NB * lo + nb, 8u * ks + 4u * h + hi,
+                                                                  K * 2u, swz_mask));
+                            V8 bfrag[kMI];
+#pragma unroll
+                            for (int mi = 0; mi < kMI; ++mi)
+                                bfrag[mi] =
+                                    *reinterpret_cast<const V8*>(stage + mi * 1024u + rd_off);
+#pragma unroll
+                            for (int mi = 0; mi < kMI; ++mi)
+#pragma unroll
+                                for (int nb = 0; nb < NB; ++nb)
+                                    acc[nb][mi] = T16::mfma32(a[nb], bfrag[mi], acc[nb][mi]);
+                        }
+                        if (ks + kDepth < ksteps) {
+#pragma unroll
+                            for (int mi = 0; mi < kMI; ++mi)
+#pragma unroll
+                                for (int h = 0; h < 2; ++h)
+                                    wraw[d][mi][h] = *reinterpret_cast<const u32x4*>(
+                                        wld[mi] + 64u * (ks + kDepth) + 32u * h);
+                        }
+                    }
+                }
+            }
+        } else {
+            // K = 32: a single 32-wide step, operands straight from global memory
             V8 a[NB];
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb)
                 a[nb] = *reinterpret_cast<const V8*>(
-                    ylds + y_chunk_offset<LOG_NB>(NB * lo + nb, 4u * ks + hi, K * 2u, swz_mask));
+                    ylds + y_chunk_offset<LOG_NB>(NB * lo + nb, hi, K * 2u, swz_mask));
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
+            for (int mi = 0; mi < kMI; ++mi) {
+                const uint32_t m = min(mb + 16u * mi + lo, M - 1u);
+                const V8 bw = *reinterpret_cast<const V8*>(W + (uint64_t)m * K + 8u * hi);
 #pragma unroll
-                for (int mi = 0; mi < 4; ++mi)
-                    acc[nb][mi] = T16::mfma32(a[nb], bcur[mi], acc[nb][mi]);
-#pragma unroll
-            for (int mi = 0; mi < 4; ++mi) bcur[mi] = bnext[mi];
+                for (int nb = 0; nb < NB; ++nb) acc[nb][mi] = T16::mfma32(a[nb], bw, acc[nb][mi]);
+            }
         }
 
         // D[m'][n']: n' = lo is the row of W; m' = 4*hi + r is the A-operand lane, which carried
         // column NB*m' + nb.  So this lane owns the contiguous run of 4*NB columns starting at
         // 4*NB*hi, in the order v[NB*r + nb].
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) {
+        for (int mi = 0; mi < kMI; ++mi) {
             const uint32_t m = mb + 16u * mi + lo;
             if (m >= m_end) continue;
             float v[16];
@@ -214,24 +278,24 @@ int launch_gemm16(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N
     const int shift = tile_stage_shift<2>(logK);
     const float fscale = (float)((double)scale * (double)(1u << shift));
     const uint32_t n_tiles = (N + BN - 1) / BN;
-    // split M so that about two workgroups per compute unit exist; each covers a multiple of
+    // split M so that about one workgroup per compute unit exists; each covers a multiple of
     // 512 rows (8 wavefronts x 64 rows)
     const uint32_t row_blocks = (M + 511u) / 512u;
-    uint32_t msplit = (512u + n_tiles - 1u) / n_tiles;
+    uint32_t msplit = (256u + n_tiles - 1u) / n_tiles;
     if (msplit < 1u) msplit = 1u;
     if (msplit > row_blocks) msplit = row_blocks;
     const uint32_t m_per_block = ((row_blocks + msplit - 1u) / msplit) * 512u;
     msplit = (M + m_per_block - 1u) / m_per_block;
-    const size_t lds = (size_t)BN * K * 2u;
+    const size_t lds = (size_t)BN * K * 2u + (size_t)kGemmWaves * kStageBytes;
     auto kern = fused_ht_gemm16_kernel<T16, BN, XB>;
     if (lds > 64u * 1024u) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
             return MI_ERR_LAUNCH;
     }
-    hipLaunchKernelGGL(kern, dim3(n_tiles, msplit), dim3(kGemmThreads), lds, s,
+    hipLaunchKernelGGL(kern, dim3(n_tiles * msplit), dim3(kGemmThreads), lds, s,
                        static_cast<const typename T16::E*>(W),
-                       static_cast<const typename T16::E*>(Xt), C, M, N, K, logK, m_per_block,
+                       static_cast<const typename T16::E*>(Xt), C, M, N, K, logK, m_per_block, msplit,
                        out_f32, fscale);
     return launch_status();
 }
