@@ -78,16 +78,22 @@ template <int LOG_NB>
 __device__ __forceinline__ uint32_t y_chunk_offset(uint32_t n, uint32_t q, uint32_t col_bytes,
                                                    uint32_t swz_mask)
 {
-    return n * col_bytes + ((q ^ ((n >> LOG_NB) & swz_mask)) << 4);
+    // built as (16-byte chunk index) << 4 so that the 16-byte alignment is visible to the compiler
+    // and every access becomes a single ds_read_b128 / ds_write_b128
+    return (n * (col_bytes >> 4) + (q ^ ((n >> LOG_NB) & swz_mask))) << 4;
 }
 
 // XB = log2(max(K,512)/512): tiles per column that need cross-tile butterflies.
-template <class T16, int BN, int XB>
+// KFIX: K when it is known at compile time (lets the K loop be scheduled without run-time guards),
+// 0 for the generic instantiation.
+template <class T16, int BN, int XB, int KFIX>
 __global__ void __launch_bounds__(kGemmThreads)
 fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16::E* __restrict__ Xt,
-                       void* __restrict__ C, uint32_t M, uint32_t N, uint32_t K, uint32_t logK,
+                       void* __restrict__ C, uint32_t M, uint32_t N, uint32_t K_rt, uint32_t logK_rt,
                        uint32_t m_per_block, uint32_t msplit, int out_f32, float fscale)
 {
+    const uint32_t K = KFIX ? (uint32_t)KFIX : K_rt;
+    const uint32_t logK = KFIX ? (uint32_t)__builtin_ctz(KFIX ? KFIX : 1) : logK_rt;
     using E = typename T16::E;
     using V8 = typename T16::V8;
     constexpr int NB = BN / 16;  // 16-column fragments of Y (A-operand blocks)
@@ -150,10 +156,10 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
     const uint32_t m_end = min(M, m_begin + m_per_block);
     unsigned char* stage = ylds + (size_t)BN * K * 2u + wave * kStageBytes;
     // staging layout for a 64-row x 32-K sub-step: row r (64 bytes), 16-byte chunk c stored at
-    // position c ^ ((r >> 2) & 3).  Writer lane l holds row 16*mi + l/4, chunk l%4; reader lane
+    // position c ^ ((r >> 1) & 3) (the variant measured conflict-free for both access orders).  Writer lane l holds row 16*mi + l/4, chunk l%4; reader lane
     // (hi, lo) takes row 16*mi + lo, chunk hi.
-    const uint32_t wr_off = (lane >> 2) * 64u + (((lane & 3u) ^ ((lane >> 4) & 3u)) << 4);
-    const uint32_t rd_off = lo * 64u + ((hi ^ ((lo >> 2) & 3u)) << 4);
+    const uint32_t wr_off = (lane >> 2) * 64u + (((lane & 3u) ^ ((lane >> 3) & 3u)) << 4);
+    const uint32_t rd_off = lo * 64u + ((hi ^ ((lo >> 1) & 3u)) << 4);
 
     for (uint32_t mb = m_begin + wave * kWaveRows; mb < m_end; mb += kGemmWaves * kWaveRows) {
         f32x4 acc[NB][kMI];
@@ -169,7 +175,7 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
                 const uint32_t m = min(mb + 16u * mi + (lane >> 2), M - 1u);  // masked at the store
                 wld[mi] = W + (uint64_t)m * K + 8u * (lane & 3u);
             }
-            constexpr int kDepth = 3;  // K64 steps in flight
+            constexpr int kDepth = 2;  // K64 steps of W in flight in registers
             const uint32_t ksteps = K >> 6;
             u32x4 wraw[kDepth][kMI][2];
 #pragma unroll
@@ -182,6 +188,26 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
                             wraw[d][mi][h] =
                                 *reinterpret_cast<const u32x4*>(wld[mi] + 64u * d + 32u * h);
                 }
+
+            // Software pipeline over 32-wide sub-steps: the LDS traffic of sub-step s+1 (staging
+            // write, W fragment reads, Y fragment reads) is issued before the MFMAs of sub-step s.
+            // LDS operations of one wavefront complete in order, so the single staging area is
+            // safe: the reads of s were issued before the writes of s+1.
+            V8 a_nx[NB], b_nx[kMI];
+            auto fetch = [&](const u32x4 (&src)[kMI][2], int h, uint32_t ks) {
+#pragma unroll
+                for (int mi = 0; mi < kMI; ++mi)
+                    *reinterpret_cast<u32x4*>(stage + mi * 1024u + wr_off) = src[mi][h];
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+                    a_nx[nb] = *reinterpret_cast<const V8*>(
+                        ylds + y_chunk_offset<LOG_NB>(NB * lo + nb, 8u * ks + 4u * h + hi, K * 2u,
+                                                      swz_mask));
+#pragma unroll
+                for (int mi = 0; mi < kMI; ++mi)
+                    b_nx[mi] = *reinterpret_cast<const V8*>(stage + mi * 1024u + rd_off);
+            };
+            fetch(wraw[0], 0, 0);
             for (uint32_t ks0 = 0; ks0 < ksteps; ks0 += kDepth) {
 #pragma unroll
                 for (int d = 0; d < kDepth; ++d) {
@@ -189,34 +215,30 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
                     if (ks < ksteps) {
 #pragma unroll
                         for (int h = 0; h < 2; ++h) {
+                            V8 a_cu[NB], b_cu[kMI];
 #pragma unroll
-                            for (int mi = 0; mi < kMI; ++mi)
-                                *reinterpret_cast<u32x4*>(stage + mi * 1024u + wr_off) =
-                                    wraw[d][mi][h];
-                            V8 a[NB];
+                            for (int nb = 0; nb < NB; ++nb) a_cu[nb] = a_nx[nb];
 #pragma unroll
-                            for (int nb = 0; nb < NB; ++nb)
-                                a[nb] = *reinterpret_cast<const V8*>(
-                                    ylds + y_chunk_offset<LOG_NB>(NB * lo + nb, 8u * ks + 4u * h + hi,
-                                                                  K * 2u, swz_mask));
-                            V8 bfrag[kMI];
+                            for (int mi = 0; mi < kMI; ++mi) b_cu[mi] = b_nx[mi];
+                            if (h == 0) {
+                                fetch(wraw[d], 1, ks);
+                                // both halves of wraw[d] are now on their way to LDS: refill it
+                                if (ks + kDepth < ksteps) {
 #pragma unroll
-                            for (int mi = 0; mi < kMI; ++mi)
-                                bfrag[mi] =
-                                    *reinterpret_cast<const V8*>(stage + mi * 1024u + rd_off);
+                                    for (int mi = 0; mi < kMI; ++mi)
+#pragma unroll
+                                        for (int hh = 0; hh < 2; ++hh)
+                                            wraw[d][mi][hh] = *reinterpret_cast<const u32x4*>(
+                                                wld[mi] + 64u * (ks + kDepth) + 32u * hh);
+                                }
+                            } else if (ks + 1 < ksteps) {
+                                fetch(wraw[(d + 1) % kDepth], 0, ks + 1);
+                            }
 #pragma unroll
                             for (int mi = 0; mi < kMI; ++mi)
 #pragma unroll
                                 for (int nb = 0; nb < NB; ++nb)
-                                    acc[nb][mi] = T16::mfma32(a[nb], bfrag[mi], acc[nb][mi]);
-                        }
-                        if (ks + kDepth < ksteps) {
-#pragma unroll
-                            for (int mi = 0; mi < kMI; ++mi)
-#pragma unroll
-                                for (int h = 0; h < 2; ++h)
-                                    wraw[d][mi][h] = *reinterpret_cast<const u32x4*>(
-                                        wld[mi] + 64u * (ks + kDepth) + 32u * h);
+                                    acc[nb][mi] = T16::mfma32(a_cu[nb], b_cu[mi], acc[nb][mi]);
                         }
                     }
                 }
@@ -270,7 +292,7 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
     }
 }
 
-template <class T16, int BN, int XB>
+template <class T16, int BN, int XB, int KFIX>
 int launch_gemm16(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
                   int out_f32, float scale, hipStream_t s)
 {
@@ -287,7 +309,7 @@ int launch_gemm16(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N
     const uint32_t m_per_block = ((row_blocks + msplit - 1u) / msplit) * 512u;
     msplit = (M + m_per_block - 1u) / m_per_block;
     const size_t lds = (size_t)BN * K * 2u + (size_t)kGemmWaves * kStageBytes;
-    auto kern = fused_ht_gemm16_kernel<T16, BN, XB>;
+    auto kern = fused_ht_gemm16_kernel<T16, BN, XB, KFIX>;
     if (lds > 64u * 1024u) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -309,10 +331,10 @@ int dispatch_gemm16(const void* W, const void* Xt, void* C, uint32_t M, uint32_t
         case 64:
         case 128:
         case 256:
-        case 512: return launch_gemm16<T16, 64, 0>(W, Xt, C, M, N, K, out_f32, scale, s);
-        case 1024: return launch_gemm16<T16, 64, 1>(W, Xt, C, M, N, K, out_f32, scale, s);
-        case 2048: return launch_gemm16<T16, 32, 2>(W, Xt, C, M, N, K, out_f32, scale, s);
-        case 4096: return launch_gemm16<T16, 16, 3>(W, Xt, C, M, N, K, out_f32, scale, s);
+        case 512: return launch_gemm16<T16, 64, 0, 0>(W, Xt, C, M, N, K, out_f32, scale, s);
+        case 1024: return launch_gemm16<T16, 64, 1, 1024>(W, Xt, C, M, N, K, out_f32, scale, s);
+        case 2048: return launch_gemm16<T16, 32, 2, 0>(W, Xt, C, M, N, K, out_f32, scale, s);
+        case 4096: return launch_gemm16<T16, 16, 3, 0>(W, Xt, C, M, N, K, out_f32, scale, s);
         default: return MI_ERR_SIZE;
     }
 }

@@ -18,7 +18,7 @@ template <int LOG_NB>
 __device__ __forceinline__ uint32_t y_off(uint32_t n, uint32_t q, uint32_t col_bytes,
                                           uint32_t swz_mask)
 {
-    return n * col_bytes + ((q ^ ((n >> LOG_NB) & swz_mask)) << 4);
+    return (n * (col_bytes >> 4) + (q ^ ((n >> LOG_NB) & swz_mask))) << 4;
 }
 
 template <int BN, int XB>
