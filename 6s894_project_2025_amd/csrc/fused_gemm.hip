@@ -30,7 +30,7 @@ constexpr int kGemmThreads = 512;
 constexpr int kGemmWaves = kGemmThreads / 64;
 constexpr int kWaveRows = 64;   // rows of W per wavefront block
 constexpr int kMI = kWaveRows / 16;
-constexpr int kStageBytes = 4096;  // per-wavefront LDS staging: 64 rows x 32 K x 2 B
+constexpr int kStageBytes = kWaveRows * 64;  // per-wavefront LDS staging: rows x 32 K x 2 B
 
 template <class T16>
 struct OutStore {
@@ -301,7 +301,7 @@ int launch_gemm16(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N
     const float fscale = (float)((double)scale * (double)(1u << shift));
     const uint32_t n_tiles = (N + BN - 1) / BN;
     // split M so that about one workgroup per compute unit exists; each covers a multiple of
-    // 512 rows (8 wavefronts x 64 rows)
+    // 512 rows (wavefronts x rows per wavefront block)
     const uint32_t row_blocks = (M + 511u) / 512u;
     uint32_t msplit = (256u + n_tiles - 1u) / n_tiles;
     if (msplit < 1u) msplit = 1u;
