@@ -28,6 +28,14 @@ HIPCC_FLAGS = [
 ]
 
 
+# Extra flags per translation unit.  The streaming kernels read every MFMA result with VALU code
+# straight away, so they keep MFMA destinations in ordinary VGPRs (no accumulator-register copies).
+PER_FILE_FLAGS = {
+    "fwht.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "rht_fp8.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
+
+
 def sources() -> list[str]:
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
@@ -41,7 +49,8 @@ def _hipcc() -> str:
 
 def _compile(src: str) -> str:
     obj = os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", src, "-o", obj]
+    cmd = [_hipcc(), *HIPCC_FLAGS, *PER_FILE_FLAGS.get(os.path.basename(src), []), "-c", src, "-o",
+           obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "recognized feature" not in l)
     if r.returncode != 0:

@@ -10,6 +10,8 @@
 //     reduction over the lanes that share a row,
 //   - v_cvt_pk_fp8_f32 for the narrowing (hardware RNE to E4M3FN), 8 codes = one 8-byte store.
 // Bandwidth-bound: 2 bytes in, 1 byte (+ 4 bytes per row) out per element.
+#include <type_traits>
+
 #include "fwht_device.hpp"
 
 namespace mi {
@@ -17,6 +19,34 @@ namespace {
 
 constexpr float kFp8Max = 448.0f;
 constexpr float kAmaxFloor = 1e-30f;
+
+// Maximum over the lanes that differ only in their low `bits` lane-index bits (bits <= 6), with
+// data-parallel primitives only: quad permutes and row mirrors for 1, 2, 4, 8 (after each step
+// the value is uniform over the group already reduced, so a mirror pairs the right groups), then
+// v_permlane16_swap / v_permlane32_swap for 16 and 32.  No LDS traffic.
+__device__ __forceinline__ float lane_max(float v, uint32_t bits)
+{
+    auto dpp = [](float x, auto ctrl) {
+        return __builtin_bit_cast(
+            float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value,
+                                               0xf, 0xf, false));
+    };
+    if (bits >= 1u) v = fmaxf(v, dpp(v, std::integral_constant<int, 0xB1>{}));   // quad_perm [1,0,3,2]
+    if (bits >= 2u) v = fmaxf(v, dpp(v, std::integral_constant<int, 0x4E>{}));   // quad_perm [2,3,0,1]
+    if (bits >= 3u) v = fmaxf(v, dpp(v, std::integral_constant<int, 0x141>{}));  // row_half_mirror
+    if (bits >= 4u) v = fmaxf(v, dpp(v, std::integral_constant<int, 0x140>{}));  // row_mirror
+    if (bits >= 5u) {
+        const uint32_t x = __builtin_bit_cast(uint32_t, v);
+        const auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+        v = fmaxf(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+    }
+    if (bits >= 6u) {
+        const uint32_t x = __builtin_bit_cast(uint32_t, v);
+        const auto r = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+        v = fmaxf(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+    }
+    return v;
+}
 
 // NT tiles per wavefront; XB cross-tile bits (n = 512 << XB when XB > 0, else n <= 512 and the
 // NT tiles are independent).
@@ -59,55 +89,64 @@ rht_quant_fp8_kernel(const __bf16* __restrict__ x, const int8_t* __restrict__ si
     for (int c = 0; c < NT; ++c) tile_transform<BF16>(in[c], ops, acc[c]);
     cross_tile_butterflies<NT, XB>(acc);
 
-    // round to bf16 (the pre-quant values), amax per row
+    // round to bf16 (the pre-quant values); amax per row on the packed magnitudes (bf16 bit
+    // patterns without the sign order like unsigned integers)
     bf16x8 y[NT];
     float amax[NT];
 #pragma unroll
     for (int c = 0; c < NT; ++c) {
-        float m = 0.0f;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const __bf16 b = (__bf16)(acc[c][t][r] * fscale);
-                y[c][4 * t + r] = b;
-                m = fmaxf(m, fabsf((float)b));
-            }
-        amax[c] = m;
+            for (int r = 0; r < 4; ++r) y[c][4 * t + r] = (__bf16)(acc[c][t][r] * fscale);
+        const u32x4 yb = __builtin_bit_cast(u32x4, y[c]);
+        typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+        u16x2 m = {0, 0};
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const u16x2 mag = __builtin_bit_cast(u16x2, yb[w] & 0x7fff7fffu);
+            m = __builtin_elementwise_max(m, mag);
+        }
+        const uint32_t top = m[0] > m[1] ? m[0] : m[1];
+        amax[c] = __builtin_bit_cast(float, top << 16);
     }
     // lanes that share a row: lane bit i carries element bit 3 + i, so the low min(6, p - 3)
-    // lane bits index inside a row
+    // lane bits index inside a row.  When one row spans all NT tiles, fold the tiles first so
+    // that a single lane reduction is needed.
     const uint32_t row_lane_bits = p >= 9u ? 6u : p - 3u;
-#pragma unroll
-    for (int c = 0; c < NT; ++c) {
-        float m = amax[c];
-        for (uint32_t b = 0; b < row_lane_bits; ++b) m = fmaxf(m, __shfl_xor(m, 1 << b, 64));
-        amax[c] = m;
-    }
-    if (XB > 0) {  // one row spans all NT tiles
+    if (XB > 0) {
         float m = amax[0];
 #pragma unroll
         for (int c = 1; c < NT; ++c) m = fmaxf(m, amax[c]);
+        m = lane_max(m, 6u);
 #pragma unroll
         for (int c = 0; c < NT; ++c) amax[c] = m;
+    } else {
+#pragma unroll
+        for (int c = 0; c < NT; ++c) amax[c] = lane_max(amax[c], row_lane_bits);
     }
 
 #pragma unroll
     for (int c = 0; c < NT; ++c) {
         const uint64_t off = (wave * NT + c) * 512u + 8u * lane;
-        if (off + 8u > total) continue;
+        if (XB == 0 && off + 8u > total) continue;  // XB > 0: whole rows, guarded per wavefront
         const float a = fmaxf(amax[c], kAmaxFloor);
         const float inv = kFp8Max / a;
         // first lane of each row writes the dequantisation factor
         const bool row_head = XB > 0 ? (c == 0 && lane == 0) : ((off & (uint64_t)(n - 1u)) == 0);
         if (row_head) row_scale[off >> p] = a / kFp8Max;
+        // |y| <= amax, so y * inv <= 448 * (1 + 2^-23): always inside the round-to-448 interval and
+        // the +-448 clamp of the stated convention never changes a finite value; it is omitted.
+        const u32x4 yb = __builtin_bit_cast(u32x4, y[c]);
         u32x2 codes;
 #pragma unroll
         for (int w = 0; w < 2; ++w) {
             float v[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                v[i] = __builtin_amdgcn_fmed3f((float)y[c][4 * w + i] * inv, -kFp8Max, kFp8Max);
+            for (int i = 0; i < 2; ++i) {
+                v[2 * i] = __builtin_bit_cast(float, yb[2 * w + i] << 16) * inv;
+                v[2 * i + 1] = __builtin_bit_cast(float, yb[2 * w + i] & 0xffff0000u) * inv;
+            }
             int pk = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
             pk = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], pk, true);
             codes[w] = (uint32_t)pk;
