@@ -74,7 +74,8 @@ int mi_fwht(const void* in, void* out, uint64_t rows, uint32_t n, int dtype, flo
  * W[row*N + k] (:146), Y[row*B + b] (:156).  scale = 1 reproduces the reference (raw +-1
  * butterfly, :118-133).
  *
- *   dtype : MI_F32 only.   N : power of two, 2 <= N <= 4096.   M, B >= 1.
+ *   dtype : MI_F32 only.   N : power of two, 2 <= N <= 2048 (the 16-column tile of the
+ *   transformed operand must fit in LDS).   M, B >= 1.
  *   Y must not overlap W or X.
  */
 int mi_fused_ht_gemv(const void* W, const void* X, void* Y, uint32_t M, uint32_t N, uint32_t B,
@@ -91,7 +92,8 @@ int mi_fused_ht_gemv(const void* W, const void* X, void* Y, uint32_t M, uint32_t
  *
  *   in_dtype  : MI_F32 (fp32 MFMA) or MI_BF16 / MI_F16 (16-bit MFMA, fp32 accumulate).
  *   out_dtype : MI_F32, or the same 16-bit type as in_dtype.
- *   K : power of two, 16 <= K <= 4096.   M, N >= 1 (edge tiles are masked).
+ *   K : power of two, 32 <= K <= 4096 (MI_F32: K <= 2048, the fp32 tile of K = 4096 does not fit
+ *   in LDS).   M, N >= 1 (edge tiles are masked).
  */
 int mi_fused_ht_gemm(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
                      int in_dtype, int out_dtype, float scale, void* stream);
@@ -99,11 +101,12 @@ int mi_fused_ht_gemm(const void* W, const void* Xt, void* C, uint32_t M, uint32_
 /*
  * Randomized Hadamard + FP8 quantize:  y[t,:] = scale * H_n * (sign .* x[t,:]) rounded to bf16,
  * then per row   amax = max|y|,  a = max(amax, 1e-30f),  row_scale[t] = a / 448,
- * q[t,j] = e4m3fn_rne(clamp(y[t,j] * (448 / a), -448, 448))   (OCP E4M3FN; IEEE fp32 ops).
+ * q[t,j] = e4m3fn_rne(clamp(y[t,j] * (448 / a), -448, 448))   (OCP E4M3FN; IEEE fp32 ops; for
+ * finite y the clamp never changes a value because |y| <= amax).
  *
  * No counterpart in the reference (it has no FP8 path); part of the build contract's hot path.
  *
- *   x         : bf16 [T,n];  n power of two, 16 <= n <= 4096... see mi_status on violation.
+ *   x         : bf16 [T,n];  n power of two, 16 <= n <= 4096.
  *   sign      : int8 [n], entries +1 / -1.
  *   q         : uint8 [T,n] E4M3FN codes.      row_scale : fp32 [T] (dequantisation factors).
  *   y_out     : optional bf16 [T,n] dump of the pre-quant values (NULL to skip).
