@@ -21,6 +21,8 @@
 //
 // Behaviour replaced: fused_ht_gemm_pipelined, fused_ht/fusion_pipelined.cu:306-563 (cp.async
 // double-buffered X tile + in-smem butterfly + scalar-FMA GEMM; fp32 only, compile-time dims).
+#include <type_traits>
+
 #include "fwht_device.hpp"
 
 namespace mi {
@@ -31,45 +33,6 @@ constexpr int kGemmWaves = kGemmThreads / 64;
 constexpr int kWaveRows = 64;   // rows of W per wavefront block
 constexpr int kMI = kWaveRows / 16;
 constexpr int kStageBytes = kWaveRows * 64;  // per-wavefront LDS staging: rows x 32 K x 2 B
-
-template <class T16>
-struct OutStore {
-    // 16 consecutive columns of one row, fp32 accumulators -> `out_f32 ? float : T16::E`
-    static __device__ __forceinline__ void row16(void* C, bool out_f32, uint64_t row, uint32_t ldc,
-                                                 uint32_t col0, uint32_t ncols, const float (&v)[16])
-    {
-        using E = typename T16::E;
-        if (out_f32) {
-            float* p = static_cast<float*>(C) + row * ldc + col0;
-            if (ncols >= 16 && (ldc & 3u) == 0) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    f32x4 o = {v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
-                    *reinterpret_cast<f32x4*>(p + 4 * q) = o;
-                }
-            } else {
-#pragma unroll
-                for (int i = 0; i < 16; ++i)
-                    if ((uint32_t)i < ncols) p[i] = v[i];
-            }
-        } else {
-            E* p = static_cast<E*>(C) + row * ldc + col0;
-            if (ncols >= 16 && (ldc & 7u) == 0) {
-#pragma unroll
-                for (int q = 0; q < 2; ++q) {
-                    typename T16::V8 o;
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) o[i] = (E)v[8 * q + i];
-                    *reinterpret_cast<typename T16::V8*>(p + 8 * q) = o;
-                }
-            } else {
-#pragma unroll
-                for (int i = 0; i < 16; ++i)
-                    if ((uint32_t)i < ncols) p[i] = (E)v[i];
-            }
-        }
-    }
-};
 
 // Byte offset of 16-byte chunk q of column n in the swizzled Y[BN][K] LDS image.
 // `col_bytes` = bytes per column, LOG_NB = log2(16-column fragments per block): the fragment
@@ -109,6 +72,41 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
     const uint32_t chunks_per_col = K >> 3;
     const uint32_t swz_mask = (chunks_per_col >= 16u ? 16u : chunks_per_col) - 1u;
 
+    const uint32_t m_end = min(M, m_begin + m_per_block);
+    unsigned char* stage = ylds + (size_t)BN * K * 2u + wave * kStageBytes;
+
+    // ---- W stream state of this wavefront's current 64-row block ---------------------------------
+    // Load pattern: for row block mi and half h, lane l reads the 16 bytes at row 16*mi + l/4,
+    // k = 64*ks + 32*h + 8*(l%4): four adjacent lanes cover 64 contiguous bytes.
+    constexpr int kDepth = 2;  // K64 steps of W in flight in registers
+    const uint32_t ksteps = K >> 6;
+    // The workgroups of one XCD stream the same rows of W in lockstep; each starts its K loop at a
+    // different step (the sum over k is order independent) so that they hit different L2 lines.
+    const uint32_t krot = (blockIdx.x / msplit) & (ksteps - 1u);
+    auto kmap = [&](uint32_t ks) { return (ks + krot) & (ksteps - 1u); };
+    const E* wld[kMI];
+    u32x4 wraw[kDepth][kMI][2];
+    auto preload = [&](uint32_t mb) {
+#pragma unroll
+        for (int mi = 0; mi < kMI; ++mi) {
+            const uint32_t m = min(mb + 16u * mi + (lane >> 2), M - 1u);  // masked at the store
+            wld[mi] = W + (uint64_t)m * K + 8u * (lane & 3u);
+        }
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d)
+            if ((uint32_t)d < ksteps) {
+#pragma unroll
+                for (int mi = 0; mi < kMI; ++mi)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+                        wraw[d][mi][h] =
+                            *reinterpret_cast<const u32x4*>(wld[mi] + 64u * kmap(d) + 32u * h);
+            }
+    };
+    uint32_t mb = m_begin + wave * kWaveRows;
+    // the first W loads do not depend on the transformed tile: put them in flight before the prologue
+    if (mb < m_end && K >= 64u) preload(mb);
+
     // ---- prologue: Y = bf16(scale * H_K * X[:, n0:n0+BN]) into LDS -------------------------------
     {
         TileOperands<T16> ops;
@@ -119,49 +117,60 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
         const uint32_t block_tiles = (BN * K) >> 9;       // 512-element tiles in this block
         const uint64_t total = (uint64_t)N * K;           // elements in Xt
         const uint64_t tile_base = ((uint64_t)n0 * K) >> 9;
-        for (uint32_t t0 = wave * BATCH; t0 < block_tiles; t0 += kGemmWaves * BATCH) {
-            V8 in[BATCH];
+        // GUARD = false: the block lies inside Xt and holds a whole number of batches
+        auto run = [&](auto guard_tag) {
+            constexpr bool GUARD = decltype(guard_tag)::value;
+            for (uint32_t t0 = wave * BATCH; t0 < block_tiles; t0 += kGemmWaves * BATCH) {
+                V8 in[BATCH];
 #pragma unroll
-            for (int c = 0; c < BATCH; ++c) {
-                const uint64_t off = (tile_base + t0 + c) * 512u + 8u * lane;
+                for (int c = 0; c < BATCH; ++c) {
+                    const uint64_t off = (tile_base + t0 + c) * 512u + 8u * lane;
+                    if (GUARD) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j) in[c][j] = (E)0.0f;  // columns past N, tiles past the block
-                if (t0 + c < block_tiles && off + 8u <= total)
-                    in[c] = *reinterpret_cast<const V8*>(Xt + off);
-            }
+                        for (int j = 0; j < 8; ++j) in[c][j] = (E)0.0f;  // past N / past the block
+                        if (t0 + c < block_tiles && off + 8u <= total)
+                            in[c] = *reinterpret_cast<const V8*>(Xt + off);
+                    } else {
+                        in[c] = *reinterpret_cast<const V8*>(Xt + off);
+                    }
+                }
 #pragma unroll
-            for (int g = 0; g < BATCH / NT; ++g) {
-                f32x4 acc[NT][2];
+                for (int g = 0; g < BATCH / NT; ++g) {
+                    f32x4 acc[NT][2];
 #pragma unroll
-                for (int c = 0; c < NT; ++c) tile_transform<T16>(in[g * NT + c], ops, acc[c]);
-                cross_tile_butterflies<NT, XB>(acc);
+                    for (int c = 0; c < NT; ++c) tile_transform<T16>(in[g * NT + c], ops, acc[c]);
+                    cross_tile_butterflies<NT, XB>(acc);
 #pragma unroll
-                for (int c = 0; c < NT; ++c) {
-                    if (t0 + g * NT + c >= block_tiles) continue;
-                    V8 o;
+                    for (int c = 0; c < NT; ++c) {
+                        if (GUARD && t0 + g * NT + c >= block_tiles) continue;
+                        V8 o;
 #pragma unroll
-                    for (int t = 0; t < 2; ++t)
+                        for (int t = 0; t < 2; ++t)
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) o[4 * t + r] = (E)(acc[c][t][r] * fscale);
-                    const uint32_t e = (t0 + g * NT + c) * 512u + 8u * lane;  // offset in the block
-                    const uint32_t n = e >> logK, q = (e & (K - 1u)) >> 3;
-                    *reinterpret_cast<V8*>(ylds + y_chunk_offset<LOG_NB>(n, q, K * 2u, swz_mask)) = o;
+                            for (int r = 0; r < 4; ++r) o[4 * t + r] = (E)(acc[c][t][r] * fscale);
+                        const uint32_t e = (t0 + g * NT + c) * 512u + 8u * lane;  // offset in the block
+                        const uint32_t n = e >> logK, q = (e & (K - 1u)) >> 3;
+                        *reinterpret_cast<V8*>(ylds + y_chunk_offset<LOG_NB>(n, q, K * 2u, swz_mask)) =
+                            o;
+                    }
                 }
             }
-        }
+        };
+        if (n0 + BN <= N && block_tiles % (kGemmWaves * BATCH) == 0)
+            run(std::false_type{});
+        else
+            run(std::true_type{});
     }
     __syncthreads();
 
     // ---- main loop ------------------------------------------------------------------------------
-    const uint32_t m_end = min(M, m_begin + m_per_block);
-    unsigned char* stage = ylds + (size_t)BN * K * 2u + wave * kStageBytes;
     // staging layout for a 64-row x 32-K sub-step: row r (64 bytes), 16-byte chunk c stored at
-    // position c ^ ((r >> 1) & 3) (the variant measured conflict-free for both access orders).  Writer lane l holds row 16*mi + l/4, chunk l%4; reader lane
-    // (hi, lo) takes row 16*mi + lo, chunk hi.
+    // position c ^ ((r >> 1) & 3) (measured conflict-free for both access orders).  Writer lane l
+    // holds row 16*mi + l/4, chunk l%4; reader lane (hi, lo) takes row 16*mi + lo, chunk hi.
     const uint32_t wr_off = (lane >> 2) * 64u + (((lane & 3u) ^ ((lane >> 3) & 3u)) << 4);
     const uint32_t rd_off = lo * 64u + ((hi ^ ((lo >> 1) & 3u)) << 4);
 
-    for (uint32_t mb = m_begin + wave * kWaveRows; mb < m_end; mb += kGemmWaves * kWaveRows) {
+    while (mb < m_end) {
         f32x4 acc[NB][kMI];
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
@@ -169,30 +178,12 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
             for (int mi = 0; mi < kMI; ++mi) acc[nb][mi] = f32x4{0.f, 0.f, 0.f, 0.f};
 
         if (K >= 64u) {
-            const E* wld[kMI];
-#pragma unroll
-            for (int mi = 0; mi < kMI; ++mi) {
-                const uint32_t m = min(mb + 16u * mi + (lane >> 2), M - 1u);  // masked at the store
-                wld[mi] = W + (uint64_t)m * K + 8u * (lane & 3u);
-            }
-            constexpr int kDepth = 2;  // K64 steps of W in flight in registers
-            const uint32_t ksteps = K >> 6;
-            u32x4 wraw[kDepth][kMI][2];
-#pragma unroll
-            for (int d = 0; d < kDepth; ++d)
-                if ((uint32_t)d < ksteps) {
-#pragma unroll
-                    for (int mi = 0; mi < kMI; ++mi)
-#pragma unroll
-                        for (int h = 0; h < 2; ++h)
-                            wraw[d][mi][h] =
-                                *reinterpret_cast<const u32x4*>(wld[mi] + 64u * d + 32u * h);
-                }
-
             // Software pipeline over 32-wide sub-steps: the LDS traffic of sub-step s+1 (staging
             // write, W fragment reads, Y fragment reads) is issued before the MFMAs of sub-step s.
-            // LDS operations of one wavefront complete in order, so the single staging area is
-            // safe: the reads of s were issued before the writes of s+1.
+            // Operand order: lane (hi, lo) needs row 16*mi + lo, k = 64*ks + 32*h + 8*hi + j; the Y
+            // fragments use the same k assignment (chunk 8*ks + 4*h + hi).  LDS operations of one
+            // wavefront complete in order, so the single staging area is safe: the reads of s were
+            // issued before the writes of s+1.
             V8 a_nx[NB], b_nx[kMI];
             auto fetch = [&](const u32x4 (&src)[kMI][2], int h, uint32_t ks) {
 #pragma unroll
@@ -201,8 +192,8 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb)
                     a_nx[nb] = *reinterpret_cast<const V8*>(
-                        ylds + y_chunk_offset<LOG_NB>(NB * lo + nb, 8u * ks + 4u * h + hi, K * 2u,
-                                                      swz_mask));
+                        ylds + y_chunk_offset<LOG_NB>(NB * lo + nb, 8u * kmap(ks) + 4u * h + hi,
+                                                      K * 2u, swz_mask));
 #pragma unroll
                 for (int mi = 0; mi < kMI; ++mi)
                     b_nx[mi] = *reinterpret_cast<const V8*>(stage + mi * 1024u + rd_off);
@@ -229,7 +220,7 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
 #pragma unroll
                                         for (int hh = 0; hh < 2; ++hh)
                                             wraw[d][mi][hh] = *reinterpret_cast<const u32x4*>(
-                                                wld[mi] + 64u * (ks + kDepth) + 32u * hh);
+                                                wld[mi] + 64u * kmap(ks + kDepth) + 32u * hh);
                                 }
                             } else if (ks + 1 < ksteps) {
                                 fetch(wraw[(d + 1) % kDepth], 0, ks + 1);
@@ -259,36 +250,108 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
             }
         }
 
+        // the next block's first W loads go out before this block's result is stored
+        const uint32_t mb_next = mb + kGemmWaves * kWaveRows;
+        if (mb_next < m_end && K >= 64u) preload(mb_next);
+
+        // ---- epilogue ----------------------------------------------------------------------------
         // D[m'][n']: n' = lo is the row of W; m' = 4*hi + r is the A-operand lane, which carried
-        // column NB*m' + nb.  So this lane owns the contiguous run of 4*NB columns starting at
-        // 4*NB*hi, in the order v[NB*r + nb].
+        // column NB*m' + nb.  So lane (hi, lo) owns, for row 16*mi + lo, the contiguous run of 4*NB
+        // columns starting at 4*NB*hi, in the order v[NB*r + nb].
+        if constexpr (NB == 4) {
+            // Through the staging area, so that adjacent lanes store adjacent 16-byte pieces of a
+            // row of C.  One round covers kStageBytes / (64 columns * element size) rows.
+            const bool vec_ok = out_f32 ? ((N & 3u) == 0) : ((N & 7u) == 0);
+            if (!out_f32) {
 #pragma unroll
-        for (int mi = 0; mi < kMI; ++mi) {
-            const uint32_t m = mb + 16u * mi + lo;
-            if (m >= m_end) continue;
-            float v[16];
+                for (int p = 0; p < kMI / 2; ++p) {  // 32 rows x 128 bytes per round
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
+                    for (int mm = 0; mm < 2; ++mm) {
+                        const int mi = 2 * p + mm;
+                        const uint32_t rl = 16u * mm + lo;
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb) v[NB * r + nb] = acc[nb][mi][r];
-            const uint32_t col0 = n0 + (4u * NB) * hi;
-            if (col0 < N) {
-                const uint32_t ncols = min((uint32_t)(4 * NB), N - col0);
-                if constexpr (NB == 4) {
-                    OutStore<T16>::row16(C, out_f32 != 0, m, N, col0, ncols, v);
-                } else {
-                    // narrower blocks: element-wise store
+                        for (int q = 0; q < 2; ++q) {
+                            V8 o;
 #pragma unroll
-                    for (int i = 0; i < 4 * NB; ++i) {
-                        if ((uint32_t)i >= ncols) break;
-                        if (out_f32)
-                            static_cast<float*>(C)[(uint64_t)m * N + col0 + i] = v[i];
-                        else
-                            static_cast<E*>(C)[(uint64_t)m * N + col0 + i] = (E)v[i];
+                            for (int i = 0; i < 8; ++i) {
+                                const int idx = 8 * q + i;  // = NB*r + nb
+                                o[i] = (E)acc[idx & 3][mi][idx >> 2];
+                            }
+                            *reinterpret_cast<V8*>(stage + rl * 128u +
+                                                   (((2u * hi + q) ^ (rl & 7u)) << 4)) = o;
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const uint32_t rl = 8u * i + (lane >> 3), ch = lane & 7u;
+                        const V8 o = *reinterpret_cast<const V8*>(stage + rl * 128u +
+                                                                  ((ch ^ (rl & 7u)) << 4));
+                        const uint32_t m = mb + 32u * p + rl, col = n0 + 8u * ch;
+                        if (m < m_end && col < N) {
+                            E* dst = static_cast<E*>(C) + (uint64_t)m * N + col;
+                            if (vec_ok && col + 8u <= N) {
+                                *reinterpret_cast<V8*>(dst) = o;
+                            } else {
+#pragma unroll
+                                for (int j = 0; j < 8; ++j)
+                                    if (col + j < N) dst[j] = o[j];
+                            }
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int mi = 0; mi < kMI; ++mi) {  // 16 rows x 256 bytes per round
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        f32x4 o;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int idx = 4 * q + i;
+                            o[i] = acc[idx & 3][mi][idx >> 2];
+                        }
+                        *reinterpret_cast<f32x4*>(stage + lo * 256u + (((4u * hi + q) ^ lo) << 4)) = o;
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const uint32_t rl = 4u * i + (lane >> 4), ch = lane & 15u;
+                        const f32x4 o =
+                            *reinterpret_cast<const f32x4*>(stage + rl * 256u + ((ch ^ rl) << 4));
+                        const uint32_t m = mb + 16u * mi + rl, col = n0 + 4u * ch;
+                        if (m < m_end && col < N) {
+                            float* dst = static_cast<float*>(C) + (uint64_t)m * N + col;
+                            if (vec_ok && col + 4u <= N) {
+                                *reinterpret_cast<f32x4*>(dst) = o;
+                            } else {
+#pragma unroll
+                                for (int j = 0; j < 4; ++j)
+                                    if (col + j < N) dst[j] = o[j];
+                            }
+                        }
                     }
                 }
             }
+        } else {
+            // narrower tiles (K >= 2048): direct element-wise stores
+#pragma unroll
+            for (int mi = 0; mi < kMI; ++mi) {
+                const uint32_t m = mb + 16u * mi + lo;
+                if (m >= m_end) continue;
+                const uint32_t col0 = n0 + (4u * NB) * hi;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) {
+                        const uint32_t col = col0 + NB * r + nb;
+                        if (col >= N) continue;
+                        if (out_f32)
+                            static_cast<float*>(C)[(uint64_t)m * N + col] = acc[nb][mi][r];
+                        else
+                            static_cast<E*>(C)[(uint64_t)m * N + col] = (E)acc[nb][mi][r];
+                    }
+            }
         }
+        mb = mb_next;
     }
 }
 
