@@ -78,7 +78,7 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
     // ---- W stream state of this wavefront's current 64-row block ---------------------------------
     // Load pattern: for row block mi and half h, lane l reads the 16 bytes at row 16*mi + l/4,
     // k = 64*ks + 32*h + 8*(l%4): four adjacent lanes cover 64 contiguous bytes.
-    constexpr int kDepth = 2;  // K64 steps of W in flight in registers
+    constexpr int kDepth = 1;  // K64 steps of W in flight in registers (deeper measured slower)
     const uint32_t ksteps = K >> 6;
     // The workgroups of one XCD stream the same rows of W in lockstep; each starts its K loop at a
     // different step (the sum over k is order independent) so that they hit different L2 lines.
@@ -230,6 +230,16 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
 #pragma unroll
                                 for (int nb = 0; nb < NB; ++nb)
                                     acc[nb][mi] = T16::mfma32(a_cu[nb], b_cu[mi], acc[nb][mi]);
+                            // spread this sub-step's LDS and global traffic between its MFMAs
+                            // instead of issuing it in one burst
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) {
+                                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // DS write
+                                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // MFMA
+                                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // DS read
+                                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // MFMA
+                                if (h == 0) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);  // VMEM read
+                            }
                         }
                     }
                 }
