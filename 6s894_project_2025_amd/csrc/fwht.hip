@@ -13,6 +13,8 @@
 //
 // Behaviour replaced: run_fht<dtype>() and its kernels, csrc/main.cu:12-122 and
 // HadaCore/hadamard_transform_cuda.cu:90-746 (normalised FWHT, n = 2..2^15).
+#include <type_traits>
+
 #include "fwht_device.hpp"
 
 namespace mi {
@@ -31,12 +33,13 @@ struct Io16 {
         typename T16::V8 a;
     };
 
+    template <bool GUARD>
     static __device__ __forceinline__ In load(const void* base, uint64_t tile, uint64_t total)
     {
         const E* p = static_cast<const E*>(base);
         const uint64_t off = tile * 512u + 8u * (threadIdx.x & 63u);
         In in;
-        if (off + 8u <= total) {
+        if (!GUARD || off + 8u <= total) {
             in.a = *reinterpret_cast<const typename T16::V8*>(p + off);
         } else {
 #pragma unroll
@@ -51,6 +54,7 @@ struct Io16 {
         tile_transform<T16>(in.a, ops, acc);
     }
 
+    template <bool GUARD>
     static __device__ __forceinline__ void store(void* base, uint64_t tile, uint64_t total,
                                                  const f32x4 (&acc)[2], float s)
     {
@@ -61,7 +65,7 @@ struct Io16 {
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int r = 0; r < 4; ++r) o[4 * t + r] = (E)(acc[t][r] * s);
-        if (off + 8u <= total) {
+        if (!GUARD || off + 8u <= total) {
             *reinterpret_cast<typename T16::V8*>(p + off) = o;
         } else {
 #pragma unroll
@@ -78,6 +82,7 @@ struct Io32 {
         float v[8];
     };
 
+    template <bool GUARD>
     static __device__ __forceinline__ In load(const void* base, uint64_t tile, uint64_t total)
     {
         const float* p = static_cast<const float*>(base);
@@ -85,7 +90,7 @@ struct Io32 {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const uint64_t off = tile * 512u + 256u * t + 4u * (threadIdx.x & 63u);
-            if (off + 4u <= total) {
+            if (!GUARD || off + 4u <= total) {
                 const f32x4 q = *reinterpret_cast<const f32x4*>(p + off);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) in.v[4 * t + r] = q[r];
@@ -103,6 +108,7 @@ struct Io32 {
         tile_transform_f32(in.v, ops, acc);
     }
 
+    template <bool GUARD>
     static __device__ __forceinline__ void store(void* base, uint64_t tile, uint64_t total,
                                                  const f32x4 (&acc)[2], float s)
     {
@@ -111,7 +117,7 @@ struct Io32 {
         for (int t = 0; t < 2; ++t) {
             const uint64_t off = tile * 512u + 256u * t + 4u * (threadIdx.x & 63u);
             const f32x4 o = acc[t] * s;
-            if (off + 4u <= total) {
+            if (!GUARD || off + 4u <= total) {
                 *reinterpret_cast<f32x4*>(p + off) = o;
             } else {
 #pragma unroll
@@ -136,18 +142,34 @@ fwht_reg_kernel(const void* in, void* out, uint64_t total, uint64_t num_waves, u
     TileOperands<typename IO::T16> ops;
     make_tile_operands<typename IO::T16, IO::ESIZE>(p, ops);
 
-    typename IO::In tin[NT];
+    // GUARD = false when every tile of this wavefront lies inside the buffer (always, except for
+    // the last wavefront of a ragged n <= 512 problem): no bounds code on the hot path.
+    auto body = [&](auto guard_tag) {
+        constexpr bool GUARD = decltype(guard_tag)::value;
+        typename IO::In tin[NT];
 #pragma unroll
-    for (int c = 0; c < NT; ++c) tin[c] = IO::load(in, wave * NT + c, total);
+        for (int c = 0; c < NT; ++c) tin[c] = IO::template load<GUARD>(in, wave * NT + c, total);
+        // keep every load of the wavefront in flight before any arithmetic is scheduled
+        __builtin_amdgcn_sched_barrier(0);
 
-    f32x4 acc[NT][2];
+        f32x4 acc[NT][2];
 #pragma unroll
-    for (int c = 0; c < NT; ++c) IO::transform(tin[c], ops, acc[c]);
+        for (int c = 0; c < NT; ++c) IO::transform(tin[c], ops, acc[c]);
 
-    cross_tile_butterflies<NT, XB>(acc);
+        cross_tile_butterflies<NT, XB>(acc);
 
 #pragma unroll
-    for (int c = 0; c < NT; ++c) IO::store(out, wave * NT + c, total, acc[c], fscale);
+        for (int c = 0; c < NT; ++c)
+            IO::template store<GUARD>(out, wave * NT + c, total, acc[c], fscale);
+    };
+    if constexpr (XB > 0) {
+        body(std::false_type{});  // one wavefront = one whole row: nothing to guard
+    } else {
+        if ((wave * NT + NT) * 512u <= total)
+            body(std::false_type{});
+        else
+            body(std::true_type{});
+    }
 }
 
 // ---- LDS kernel: one workgroup of W = 2^LW wavefronts per row of n = 4096 * W ----------------
@@ -174,7 +196,7 @@ fwht_lds_kernel(const void* in, void* out, uint64_t rows, float fscale)
     {
         typename IO::In tin[8];
 #pragma unroll
-        for (int c = 0; c < 8; ++c) tin[c] = IO::load(in, tile0 + w * 8u + c, total);
+        for (int c = 0; c < 8; ++c) tin[c] = IO::template load<false>(in, tile0 + w * 8u + c, total);
         f32x4 acc[8][2];
 #pragma unroll
         for (int c = 0; c < 8; ++c) IO::transform(tin[c], ops, acc[c]);
@@ -215,7 +237,8 @@ fwht_lds_kernel(const void* in, void* out, uint64_t rows, float fscale)
     for (int s = 0; s < W; ++s)
 #pragma unroll
         for (int cc = 0; cc < OWN; ++cc)
-            IO::store(out, tile0 + s * 8u + w * OWN + cc, total, g[s * OWN + cc], fscale);
+            IO::template store<false>(out, tile0 + s * 8u + w * OWN + cc, total, g[s * OWN + cc],
+                                      fscale);
 }
 
 // ---- host dispatch --------------------------------------------------------------------------------
