@@ -54,7 +54,7 @@ struct Io16 {
         tile_transform<T16>(in.a, ops, acc);
     }
 
-    template <bool GUARD>
+    template <bool GUARD, bool MUL>
     static __device__ __forceinline__ void store(void* base, uint64_t tile, uint64_t total,
                                                  const f32x4 (&acc)[2], float s)
     {
@@ -64,7 +64,7 @@ struct Io16 {
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) o[4 * t + r] = (E)(acc[t][r] * s);
+            for (int r = 0; r < 4; ++r) o[4 * t + r] = (E)(MUL ? acc[t][r] * s : acc[t][r]);
         if (!GUARD || off + 8u <= total) {
             *reinterpret_cast<typename T16::V8*>(p + off) = o;
         } else {
@@ -108,7 +108,7 @@ struct Io32 {
         tile_transform_f32(in.v, ops, acc);
     }
 
-    template <bool GUARD>
+    template <bool GUARD, bool MUL>
     static __device__ __forceinline__ void store(void* base, uint64_t tile, uint64_t total,
                                                  const f32x4 (&acc)[2], float s)
     {
@@ -116,7 +116,7 @@ struct Io32 {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const uint64_t off = tile * 512u + 256u * t + 4u * (threadIdx.x & 63u);
-            const f32x4 o = acc[t] * s;
+            const f32x4 o = MUL ? acc[t] * s : acc[t];
             if (!GUARD || off + 4u <= total) {
                 *reinterpret_cast<f32x4*>(p + off) = o;
             } else {
@@ -128,28 +128,32 @@ struct Io32 {
     }
 };
 
-// ---- register kernel: NT tiles per wavefront, XB cross-tile bits ------------------------------
-template <class IO, int NT, int XB>
+// ---- register kernel: NT tiles per wavefront step, XB cross-tile bits ----------------------------
+// A wavefront handles the steps  first, first + stride, ...  (one step = NT tiles = one row when
+// XB > 0), so the operand set-up is paid once per wavefront.  MUL = false when the output scale is
+// a power of two (folded into the stage-2 operand).
+template <class IO, int NT, int XB, bool MUL>
 __global__ void __launch_bounds__(256)
-fwht_reg_kernel(const void* in, void* out, uint64_t total, uint64_t num_waves, uint32_t p,
-                float fscale)
+fwht_reg_kernel(const void* in, void* out, uint64_t total, uint64_t num_steps, uint32_t p, int exp2,
+                float mult)
 {
-    // `in` may equal `out`: a wavefront reads all of its tiles before it writes any, and
-    // wavefronts own disjoint tiles, which is what makes in-place operation safe.
-    const uint64_t wave = (uint64_t)blockIdx.x * 4u + (threadIdx.x >> 6);
-    if (wave >= num_waves) return;  // uniform per wavefront
+    // `in` may equal `out`: a wavefront reads all tiles of a step before it writes any, and steps
+    // own disjoint tiles, which is what makes in-place operation safe.
+    const uint64_t first = (uint64_t)blockIdx.x * 4u + (threadIdx.x >> 6);
+    const uint64_t stride = (uint64_t)gridDim.x * 4u;
+    if (first >= num_steps) return;  // uniform per wavefront
 
     TileOperands<typename IO::T16> ops;
-    make_tile_operands<typename IO::T16, IO::ESIZE>(p, ops);
+    make_tile_operands<typename IO::T16, IO::ESIZE>(p, ops, exp2);
 
-    // GUARD = false when every tile of this wavefront lies inside the buffer (always, except for
-    // the last wavefront of a ragged n <= 512 problem): no bounds code on the hot path.
-    auto body = [&](auto guard_tag) {
+    // GUARD = false when every tile of the step lies inside the buffer (always, except for the
+    // last step of a ragged n <= 512 problem): no bounds code on the hot path.
+    auto body = [&](uint64_t step, auto guard_tag) {
         constexpr bool GUARD = decltype(guard_tag)::value;
         typename IO::In tin[NT];
 #pragma unroll
-        for (int c = 0; c < NT; ++c) tin[c] = IO::template load<GUARD>(in, wave * NT + c, total);
-        // keep every load of the wavefront in flight before any arithmetic is scheduled
+        for (int c = 0; c < NT; ++c) tin[c] = IO::template load<GUARD>(in, step * NT + c, total);
+        // keep every load of the step in flight before any arithmetic is scheduled
         __builtin_amdgcn_sched_barrier(0);
 
         f32x4 acc[NT][2];
@@ -160,15 +164,17 @@ fwht_reg_kernel(const void* in, void* out, uint64_t total, uint64_t num_waves, u
 
 #pragma unroll
         for (int c = 0; c < NT; ++c)
-            IO::template store<GUARD>(out, wave * NT + c, total, acc[c], fscale);
+            IO::template store<GUARD, MUL>(out, step * NT + c, total, acc[c], mult);
     };
-    if constexpr (XB > 0) {
-        body(std::false_type{});  // one wavefront = one whole row: nothing to guard
-    } else {
-        if ((wave * NT + NT) * 512u <= total)
-            body(std::false_type{});
-        else
-            body(std::true_type{});
+    for (uint64_t step = first; step < num_steps; step += stride) {
+        if constexpr (XB > 0) {
+            body(step, std::false_type{});  // whole rows: nothing to guard
+        } else {
+            if ((step * NT + NT) * 512u <= total)
+                body(step, std::false_type{});
+            else
+                body(step, std::true_type{});
+        }
     }
 }
 
@@ -176,9 +182,9 @@ fwht_reg_kernel(const void* in, void* out, uint64_t total, uint64_t num_waves, u
 // Pass 1: wavefront w transforms elements [4096w, 4096w+4096) (12 bits).  Exchange: every
 // accumulator quad goes to LDS once; wavefront w then gathers, from all W sub-rows, the 8/W tiles
 // it owns, runs the LW remaining butterflies in registers and stores.
-template <class IO, int LW>
+template <class IO, int LW, bool MUL>
 __global__ void __launch_bounds__(64 << LW)
-fwht_lds_kernel(const void* in, void* out, uint64_t rows, float fscale)
+fwht_lds_kernel(const void* in, void* out, uint64_t rows, int exp2, float mult)
 {
     constexpr int W = 1 << LW;
     constexpr int OWN = 8 / W;  // tiles per sub-row owned by a wavefront in pass 2
@@ -191,7 +197,7 @@ fwht_lds_kernel(const void* in, void* out, uint64_t rows, float fscale)
     const uint64_t tile0 = row * (8u * W);
 
     TileOperands<typename IO::T16> ops;
-    make_tile_operands<typename IO::T16, IO::ESIZE>(12 + LW, ops);
+    make_tile_operands<typename IO::T16, IO::ESIZE>(12 + LW, ops, exp2);
 
     {
         typename IO::In tin[8];
@@ -237,36 +243,46 @@ fwht_lds_kernel(const void* in, void* out, uint64_t rows, float fscale)
     for (int s = 0; s < W; ++s)
 #pragma unroll
         for (int cc = 0; cc < OWN; ++cc)
-            IO::template store<false>(out, tile0 + s * 8u + w * OWN + cc, total, g[s * OWN + cc],
-                                      fscale);
+            IO::template store<false, MUL>(out, tile0 + s * 8u + w * OWN + cc, total,
+                                           g[s * OWN + cc], mult);
 }
 
 // ---- host dispatch --------------------------------------------------------------------------------
 template <class IO, int NT, int XB>
-int launch_reg(const void* in, void* out, uint64_t total, uint64_t num_waves, uint32_t p,
-               float fscale, hipStream_t s)
+int launch_reg(const void* in, void* out, uint64_t total, uint64_t num_steps, uint32_t p,
+               OutputScale os, hipStream_t s)
 {
-    const uint64_t blocks = (num_waves + 3u) / 4u;
-    if (blocks == 0) return MI_OK;
+    if (num_steps == 0) return MI_OK;
+    // up to four steps per wavefront once every compute unit has a full set of wavefronts
+    uint64_t waves = num_steps;
+    const uint64_t resident = 256u * 16u;
+    if (waves > resident) waves = (num_steps + 3u) / 4u > resident ? (num_steps + 3u) / 4u : resident;
+    const uint64_t blocks = (waves + 3u) / 4u;
     if (blocks > 0x7fffffffull) return MI_ERR_SHAPE;
-    hipLaunchKernelGGL((fwht_reg_kernel<IO, NT, XB>), dim3((uint32_t)blocks), dim3(256), 0, s, in,
-                       out, total, num_waves, p, fscale);
+    if (os.mult == 1.0f)
+        hipLaunchKernelGGL((fwht_reg_kernel<IO, NT, XB, false>), dim3((uint32_t)blocks), dim3(256), 0,
+                           s, in, out, total, num_steps, p, os.exp2, os.mult);
+    else
+        hipLaunchKernelGGL((fwht_reg_kernel<IO, NT, XB, true>), dim3((uint32_t)blocks), dim3(256), 0,
+                           s, in, out, total, num_steps, p, os.exp2, os.mult);
     return launch_status();
 }
 
 template <class IO, int LW>
-int launch_lds(const void* in, void* out, uint64_t rows, float fscale, hipStream_t s)
+int launch_lds(const void* in, void* out, uint64_t rows, OutputScale os, hipStream_t s)
 {
     if (rows == 0) return MI_OK;
     if (rows > 0x7fffffffull) return MI_ERR_SHAPE;
     constexpr size_t lds = sizeof(f32x4) * 64u * 16u * (1u << LW);
-    auto kern = fwht_lds_kernel<IO, LW>;
+    const bool mul = os.mult != 1.0f;
+    auto kern = mul ? fwht_lds_kernel<IO, LW, true> : fwht_lds_kernel<IO, LW, false>;
     if (lds > 64u * 1024u) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
             return MI_ERR_LAUNCH;
     }
-    hipLaunchKernelGGL(kern, dim3((uint32_t)rows), dim3(64u << LW), lds, s, in, out, rows, fscale);
+    hipLaunchKernelGGL(kern, dim3((uint32_t)rows), dim3(64u << LW), lds, s, in, out, rows, os.exp2,
+                       os.mult);
     return launch_status();
 }
 
@@ -275,22 +291,21 @@ int dispatch(const void* in, void* out, uint64_t rows, uint32_t n, float scale, 
 {
     const uint32_t p = ilog2(n);
     const uint64_t total = rows * (uint64_t)n;
-    const int shift = tile_stage_shift<IO::ESIZE>(p);
-    const float fscale = (float)((double)scale * (double)(1u << shift));
+    const OutputScale os = split_output_scale((double)scale, tile_stage_shift<IO::ESIZE>(p));
     if (p <= 9) {
         const uint64_t tiles = (total + 511u) / 512u;
-        // several independent tiles per wavefront once there is enough work to fill the chip
+        // several independent tiles per step once there is enough work to fill the chip
         if (tiles >= 4u * 16384u)
-            return launch_reg<IO, 4, 0>(in, out, total, (tiles + 3u) / 4u, p, fscale, s);
-        return launch_reg<IO, 1, 0>(in, out, total, tiles, p, fscale, s);
+            return launch_reg<IO, 4, 0>(in, out, total, (tiles + 3u) / 4u, p, os, s);
+        return launch_reg<IO, 1, 0>(in, out, total, tiles, p, os, s);
     }
     switch (p) {
-        case 10: return launch_reg<IO, 2, 1>(in, out, total, rows, p, fscale, s);
-        case 11: return launch_reg<IO, 4, 2>(in, out, total, rows, p, fscale, s);
-        case 12: return launch_reg<IO, 8, 3>(in, out, total, rows, p, fscale, s);
-        case 13: return launch_lds<IO, 1>(in, out, rows, fscale, s);
-        case 14: return launch_lds<IO, 2>(in, out, rows, fscale, s);
-        case 15: return launch_lds<IO, 3>(in, out, rows, fscale, s);
+        case 10: return launch_reg<IO, 2, 1>(in, out, total, rows, p, os, s);
+        case 11: return launch_reg<IO, 4, 2>(in, out, total, rows, p, os, s);
+        case 12: return launch_reg<IO, 8, 3>(in, out, total, rows, p, os, s);
+        case 13: return launch_lds<IO, 1>(in, out, rows, os, s);
+        case 14: return launch_lds<IO, 2>(in, out, rows, os, s);
+        case 15: return launch_lds<IO, 3>(in, out, rows, os, s);
         default: return MI_ERR_SIZE;
     }
 }

@@ -21,7 +21,7 @@
 //
 // Bits >= log2(n) are masked out of G1/G2 (identity), so one tile can hold several short rows.
 // Both stages carry a power-of-two factor (exact) that keeps 16-bit intermediates in range; the
-// caller folds the inverse into its final scale via tile_stage_gain().
+// caller folds the inverse into its output scale (tile_stage_shift, split_output_scale).
 #pragma once
 
 #include "common.hpp"
@@ -59,6 +59,30 @@ __host__ __device__ inline void tile_masks(uint32_t p, uint32_t& mask1, uint32_t
         if ((uint32_t)(TileMap<ESIZE>::lo_e0 + b) < p) mask2 |= 1u << b;
 }
 
+// Splits the factor that must follow the two MFMA stages, scale * 2^tile_stage_shift(p), into a
+// power of two folded into the stage-2 operand (exp2, kept small enough for fp16 operands) and a
+// residual multiplier (1.0f exactly when the scale is a power of two).
+struct OutputScale {
+    int exp2;
+    float mult;
+};
+inline OutputScale split_output_scale(double scale, int stage_shift)
+{
+    OutputScale r{0, 1.0f};
+    const double f = scale * (double)(1u << stage_shift);
+    if (!(f > 0.0) || f != f || f > 1e30) {  // zero, negative, NaN, huge: plain multiplier
+        r.mult = (float)f;
+        return r;
+    }
+    int e;
+    (void)__builtin_frexp(f, &e);  // f = m * 2^e, m in [0.5, 1)
+    e -= 1;                        // f = (2m) * 2^e, 2m in [1, 2)
+    const int ec = e < -10 ? -10 : (e > 10 ? 10 : e);
+    r.exp2 = ec;
+    r.mult = (float)(f / __builtin_ldexp(1.0, ec));
+    return r;
+}
+
 // log2 of the (power-of-two) attenuation the two MFMA stages apply for a transform of length 2^p.
 template <int ESIZE>
 __host__ __device__ inline int tile_stage_shift(uint32_t p)
@@ -75,8 +99,10 @@ struct TileOperands {
     typename T16::V4 g2;     // stage-2 B operand
 };
 
+// `exp2` is an extra power-of-two factor folded (exactly) into the stage-2 operand, so that a
+// power-of-two output scale costs no multiply at all.
 template <class T16, int ESIZE>
-__device__ __forceinline__ void make_tile_operands(uint32_t p, TileOperands<T16>& ops)
+__device__ __forceinline__ void make_tile_operands(uint32_t p, TileOperands<T16>& ops, int exp2 = 0)
 {
     using E = typename T16::E;
     const uint32_t lane = threadIdx.x & 63u;
@@ -84,7 +110,7 @@ __device__ __forceinline__ void make_tile_operands(uint32_t p, TileOperands<T16>
     uint32_t mask1, mask2;
     tile_masks<ESIZE>(p, mask1, mask2);
     const float c1 = __builtin_ldexpf(1.0f, -(__popc(mask1) >> 1));
-    const float c2 = __builtin_ldexpf(1.0f, -(__popc(mask2) >> 1));
+    const float c2 = __builtin_ldexpf(1.0f, exp2 - (__popc(mask2) >> 1));
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
         const uint32_t np = 16u * t + lo;  // stage-1 output column

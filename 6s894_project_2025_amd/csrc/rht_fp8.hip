@@ -48,123 +48,145 @@ __device__ __forceinline__ float lane_max(float v, uint32_t bits)
     return v;
 }
 
-// NT tiles per wavefront; XB cross-tile bits (n = 512 << XB when XB > 0, else n <= 512 and the
-// NT tiles are independent).
-template <int NT, int XB>
+// NT tiles per wavefront step; XB cross-tile bits (n = 512 << XB when XB > 0: one step = one row;
+// else n <= 512 and the NT tiles are independent).  A wavefront handles the steps first,
+// first + stride, ... so the operand and sign-mask set-up is paid once.  MUL = false when the
+// transform's output scale is a power of two (folded into the stage-2 operand).
+template <int NT, int XB, bool MUL>
 __global__ void __launch_bounds__(256)
 rht_quant_fp8_kernel(const __bf16* __restrict__ x, const int8_t* __restrict__ sign,
                      uint8_t* __restrict__ q, float* __restrict__ row_scale,
-                     __bf16* __restrict__ y_out, uint64_t total, uint64_t num_waves, uint32_t p,
-                     float fscale)
+                     __bf16* __restrict__ y_out, uint64_t total, uint64_t num_steps, uint32_t p,
+                     int exp2, float mult)
 {
-    const uint64_t wave = (uint64_t)blockIdx.x * 4u + (threadIdx.x >> 6);
-    if (wave >= num_waves) return;
+    const uint64_t first = (uint64_t)blockIdx.x * 4u + (threadIdx.x >> 6);
+    const uint64_t stride = (uint64_t)gridDim.x * 4u;
+    if (first >= num_steps) return;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t n = 1u << p;
 
     TileOperands<BF16> ops;
-    make_tile_operands<BF16, 2>(p, ops);
+    make_tile_operands<BF16, 2>(p, ops, exp2);
 
-    // load + sign flip
-    bf16x8 in[NT];
+    // sign-bit masks of this lane's 8 columns in each tile of a step; the column pattern repeats
+    // from step to step (a step covers a whole number of rows)
+    u32x4 flip[NT];
 #pragma unroll
     for (int c = 0; c < NT; ++c) {
-        const uint64_t off = (wave * NT + c) * 512u + 8u * lane;
-        u32x4 bits = {0u, 0u, 0u, 0u};
-        if (off + 8u <= total) bits = *reinterpret_cast<const u32x4*>(x + off);
-        const uint32_t col = (uint32_t)(off & (uint64_t)(n - 1u));
+        const uint32_t col = (uint32_t)((first * NT + c) * 512u + 8u * lane) & (n - 1u);
         const u32x2 sg = *reinterpret_cast<const u32x2*>(sign + col);  // 8 int8, +1 / -1
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
             const uint32_t s2 = (w < 2 ? sg[0] : sg[1]) >> (16 * (w & 1));
             // byte 0 -> element 2w, byte 1 -> element 2w+1; -1 = 0xff has bit 7 set
-            const uint32_t flip = ((s2 & 0x80u) << 8) | ((s2 & 0x8000u) << 16);
-            bits[w] ^= flip;
+            flip[c][w] = ((s2 & 0x80u) << 8) | ((s2 & 0x8000u) << 16);
         }
-        in[c] = __builtin_bit_cast(bf16x8, bits);
-    }
-
-    f32x4 acc[NT][2];
-#pragma unroll
-    for (int c = 0; c < NT; ++c) tile_transform<BF16>(in[c], ops, acc[c]);
-    cross_tile_butterflies<NT, XB>(acc);
-
-    // round to bf16 (the pre-quant values); amax per row on the packed magnitudes (bf16 bit
-    // patterns without the sign order like unsigned integers)
-    bf16x8 y[NT];
-    float amax[NT];
-#pragma unroll
-    for (int c = 0; c < NT; ++c) {
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) y[c][4 * t + r] = (__bf16)(acc[c][t][r] * fscale);
-        const u32x4 yb = __builtin_bit_cast(u32x4, y[c]);
-        typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
-        u16x2 m = {0, 0};
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const u16x2 mag = __builtin_bit_cast(u16x2, yb[w] & 0x7fff7fffu);
-            m = __builtin_elementwise_max(m, mag);
-        }
-        const uint32_t top = m[0] > m[1] ? m[0] : m[1];
-        amax[c] = __builtin_bit_cast(float, top << 16);
     }
     // lanes that share a row: lane bit i carries element bit 3 + i, so the low min(6, p - 3)
-    // lane bits index inside a row.  When one row spans all NT tiles, fold the tiles first so
-    // that a single lane reduction is needed.
+    // lane bits index inside a row
     const uint32_t row_lane_bits = p >= 9u ? 6u : p - 3u;
-    if (XB > 0) {
-        float m = amax[0];
+
+    for (uint64_t step = first; step < num_steps; step += stride) {
+        // load + sign flip
+        bf16x8 in[NT];
 #pragma unroll
-        for (int c = 1; c < NT; ++c) m = fmaxf(m, amax[c]);
-        m = lane_max(m, 6u);
+        for (int c = 0; c < NT; ++c) {
+            const uint64_t off = (step * NT + c) * 512u + 8u * lane;
+            u32x4 bits = {0u, 0u, 0u, 0u};
+            if (XB > 0 || off + 8u <= total) bits = *reinterpret_cast<const u32x4*>(x + off);
+            in[c] = __builtin_bit_cast(bf16x8, bits ^ flip[c]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        f32x4 acc[NT][2];
 #pragma unroll
-        for (int c = 0; c < NT; ++c) amax[c] = m;
-    } else {
+        for (int c = 0; c < NT; ++c) tile_transform<BF16>(in[c], ops, acc[c]);
+        cross_tile_butterflies<NT, XB>(acc);
+
+        // round to bf16 (the pre-quant values); amax per row on the packed magnitudes (bf16 bit
+        // patterns without the sign order like unsigned integers)
+        bf16x8 y[NT];
+        float amax[NT];
 #pragma unroll
-        for (int c = 0; c < NT; ++c) amax[c] = lane_max(amax[c], row_lane_bits);
-    }
+        for (int c = 0; c < NT; ++c) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    y[c][4 * t + r] = (__bf16)(MUL ? acc[c][t][r] * mult : acc[c][t][r]);
+            const u32x4 yb = __builtin_bit_cast(u32x4, y[c]);
+            typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+            u16x2 m = {0, 0};
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const u16x2 mag = __builtin_bit_cast(u16x2, yb[w] & 0x7fff7fffu);
+                m = __builtin_elementwise_max(m, mag);
+            }
+            const uint32_t top = m[0] > m[1] ? m[0] : m[1];
+            amax[c] = __builtin_bit_cast(float, top << 16);
+        }
+        if (XB > 0) {  // one row spans all NT tiles: fold the tiles, then one lane reduction
+            float m = amax[0];
+#pragma unroll
+            for (int c = 1; c < NT; ++c) m = fmaxf(m, amax[c]);
+            m = lane_max(m, 6u);
+#pragma unroll
+            for (int c = 0; c < NT; ++c) amax[c] = m;
+        } else {
+#pragma unroll
+            for (int c = 0; c < NT; ++c) amax[c] = lane_max(amax[c], row_lane_bits);
+        }
 
 #pragma unroll
-    for (int c = 0; c < NT; ++c) {
-        const uint64_t off = (wave * NT + c) * 512u + 8u * lane;
-        if (XB == 0 && off + 8u > total) continue;  // XB > 0: whole rows, guarded per wavefront
-        const float a = fmaxf(amax[c], kAmaxFloor);
-        const float inv = kFp8Max / a;
-        // first lane of each row writes the dequantisation factor
-        const bool row_head = XB > 0 ? (c == 0 && lane == 0) : ((off & (uint64_t)(n - 1u)) == 0);
-        if (row_head) row_scale[off >> p] = a / kFp8Max;
-        // |y| <= amax, so y * inv <= 448 * (1 + 2^-23): always inside the round-to-448 interval and
-        // the +-448 clamp of the stated convention never changes a finite value; it is omitted.
-        const u32x4 yb = __builtin_bit_cast(u32x4, y[c]);
-        u32x2 codes;
+        for (int c = 0; c < NT; ++c) {
+            const uint64_t off = (step * NT + c) * 512u + 8u * lane;
+            if (XB == 0 && off + 8u > total) continue;  // XB > 0: whole rows
+            const float a = fmaxf(amax[c], kAmaxFloor);
+            const float inv = kFp8Max / a;
+            // first lane of each row writes the dequantisation factor
+            const bool row_head = XB > 0 ? (c == 0 && lane == 0) : ((off & (uint64_t)(n - 1u)) == 0);
+            if (row_head) row_scale[off >> p] = a / kFp8Max;
+            // |y| <= amax, so y * inv <= 448 * (1 + 2^-23): always inside the round-to-448 interval
+            // and the +-448 clamp of the stated convention never changes a finite value; omitted.
+            const u32x4 yb = __builtin_bit_cast(u32x4, y[c]);
+            u32x2 codes;
 #pragma unroll
-        for (int w = 0; w < 2; ++w) {
-            float v[4];
+            for (int w = 0; w < 2; ++w) {
+                float v[4];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                v[2 * i] = __builtin_bit_cast(float, yb[2 * w + i] << 16) * inv;
-                v[2 * i + 1] = __builtin_bit_cast(float, yb[2 * w + i] & 0xffff0000u) * inv;
+                for (int i = 0; i < 2; ++i) {
+                    v[2 * i] = __builtin_bit_cast(float, yb[2 * w + i] << 16) * inv;
+                    v[2 * i + 1] = __builtin_bit_cast(float, yb[2 * w + i] & 0xffff0000u) * inv;
+                }
+                int pk = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
+                pk = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], pk, true);
+                codes[w] = (uint32_t)pk;
             }
-            int pk = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
-            pk = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], pk, true);
-            codes[w] = (uint32_t)pk;
+            *reinterpret_cast<u32x2*>(q + off) = codes;
+            if (y_out) *reinterpret_cast<bf16x8*>(y_out + off) = y[c];
         }
-        *reinterpret_cast<u32x2*>(q + off) = codes;
-        if (y_out) *reinterpret_cast<bf16x8*>(y_out + off) = y[c];
     }
 }
 
 template <int NT, int XB>
 int launch_quant(const void* x, const int8_t* sign, void* q, float* rs, void* y_out, uint64_t total,
-                 uint64_t num_waves, uint32_t p, float fscale, hipStream_t s)
+                 uint64_t num_steps, uint32_t p, OutputScale os, hipStream_t s)
 {
-    const uint64_t blocks = (num_waves + 3u) / 4u;
+    // a wavefront's steps must all see the same column pattern: with NT tiles per step a step
+    // covers NT * 512 elements, a whole number of rows for every n <= NT * 512 (true here)
+    uint64_t waves = num_steps;
+    const uint64_t resident = 256u * 16u;
+    if (waves > resident) waves = (num_steps + 3u) / 4u > resident ? (num_steps + 3u) / 4u : resident;
+    const uint64_t blocks = (waves + 3u) / 4u;
     if (blocks > 0x7fffffffull) return MI_ERR_SHAPE;
-    hipLaunchKernelGGL((rht_quant_fp8_kernel<NT, XB>), dim3((uint32_t)blocks), dim3(256), 0, s,
-                       static_cast<const __bf16*>(x), sign, static_cast<uint8_t*>(q), rs,
-                       static_cast<__bf16*>(y_out), total, num_waves, p, fscale);
+    if (os.mult == 1.0f)
+        hipLaunchKernelGGL((rht_quant_fp8_kernel<NT, XB, false>), dim3((uint32_t)blocks), dim3(256), 0,
+                           s, static_cast<const __bf16*>(x), sign, static_cast<uint8_t*>(q), rs,
+                           static_cast<__bf16*>(y_out), total, num_steps, p, os.exp2, os.mult);
+    else
+        hipLaunchKernelGGL((rht_quant_fp8_kernel<NT, XB, true>), dim3((uint32_t)blocks), dim3(256), 0,
+                           s, static_cast<const __bf16*>(x), sign, static_cast<uint8_t*>(q), rs,
+                           static_cast<__bf16*>(y_out), total, num_steps, p, os.exp2, os.mult);
     return launch_status();
 }
 
@@ -247,17 +269,16 @@ extern "C" int mi_rht_quant_fp8(const void* x, const int8_t* sign, void* q, floa
         return MI_ERR_ALIGN;
     const uint32_t p = ilog2(n);
     const uint64_t total = T * (uint64_t)n;
-    const int shift = tile_stage_shift<2>(p);
-    const float fscale = (float)((double)scale * (double)(1u << shift));
+    const OutputScale os = split_output_scale((double)scale, tile_stage_shift<2>(p));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (p <= 9) {
         const uint64_t tiles = (total + 511u) / 512u;
-        return launch_quant<1, 0>(x, sign, q, row_scale, y_out, total, tiles, p, fscale, s);
+        return launch_quant<1, 0>(x, sign, q, row_scale, y_out, total, tiles, p, os, s);
     }
     switch (p) {
-        case 10: return launch_quant<2, 1>(x, sign, q, row_scale, y_out, total, T, p, fscale, s);
-        case 11: return launch_quant<4, 2>(x, sign, q, row_scale, y_out, total, T, p, fscale, s);
-        default: return launch_quant<8, 3>(x, sign, q, row_scale, y_out, total, T, p, fscale, s);
+        case 10: return launch_quant<2, 1>(x, sign, q, row_scale, y_out, total, T, p, os, s);
+        case 11: return launch_quant<4, 2>(x, sign, q, row_scale, y_out, total, T, p, os, s);
+        default: return launch_quant<8, 3>(x, sign, q, row_scale, y_out, total, T, p, os, s);
     }
 }
 
