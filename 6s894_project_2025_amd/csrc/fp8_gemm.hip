@@ -1,0 +1,229 @@
+// FP8 (OCP E4M3FN) GEMM with per-row scales (mi_fp8_gemm_rowscale), gfx950:
+//     out[t][n] = bf16( (sum_k qa[t][k] * qb[n][k]) * sa[t] * sb[n] ),  fp32 accumulate.
+// The reference has no FP8 path.  MFMA-bound shape (T = 8192, N = 14336, K = 4096 in the
+// benchmark configuration).
+//
+// Workgroup tile 256 x 256, four wavefronts of 128 x 128, K walked in steps of 128 bytes with
+// v_mfma_f32_16x16x128_f8f6f4 (unscaled form).  Both operand tiles go global -> registers (eight
+// lanes per 128-byte row segment, so the L1 coalesces) -> LDS, double buffered: the loads of
+// step s+1 are in flight while step s is multiplied.  LDS tiles are [256 rows][8 chunks of 16 B]
+// with chunk c of LDS row r stored at c ^ (r & 7); a lane of K-group hi reads chunks hi and hi + 4
+// of its row (any K assignment works as long as both operands use the same one).  Both the staging
+// writes and these fragment reads measured bank-conflict free; chunks 2*hi, 2*hi + 1 did not.
+// qb rows are the MFMA A operand and are stored in LDS in the order that lets a lane own 32
+// consecutive output columns; the result is staged through LDS once more so that C rows are
+// written as whole 512-byte runs.
+#include "common.hpp"
+
+namespace mi {
+namespace {
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kTile = 256;           // rows of qa and of qb per workgroup
+constexpr int kStepBytes = 128;      // K bytes per step
+constexpr int kTileBytes = kTile * kStepBytes;  // 32 KB
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ uint32_t tile_off(uint32_t row, uint32_t chunk)
+{
+    return (row * 8u + (chunk ^ (row & 7u))) << 4;
+}
+
+// LDS row r of the qb tile holds tile row 128*(r>>7) + 8*(r&15) + ((r>>4)&7): fragment block nb of
+// a wavefront (LDS rows 16*nb .. 16*nb+15) then carries columns 8*lo + nb.
+__device__ __forceinline__ uint32_t qb_tile_row(uint32_t r)
+{
+    return (r & 128u) + 8u * (r & 15u) + ((r >> 4) & 7u);
+}
+
+__global__ void __launch_bounds__(kThreads)
+fp8_gemm_rowscale_kernel(const uint8_t* __restrict__ qa, const float* __restrict__ sa,
+                         const uint8_t* __restrict__ qb, const float* __restrict__ sb,
+                         __bf16* __restrict__ out, uint32_t T, uint32_t N, uint32_t K,
+                         uint32_t tiles_t, uint32_t tiles_n)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // 2 x (A tile + B tile)
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t lo = lane & 15u, hi = lane >> 4;
+    const uint32_t wt = wave >> 1, wn = wave & 1u;
+
+    // tile order: consecutive workgroup ids land on different XCDs; an XCD works on 4 row tiles x
+    // a run of column tiles at a time, so its L2 serves most operand re-reads
+    uint32_t tm, tn;
+    {
+        const uint32_t id = blockIdx.x;
+        const uint32_t groups_t = (tiles_t + 3u) / 4u;  // groups of 4 row tiles
+        const uint32_t per_group = 4u * tiles_n;
+        // spread groups over XCDs round-robin
+        const uint32_t xcd = id & 7u, j = id >> 3;
+        const uint32_t slots = (groups_t + 7u) / 8u;           // groups per XCD
+        const uint32_t g = xcd * slots + j / per_group;         // group of this workgroup
+        const uint32_t w = j % per_group;
+        tm = g * 4u + (w & 3u);
+        tn = w >> 2;
+        if (g >= groups_t || tm >= tiles_t) return;  // padding ids of an uneven split
+    }
+    const uint32_t t0 = tm * kTile, n0 = tn * kTile;
+
+    // Operand staging, global -> LDS directly (no register hop): wavefront w, instruction i fills
+    // the 1 KB of LDS rows 32*i + 8*w .. +7 of a tile, lane l landing at byte 16*l of that run.
+    // Under the swizzle, slot l of the run is row r = 32*i + 8*w + l/8, position l%8, which holds
+    // global chunk (l%8) ^ (r & 7) = (l%8) ^ (l/8 % 8): eight adjacent lanes still cover one whole
+    // 128-byte row segment, so the loads coalesce.
+    const uint32_t cg = (lane & 7u) ^ ((lane >> 3) & 7u);
+    uint32_t oa[8], ob[8];  // 32-bit byte offsets (operands are checked to be below 4 GiB)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t r = 32u * i + 8u * wave + (lane >> 3);
+        const uint32_t ra = min(t0 + r, T - 1u);               // qa tile: LDS row = tile row
+        const uint32_t rb = min(n0 + qb_tile_row(r), N - 1u);  // qb tile: permuted
+        oa[i] = ra * K + 16u * cg;
+        ob[i] = rb * K + 16u * cg;
+    }
+    typedef __attribute__((address_space(1))) const void* gptr_t;
+    typedef __attribute__((address_space(3))) void* lptr_t;
+    auto stage = [&](uint32_t buf, uint32_t k0) {
+        unsigned char* A = lds + buf * (2u * kTileBytes);
+        unsigned char* B = A + kTileBytes;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t run = (32u * i + 8u * wave) * 128u;  // wavefront-uniform
+            __builtin_amdgcn_global_load_lds((gptr_t)(qb + (ob[i] + k0)), (lptr_t)(B + run), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(qa + (oa[i] + k0)), (lptr_t)(A + run), 16, 0, 0);
+        }
+    };
+
+    f32x4 acc[8][8];  // [nb][ti]
+#pragma unroll
+    for (int nb = 0; nb < 8; ++nb)
+#pragma unroll
+        for (int ti = 0; ti < 8; ++ti) acc[nb][ti] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const uint32_t ksteps = K / kStepBytes;
+    // Pipeline: the operands of step ks+1 stream into the other LDS buffer while step ks is
+    // multiplied; every wavefront waits for its own transfers before the barrier that ends the step.
+    stage(0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    for (uint32_t ks = 0; ks < ksteps; ++ks) {
+        const uint32_t buf = ks & 1u;
+        if (ks + 1 < ksteps) stage(buf ^ 1u, (ks + 1) * kStepBytes);
+        const unsigned char* A = lds + buf * (2u * kTileBytes);  // qa tile
+        const unsigned char* B = A + kTileBytes;                  // qb tile
+
+        i32x8 af[8];  // MFMA A operand fragments: qb rows, block nb
+#pragma unroll
+        for (int nb = 0; nb < 8; ++nb) {
+            const uint32_t r = 128u * wn + 16u * nb + lo;
+            const u32x4 x0 = *reinterpret_cast<const u32x4*>(B + tile_off(r, hi));
+            const u32x4 x1 = *reinterpret_cast<const u32x4*>(B + tile_off(r, hi + 4u));
+            af[nb] = i32x8{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3],
+                           (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
+        }
+        auto read_b = [&](int ti) {
+            const uint32_t r = 128u * wt + 16u * ti + lo;
+            const u32x4 x0 = *reinterpret_cast<const u32x4*>(A + tile_off(r, hi));
+            const u32x4 x1 = *reinterpret_cast<const u32x4*>(A + tile_off(r, hi + 4u));
+            return i32x8{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3],
+                         (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
+        };
+        i32x8 bf_nx = read_b(0);
+#pragma unroll
+        for (int ti = 0; ti < 8; ++ti) {
+            const i32x8 bf = bf_nx;
+            if (ti + 1 < 8) bf_nx = read_b(ti + 1);
+#pragma unroll
+            for (int nb = 0; nb < 8; ++nb)
+                acc[nb][ti] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[nb], bf, acc[nb][ti],
+                                                                              0, 0, 0, 0, 0, 0);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    }
+
+    // ---- epilogue: scale, narrow, stage through LDS, store whole rows ---------------------------
+    // D[m'][n']: n' = lo -> qa row t0 + 128*wt + 16*ti + lo; m' = 4*hi + r -> column
+    // 128*wn + 8*m' + nb = 128*wn + 32*hi + 8*r + nb.  LDS image: [256 rows][512 B], 16-byte chunk
+    // ch of row r stored at ch ^ (r & 31).
+    typedef __bf16 bf16x8v __attribute__((ext_vector_type(8)));
+    // this lane's 32 column scales (columns 128*wn + 32*hi + 0..31), loaded once
+    float sbv[32];
+    {
+        const uint32_t cbase = n0 + 128u * wn + 32u * hi;
+        if (cbase + 32u <= N) {
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                const f32x4 x = *reinterpret_cast<const f32x4*>(sb + cbase + 4u * v);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) sbv[4 * v + j] = x[j];
+            }
+        } else {
+#pragma unroll
+            for (int v = 0; v < 32; ++v) sbv[v] = sb[min(cbase + v, N - 1u)];
+        }
+    }
+#pragma unroll
+    for (int ti = 0; ti < 8; ++ti) {
+        const uint32_t rl = 128u * wt + 16u * ti + lo;
+        const float st = sa[min(t0 + rl, T - 1u)];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t col = 128u * wn + 32u * hi + 8u * r;  // 8 consecutive columns: nb = 0..7
+            bf16x8v o;
+#pragma unroll
+            for (int nb = 0; nb < 8; ++nb) o[nb] = (__bf16)(acc[nb][ti][r] * st * sbv[8 * r + nb]);
+            const uint32_t ch = col >> 3;
+            *reinterpret_cast<bf16x8v*>(lds + rl * 512u + ((ch ^ (rl & 31u)) << 4)) = o;
+        }
+    }
+    __syncthreads();
+    const bool vec_ok = (N & 7u) == 0;
+#pragma unroll 4
+    for (uint32_t i = 0; i < 32; ++i) {
+        const uint32_t rl = 8u * i + (tid >> 5), ch = tid & 31u;
+        const bf16x8v o = *reinterpret_cast<const bf16x8v*>(lds + rl * 512u + ((ch ^ (rl & 31u)) << 4));
+        const uint32_t t = t0 + rl, col = n0 + 8u * ch;
+        if (t < T && col < N) {
+            __bf16* dst = out + (uint64_t)t * N + col;
+            if (vec_ok && col + 8u <= N) {
+                *reinterpret_cast<bf16x8v*>(dst) = o;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (col + j < N) dst[j] = o[j];
+            }
+        }
+    }
+}
+
+}  // namespace
+}  // namespace mi
+
+extern "C" int mi_fp8_gemm_rowscale(const void* qa, const float* sa, const void* qb,
+                                    const float* sb, void* out, uint32_t T, uint32_t N, uint32_t K,
+                                    void* stream)
+{
+    using namespace mi;
+    if (K == 0 || (K & 127u)) return MI_ERR_SHAPE;
+    if (T == 0 || N == 0) return MI_OK;
+    if (!qa || !sa || !qb || !sb || !out) return MI_ERR_NULL;
+    if (!aligned16(qa) || !aligned16(qb) || !aligned16(out)) return MI_ERR_ALIGN;
+    if ((uint64_t)T * K > 0xffffffffull || (uint64_t)N * K > 0xffffffffull) return MI_ERR_SHAPE;
+    const uint32_t tiles_t = (T + kTile - 1) / kTile, tiles_n = (N + kTile - 1) / kTile;
+    // ids: 8 XCDs x (groups of 4 row tiles per XCD) x (4 * tiles_n); uneven splits are padded
+    const uint32_t groups_t = (tiles_t + 3u) / 4u;
+    const uint32_t slots = (groups_t + 7u) / 8u;
+    const uint64_t grid = (uint64_t)8u * slots * 4u * tiles_n;
+    if (grid > 0x7fffffffull) return MI_ERR_SHAPE;
+    const size_t lds = 4u * kTileBytes;  // 128 KB (also holds the 256 x 512 B result image)
+    auto kern = fp8_gemm_rowscale_kernel;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return MI_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3((uint32_t)grid), dim3(kThreads), lds, static_cast<hipStream_t>(stream),
+                       static_cast<const uint8_t*>(qa), sa, static_cast<const uint8_t*>(qb), sb,
+                       static_cast<__bf16*>(out), T, N, K, tiles_t, tiles_n);
+    return launch_status();
+}

@@ -1,6 +1,5 @@
-// Randomized Hadamard + FP8 (OCP E4M3FN) quantize epilogue (mi_rht_quant_fp8) and the FP8 GEMM
-// with per-row scales (mi_fp8_gemm_rowscale), gfx950.  The reference has no FP8 path; the
-// arithmetic convention is the one stated in include/mi_hadamard.h.
+// Randomized Hadamard + FP8 (OCP E4M3FN) quantize epilogue (mi_rht_quant_fp8), gfx950.  The
+// reference has no FP8 path; the arithmetic convention is the one stated in include/mi_hadamard.h.
 //
 // Quantize kernel: same skeleton as the stand-alone transform (one 16-byte load per 8 elements,
 // two MFMA stages per 512-element tile, fp32 butterflies across tiles), with
@@ -190,70 +189,6 @@ int launch_quant(const void* x, const int8_t* sign, void* q, float* rs, void* y_
     return launch_status();
 }
 
-// ---- FP8 GEMM, per-row scales -----------------------------------------------------------------------
-// out[t][n] = bf16( sum_k a[t][k] * b[n][k] * sa[t] * sb[n] ).  Workgroup tile 128 x 128, four
-// wavefronts of 64 x 64, operands read K-contiguously (8 codes per lane per MFMA) with
-// v_mfma_f32_16x16x32_fp8_fp8; qb rows play the A operand so that a lane owns consecutive
-// output columns.
-__global__ void __launch_bounds__(256)
-fp8_gemm_rowscale_kernel(const uint8_t* __restrict__ qa, const float* __restrict__ sa,
-                         const uint8_t* __restrict__ qb, const float* __restrict__ sb,
-                         __bf16* __restrict__ out, uint32_t T, uint32_t N, uint32_t K)
-{
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const uint32_t lo = lane & 15u, hi = lane >> 4;
-    const uint32_t t0 = blockIdx.y * 128u + (wave >> 1) * 64u;
-    const uint32_t n0 = blockIdx.x * 128u + (wave & 1u) * 64u;
-    if (t0 >= T || n0 >= N) return;
-
-    // A operand: qb rows (columns of out), lane `lo` carries column n0 + 4*lo + nb
-    // B operand: qa rows, lane `lo` carries row t0 + 16*ti + lo
-    const uint8_t* prow_b[4];
-    const uint8_t* prow_a[4];
-#pragma unroll
-    for (int nb = 0; nb < 4; ++nb)
-        prow_b[nb] = qb + (uint64_t)min(n0 + 4u * lo + nb, N - 1u) * K + 8u * hi;
-#pragma unroll
-    for (int ti = 0; ti < 4; ++ti)
-        prow_a[ti] = qa + (uint64_t)min(t0 + 16u * ti + lo, T - 1u) * K + 8u * hi;
-
-    f32x4 acc[4][4];
-#pragma unroll
-    for (int nb = 0; nb < 4; ++nb)
-#pragma unroll
-        for (int ti = 0; ti < 4; ++ti) acc[nb][ti] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    for (uint32_t k = 0; k < K; k += 32u) {
-        long a[4], b[4];
-#pragma unroll
-        for (int nb = 0; nb < 4; ++nb) a[nb] = *reinterpret_cast<const long*>(prow_b[nb] + k);
-#pragma unroll
-        for (int ti = 0; ti < 4; ++ti) b[ti] = *reinterpret_cast<const long*>(prow_a[ti] + k);
-#pragma unroll
-        for (int nb = 0; nb < 4; ++nb)
-#pragma unroll
-            for (int ti = 0; ti < 4; ++ti)
-                acc[nb][ti] =
-                    __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[nb], b[ti], acc[nb][ti], 0, 0, 0);
-    }
-
-    // D[m'][n']: n' = lo -> row t;  m' = 4*hi + r -> column n0 + 4*m' + nb = n0 + 16*hi + 4*r + nb
-#pragma unroll
-    for (int ti = 0; ti < 4; ++ti) {
-        const uint32_t t = t0 + 16u * ti + lo;
-        if (t >= T) continue;
-        const float st = sa[t];
-        const uint32_t col0 = n0 + 16u * hi;
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-#pragma unroll
-            for (int nb = 0; nb < 4; ++nb) {
-                const uint32_t col = col0 + 4u * r + nb;
-                if (col < N) out[(uint64_t)t * N + col] = (__bf16)(acc[nb][ti][r] * st * sb[col]);
-            }
-    }
-}
-
 }  // namespace
 }  // namespace mi
 
@@ -280,20 +215,4 @@ extern "C" int mi_rht_quant_fp8(const void* x, const int8_t* sign, void* q, floa
         case 11: return launch_quant<4, 2>(x, sign, q, row_scale, y_out, total, T, p, os, s);
         default: return launch_quant<8, 3>(x, sign, q, row_scale, y_out, total, T, p, os, s);
     }
-}
-
-extern "C" int mi_fp8_gemm_rowscale(const void* qa, const float* sa, const void* qb,
-                                    const float* sb, void* out, uint32_t T, uint32_t N, uint32_t K,
-                                    void* stream)
-{
-    using namespace mi;
-    if (K == 0 || (K & 127u)) return MI_ERR_SHAPE;
-    if (T == 0 || N == 0) return MI_OK;
-    if (!qa || !sa || !qb || !sb || !out) return MI_ERR_NULL;
-    if (!aligned16(qa) || !aligned16(qb) || !aligned16(out)) return MI_ERR_ALIGN;
-    const dim3 grid((N + 127u) / 128u, (T + 127u) / 128u);
-    hipLaunchKernelGGL(fp8_gemm_rowscale_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const uint8_t*>(qa), sa, static_cast<const uint8_t*>(qb), sb,
-                       static_cast<__bf16*>(out), T, N, K);
-    return launch_status();
 }
