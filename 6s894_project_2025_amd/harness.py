@@ -1,0 +1,260 @@
+"""Benchmark / check harness around the ops, following the reference's protocols.
+
+Two sub-commands (run from the repository root)::
+
+    python -m 6s894_project_2025_amd.harness fwht  [--check] [--runs-per-size 400] [--sizes ...]
+    python -m 6s894_project_2025_amd.harness fused [--dtype bf16|f32] [--runs 8]
+
+``fwht`` keeps the structure of the reference's bench/bench.py: a registry of in-place cases
+(three AddOne roofline proxies around the transform, :96-103), a correctness pass of every case
+against its ``call_ref`` with ``allclose(atol=1e-2 fp16 / 5e-2 bf16, rtol=0)`` (:159-203), the
+timing protocol "3 warm-up calls, then N back-to-back calls on the same buffer inside one event
+window" (:112-127), and a JSON dump with the same fields (:226-237, :291-300).  The reference
+checks its own kernel against HadaCore; here ``call_ref`` is the matrix truth path
+``t @ (hadamard(n) * n**-0.5)`` evaluated with torch on the GPU (bench/bench.py:49-59).
+
+``fused`` covers the 15 (K, N, M) shapes of fused_ht/benchmark_sweep.py:20-45 with its FLOP and
+byte models (:123-140), but with run-time shapes (no regex edit + recompile), and times the
+unfused baseline next to the fused kernel the way fused_ht/fusion_pipelined.cu:640-683 does:
+"transform kernel, then GEMM" (here: ``hadamard_transform`` + ``torch.matmul``, i.e. the vendor
+GEMM) versus ``fused_ht_gemm``; min over runs after 2 warm-ups (:631-683), max-abs difference
+between the two reported like :694-703.
+"""
+from __future__ import annotations
+
+import argparse
+import csv
+import functools
+import json
+import math
+import sys
+from dataclasses import dataclass, field
+from datetime import datetime
+from typing import Any, Callable
+
+import torch
+
+from .ops import fused_ht_gemm, hadamard_transform
+
+ATOL = {torch.float16: 1e-2, torch.bfloat16: 5e-2, torch.float32: 1e-4}
+DTYPES = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}
+
+
+def get_scale(size: int) -> float:
+    return math.sqrt(1.0 / size)
+
+
+@functools.lru_cache(maxsize=None)
+def _hadamard_cache(size: int) -> torch.Tensor:
+    """Sylvester matrix times n**-0.5 on the GPU, H[i][j] = (-1)**popcount(i & j)."""
+    idx = torch.arange(size, device="cuda")
+    bits = idx[:, None] & idx[None, :]
+    par = torch.zeros_like(bits)
+    for b in range(max(1, size.bit_length())):
+        par ^= (bits >> b) & 1
+    return (1.0 - 2.0 * par.to(torch.float32)) * get_scale(size)
+
+
+def hadamard_ref(t: torch.Tensor) -> None:
+    m = int(t.shape[-1])
+    t.copy_(t @ _hadamard_cache(m).to(t.dtype))
+
+
+class AddOne:
+    """In-place add: the achieved-bandwidth proxy (bench/bench.py:88-93)."""
+
+    def call(self, t: torch.Tensor) -> None:
+        t.add_(1)
+
+    def call_ref(self, t: torch.Tensor) -> None:
+        t.add_(1)
+
+
+class Ours:
+    def call(self, t: torch.Tensor) -> None:
+        hadamard_transform(t, inplace=True)
+
+    def call_ref(self, t: torch.Tensor) -> None:
+        hadamard_ref(t)
+
+
+CASES: dict[str, Any] = {"AddOne1": AddOne(), "AddOne2": AddOne(), "Ours": Ours(), "AddOne3": AddOne()}
+
+
+def _bench_many(fn: Callable[[], None], iters: int, warmup: int = 3) -> dict[str, float]:
+    torch.cuda.synchronize()
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    end.record()
+    end.synchronize()
+    total_ms = float(start.elapsed_time(end))
+    return {"total_ms": total_ms, "per_iter_ms": total_ms / max(iters, 1)}
+
+
+@dataclass
+class TestConfig:
+    check: bool = False
+    runs_per_size: int = 400
+    json_output_file: str | None = None
+    benchmark_cases: list[str] = field(default_factory=lambda: list(CASES))
+    test_sizes: list[int] = field(default_factory=lambda: [1 << x for x in range(8, 16)])
+    elem_counts: list[int] = field(default_factory=lambda: [1 << 30])
+    dtypes: tuple[torch.dtype, ...] = (torch.float16, torch.bfloat16)
+
+
+def run_fwht(cfg: TestConfig) -> list[dict[str, Any]]:
+    print("test_sizes_m: ", cfg.test_sizes)
+    print("test_elem_counts: ", cfg.elem_counts)
+    print("cases: ", cfg.benchmark_cases)
+    torch.manual_seed(0)
+    device_name = torch.cuda.get_device_name(0)
+    print(f"running on {device_name}\n")
+    results: list[dict[str, Any]] = []
+    for m in cfg.test_sizes:
+        for elem_c in cfg.elem_counts:
+            n = elem_c // m
+            if elem_c < m:
+                continue
+            print(f"Testing size {m}x{n}")
+            a = torch.randn((n, m), device="cuda", dtype=torch.float32)
+            for case_name in cfg.benchmark_cases:
+                target = CASES[case_name]
+                # correctness on a bounded slice (the matrix truth path is O(rows * m^2))
+                rows_chk = min(n, max(1, (1 << 22) // m))
+                for dtype in cfg.dtypes:
+                    got = a[:rows_chk].clone().to(dtype)
+                    want = a[:rows_chk].clone().to(dtype)
+                    target.call(got)
+                    target.call_ref(want)
+                    if not torch.allclose(want, got, atol=ATOL.get(dtype, 1e-2), rtol=0):
+                        diff = (want.float() - got.float()).abs()
+                        print(f"Failed test: {case_name} {m}x{n} {dtype}; max diff {diff.max().item()}")
+                        raise SystemExit(1)
+                if cfg.check:
+                    continue
+                for dtype in cfg.dtypes:
+                    a_run = a.to(dtype).contiguous()
+                    stats = _bench_many(lambda: target.call(a_run), cfg.runs_per_size)
+                    gbs = 2 * a_run.numel() * a_run.element_size() / stats["per_iter_ms"] / 1e6
+                    print(f"{case_name} m={m} n={n} {str(dtype).replace('torch.', '')} | "
+                          f"{stats['per_iter_ms']:.4f} ms/iter over {cfg.runs_per_size} iters "
+                          f"({gbs:.0f} GB/s)")
+                    results.append({"device": device_name, "case": case_name, "m": m, "n": n,
+                                    "dtype": str(dtype).replace("torch.", ""),
+                                    "runs": cfg.runs_per_size, "per_iter_ms": stats["per_iter_ms"],
+                                    "total_ms": stats["total_ms"], "GB/s": gbs})
+                    del a_run
+            del a
+    if not cfg.check and cfg.json_output_file:
+        with open(cfg.json_output_file, "w") as f:
+            json.dump({"device": device_name, "cases": cfg.benchmark_cases,
+                       "pytorch": torch.__version__, "results": results}, f, indent=2)
+        print(f"Wrote {cfg.json_output_file}")
+    return results
+
+
+# (KDIM, NDIM, MDIM) of fused_ht/benchmark_sweep.py:20-45
+FUSED_CONFIGS = [(k, s, s) for k in (256, 512, 1024, 2048, 4096) for s in (1024, 2048, 4096)]
+
+
+def compute_metrics(kdim: int, ndim: int, mdim: int, time_ms: float, esize: int = 4):
+    """GFLOPS and GB/s under the reference's model (benchmark_sweep.py:123-140)."""
+    ht_flops = kdim * (kdim.bit_length() - 1) * ndim * 2
+    gemm_flops = 2 * mdim * ndim * kdim
+    gflops = (ht_flops + gemm_flops) / 1e9 / (time_ms / 1e3)
+    bytes_rw = (kdim * ndim + mdim * kdim + mdim * ndim) * esize
+    return gflops, bytes_rw / 1e9 / (time_ms / 1e3)
+
+
+def _min_time_ms(fn: Callable[[], None], runs: int, warmup: int = 2) -> float:
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    best = float("inf")
+    for _ in range(runs):
+        s = torch.cuda.Event(enable_timing=True)
+        e = torch.cuda.Event(enable_timing=True)
+        s.record()
+        fn()
+        e.record()
+        e.synchronize()
+        best = min(best, float(s.elapsed_time(e)))
+    return best
+
+
+def run_fused(dtype: torch.dtype, runs: int = 8, configs=None, out_prefix: str | None = None):
+    rows = []
+    g = torch.Generator().manual_seed(123)
+    for (K, N, M) in configs or FUSED_CONFIGS:
+        if dtype == torch.float32 and K > 2048:
+            print(f"K={K} N={N} M={M}: skipped (fp32 tile of K=4096 does not fit in LDS)")
+            continue
+        W = torch.rand(M, K, generator=g).to(dtype).cuda()      # uniform [0,1) like drand48
+        Xt = torch.rand(N, K, generator=g).to(dtype).cuda()
+        scale = 1.0 / math.sqrt(K)
+        fused = lambda: fused_ht_gemm(W, Xt, scale)
+        unfused = lambda: torch.matmul(W, hadamard_transform(Xt, scale).t())
+        t_f = _min_time_ms(fused, runs)
+        t_u = _min_time_ms(unfused, runs)
+        diff = (fused().float() - unfused().float()).abs().max().item()
+        ref_scale = unfused().float().abs().max().item()
+        esize = W.element_size()
+        gf, bw = compute_metrics(K, N, M, t_f, esize)
+        gu, _ = compute_metrics(K, N, M, t_u, esize)
+        print(f"K={K:5d} N={N:5d} M={M:5d} {str(dtype).replace('torch.', ''):9s} "
+              f"unfused {t_u * 1e3:9.1f} us ({gu / 1e3:7.1f} TFLOP/s)  fused {t_f * 1e3:9.1f} us "
+              f"({gf / 1e3:7.1f} TFLOP/s)  speedup {t_u / t_f:5.2f}x  max|diff| {diff:.3e} "
+              f"(scale {ref_scale:.3e})")
+        rows.append({"kdim": K, "ndim": N, "mdim": M, "dtype": str(dtype).replace("torch.", ""),
+                     "baseline_ms": t_u, "fused_ms": t_f, "speedup": t_u / t_f,
+                     "fused_gflops": gf, "baseline_gflops": gu, "fused_bandwidth_gbps": bw,
+                     "max_error": diff, "max_abs_reference": ref_scale})
+        del W, Xt
+    if out_prefix:
+        with open(out_prefix + ".json", "w") as f:
+            json.dump(rows, f, indent=2)
+        with open(out_prefix + ".csv", "w", newline="") as f:
+            w = csv.DictWriter(f, fieldnames=list(rows[0].keys()) if rows else [])
+            w.writeheader()
+            w.writerows(rows)
+        print(f"Wrote {out_prefix}.json / .csv")
+    return rows
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="harness")
+    sub = ap.add_subparsers(dest="cmd", required=True)
+    p1 = sub.add_parser("fwht")
+    p1.add_argument("--check", action="store_true")
+    p1.add_argument("--runs-per-size", type=int, default=400)
+    p1.add_argument("--json-output-file", default=f"benchmark_{datetime.now():%Y-%m-%d_%H-%M-%S}.json")
+    p1.add_argument("--cases", nargs="*", default=list(CASES))
+    p1.add_argument("--sizes", nargs="*", type=int, default=[1 << x for x in range(8, 16)])
+    p1.add_argument("--elem-counts", nargs="*", type=int, default=[1 << 30])
+    p1.add_argument("--dtypes", nargs="*", default=["f16", "bf16"])
+    p2 = sub.add_parser("fused")
+    p2.add_argument("--dtype", default="bf16", choices=list(DTYPES))
+    p2.add_argument("--runs", type=int, default=8)
+    p2.add_argument("--out-prefix", default=None)
+    args = ap.parse_args(argv)
+    if not torch.cuda.is_available():
+        sys.stderr.write("harness: no GPU visible\n")
+        return 2
+    if args.cmd == "fwht":
+        run_fwht(TestConfig(check=args.check, runs_per_size=args.runs_per_size,
+                            json_output_file=args.json_output_file, benchmark_cases=args.cases,
+                            test_sizes=args.sizes, elem_counts=args.elem_counts,
+                            dtypes=tuple(DTYPES[d] for d in args.dtypes)))
+    else:
+        run_fused(DTYPES[args.dtype], args.runs, out_prefix=args.out_prefix)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

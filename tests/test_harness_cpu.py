@@ -1,0 +1,49 @@
+"""Host logic of the benchmark harness (no GPU): the shape list and the FLOP/byte model match the
+reference's sweep (fused_ht/benchmark_sweep.py:20-45,123-140), and the case registry and
+tolerances match its benchmark (bench/bench.py:96-103,177)."""
+import importlib
+
+import pytest
+import torch
+
+
+@pytest.fixture(scope="module")
+def harness(pkg):
+    return importlib.import_module(pkg.__name__ + ".harness")
+
+
+def test_fused_shape_list(harness):
+    cfgs = harness.FUSED_CONFIGS
+    assert len(cfgs) == 15 and len(set(cfgs)) == 15
+    assert cfgs[0] == (256, 1024, 1024) and cfgs[8] == (1024, 4096, 4096) and cfgs[-1] == (4096, 4096, 4096)
+    assert all(n == m for _, n, m in cfgs)
+    assert [k for k, _, _ in cfgs] == sorted(k for k, _, _ in cfgs)
+
+
+def test_compute_metrics_known_values(harness):
+    # K=1024, N=M=4096, 1 ms: transform 1024*10*4096*2 flops + GEMM 2*4096*4096*1024 flops;
+    # bytes (K*N + M*K + M*N) * 4.  Numbers written out by hand, not recomputed from the formula.
+    gflops, gbps = harness.compute_metrics(1024, 4096, 4096, 1.0)
+    assert gflops == pytest.approx((83_886_080 + 34_359_738_368) / 1e9 / 1e-3)
+    assert gbps == pytest.approx(100_663_296 / 1e9 / 1e-3)
+    # halving the time doubles both; 2-byte elements halve the bytes only
+    g2, b2 = harness.compute_metrics(1024, 4096, 4096, 0.5, esize=2)
+    assert g2 == pytest.approx(2 * gflops) and b2 == pytest.approx(gbps)
+
+
+def test_case_registry_and_tolerances(harness):
+    assert list(harness.CASES) == ["AddOne1", "AddOne2", "Ours", "AddOne3"]
+    assert harness.ATOL[torch.float16] == 1e-2 and harness.ATOL[torch.bfloat16] == 5e-2
+    cfg = harness.TestConfig()
+    assert cfg.runs_per_size == 400
+    assert cfg.test_sizes == [256, 512, 1024, 2048, 4096, 8192, 16384, 32768]
+    assert cfg.elem_counts == [1 << 30]
+    t = torch.zeros(4, 8)
+    harness.CASES["AddOne1"].call(t)
+    assert torch.equal(t, torch.ones(4, 8))
+
+
+def test_cli_without_gpu_exits_nonzero(harness):
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    assert harness.main(["fwht", "--check"]) == 2

@@ -1,0 +1,63 @@
+"""The harness end to end on the GPU at small sizes: --check passes for every case and dtype, the
+timed run writes the reference's JSON fields (bench/bench.py:226-237,291-300), and the fused sweep
+reports fused vs. unfused within the 16-bit tolerance."""
+import importlib
+import json
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def harness(pkg):
+    return importlib.import_module(pkg.__name__ + ".harness")
+
+
+def test_check_mode_all_cases(harness):
+    cfg = harness.TestConfig(check=True, test_sizes=[256, 2048, 32768], elem_counts=[1 << 20])
+    assert harness.run_fwht(cfg) == []
+
+
+def test_check_mode_detects_a_wrong_case(harness):
+    class Wrong:
+        def call(self, t):
+            t.add_(1)
+
+        def call_ref(self, t):
+            t.add_(2)
+
+    harness.CASES["Wrong"] = Wrong()
+    try:
+        with pytest.raises(SystemExit):
+            harness.run_fwht(harness.TestConfig(check=True, benchmark_cases=["Wrong"],
+                                                test_sizes=[256], elem_counts=[1 << 16]))
+    finally:
+        del harness.CASES["Wrong"]
+
+
+def test_timed_run_json(harness, tmp_path):
+    out = tmp_path / "b.json"
+    cfg = harness.TestConfig(runs_per_size=5, json_output_file=str(out), test_sizes=[1024],
+                             elem_counts=[1 << 20])
+    res = harness.run_fwht(cfg)
+    assert len(res) == 4 * 2
+    payload = json.loads(out.read_text())
+    assert set(payload) == {"device", "cases", "pytorch", "results"}
+    for r in payload["results"]:
+        assert {"device", "case", "m", "n", "dtype", "runs", "per_iter_ms", "total_ms"} <= set(r)
+        assert r["m"] == 1024 and r["n"] == 1024 and r["runs"] == 5 and r["per_iter_ms"] > 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_fused_sweep_small(harness, dtype, tmp_path):
+    rows = harness.run_fused(dtype, runs=2, configs=[(256, 128, 192), (1024, 256, 256)],
+                             out_prefix=str(tmp_path / "s"))
+    assert len(rows) == 2
+    for r in rows:
+        tol = 2e-2 if dtype == torch.bfloat16 else 1e-4
+        assert r["max_error"] <= tol * r["max_abs_reference"]
+        assert r["fused_ms"] > 0 and r["baseline_ms"] > 0
+    assert json.loads((tmp_path / "s.json").read_text())[0]["kdim"] == 256
+    assert (tmp_path / "s.csv").read_text().startswith("kdim,ndim,mdim")
