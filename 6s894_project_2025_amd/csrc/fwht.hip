@@ -15,118 +15,10 @@
 // HadaCore/hadamard_transform_cuda.cu:90-746 (normalised FWHT, n = 2..2^15).
 #include <type_traits>
 
-#include "fwht_device.hpp"
+#include "hadamard_device.hpp"
 
 namespace mi {
 namespace {
-
-// ---- element I/O -------------------------------------------------------------------------------
-// Each IO policy loads a lane's share of one tile into MFMA input form and stores two f32x4
-// accumulators back, both guarded against the end of the buffer (`total` elements).
-
-template <class T16_>
-struct Io16 {
-    using T16 = T16_;
-    using E = typename T16::E;
-    static constexpr int ESIZE = 2;
-    struct In {
-        typename T16::V8 a;
-    };
-
-    template <bool GUARD>
-    static __device__ __forceinline__ In load(const void* base, uint64_t tile, uint64_t total)
-    {
-        const E* p = static_cast<const E*>(base);
-        const uint64_t off = tile * 512u + 8u * (threadIdx.x & 63u);
-        In in;
-        if (!GUARD || off + 8u <= total) {
-            in.a = *reinterpret_cast<const typename T16::V8*>(p + off);
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) in.a[j] = (off + j < total) ? p[off + j] : (E)0.0f;
-        }
-        return in;
-    }
-
-    static __device__ __forceinline__ void transform(const In& in, const TileOperands<T16>& ops,
-                                                     f32x4 (&acc)[2])
-    {
-        tile_transform<T16>(in.a, ops, acc);
-    }
-
-    template <bool GUARD, bool MUL>
-    static __device__ __forceinline__ void store(void* base, uint64_t tile, uint64_t total,
-                                                 const f32x4 (&acc)[2], float s)
-    {
-        E* p = static_cast<E*>(base);
-        const uint64_t off = tile * 512u + 8u * (threadIdx.x & 63u);
-        typename T16::V8 o;
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) o[4 * t + r] = (E)(MUL ? acc[t][r] * s : acc[t][r]);
-        if (!GUARD || off + 8u <= total) {
-            *reinterpret_cast<typename T16::V8*>(p + off) = o;
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                if (off + j < total) p[off + j] = o[j];
-        }
-    }
-};
-
-struct Io32 {
-    using T16 = BF16;  // matrix-core type used for the three-piece products
-    static constexpr int ESIZE = 4;
-    struct In {
-        float v[8];
-    };
-
-    template <bool GUARD>
-    static __device__ __forceinline__ In load(const void* base, uint64_t tile, uint64_t total)
-    {
-        const float* p = static_cast<const float*>(base);
-        In in;
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const uint64_t off = tile * 512u + 256u * t + 4u * (threadIdx.x & 63u);
-            if (!GUARD || off + 4u <= total) {
-                const f32x4 q = *reinterpret_cast<const f32x4*>(p + off);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) in.v[4 * t + r] = q[r];
-            } else {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) in.v[4 * t + r] = (off + r < total) ? p[off + r] : 0.0f;
-            }
-        }
-        return in;
-    }
-
-    static __device__ __forceinline__ void transform(const In& in, const TileOperands<BF16>& ops,
-                                                     f32x4 (&acc)[2])
-    {
-        tile_transform_f32(in.v, ops, acc);
-    }
-
-    template <bool GUARD, bool MUL>
-    static __device__ __forceinline__ void store(void* base, uint64_t tile, uint64_t total,
-                                                 const f32x4 (&acc)[2], float s)
-    {
-        float* p = static_cast<float*>(base);
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const uint64_t off = tile * 512u + 256u * t + 4u * (threadIdx.x & 63u);
-            const f32x4 o = MUL ? acc[t] * s : acc[t];
-            if (!GUARD || off + 4u <= total) {
-                *reinterpret_cast<f32x4*>(p + off) = o;
-            } else {
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    if (off + r < total) p[off + r] = o[r];
-            }
-        }
-    }
-};
 
 // ---- register kernel: NT tiles per wavefront step, XB cross-tile bits ----------------------------
 // A wavefront handles the steps  first, first + stride, ...  (one step = NT tiles = one row when
@@ -137,8 +29,6 @@ __global__ void __launch_bounds__(256)
 fwht_reg_kernel(const void* in, void* out, uint64_t total, uint64_t num_steps, uint32_t p, int exp2,
                 float mult)
 {
-    // `in` may equal `out`: a wavefront reads all tiles of a step before it writes any, and steps
-    // own disjoint tiles, which is what makes in-place operation safe.
     const uint64_t first = (uint64_t)blockIdx.x * 4u + (threadIdx.x >> 6);
     const uint64_t stride = (uint64_t)gridDim.x * 4u;
     if (first >= num_steps) return;  // uniform per wavefront
@@ -146,105 +36,33 @@ fwht_reg_kernel(const void* in, void* out, uint64_t total, uint64_t num_steps, u
     TileOperands<typename IO::T16> ops;
     make_tile_operands<typename IO::T16, IO::ESIZE>(p, ops, exp2);
 
-    // GUARD = false when every tile of the step lies inside the buffer (always, except for the
-    // last step of a ragged n <= 512 problem): no bounds code on the hot path.
-    auto body = [&](uint64_t step, auto guard_tag) {
-        constexpr bool GUARD = decltype(guard_tag)::value;
-        typename IO::In tin[NT];
-#pragma unroll
-        for (int c = 0; c < NT; ++c) tin[c] = IO::template load<GUARD>(in, step * NT + c, total);
-        // keep every load of the step in flight before any arithmetic is scheduled
-        __builtin_amdgcn_sched_barrier(0);
-
-        f32x4 acc[NT][2];
-#pragma unroll
-        for (int c = 0; c < NT; ++c) IO::transform(tin[c], ops, acc[c]);
-
-        cross_tile_butterflies<NT, XB>(acc);
-
-#pragma unroll
-        for (int c = 0; c < NT; ++c)
-            IO::template store<GUARD, MUL>(out, step * NT + c, total, acc[c], mult);
-    };
+    // Unguarded when every tile of the step lies inside the buffer (always, except for the last
+    // step of a ragged n <= 512 problem): no bounds code on the hot path.
     for (uint64_t step = first; step < num_steps; step += stride) {
         if constexpr (XB > 0) {
-            body(step, std::false_type{});  // whole rows: nothing to guard
+            wave_fwht_step<IO, NT, XB, false, MUL>(in, out, step, total, ops, mult);
         } else {
             if ((step * NT + NT) * 512u <= total)
-                body(step, std::false_type{});
+                wave_fwht_step<IO, NT, XB, false, MUL>(in, out, step, total, ops, mult);
             else
-                body(step, std::true_type{});
+                wave_fwht_step<IO, NT, XB, true, MUL>(in, out, step, total, ops, mult);
         }
     }
 }
 
 // ---- LDS kernel: one workgroup of W = 2^LW wavefronts per row of n = 4096 * W ----------------
-// Pass 1: wavefront w transforms elements [4096w, 4096w+4096) (12 bits).  Exchange: every
-// accumulator quad goes to LDS once; wavefront w then gathers, from all W sub-rows, the 8/W tiles
-// it owns, runs the LW remaining butterflies in registers and stores.
 template <class IO, int LW, bool MUL>
 __global__ void __launch_bounds__(64 << LW)
 fwht_lds_kernel(const void* in, void* out, uint64_t rows, int exp2, float mult)
 {
-    constexpr int W = 1 << LW;
-    constexpr int OWN = 8 / W;  // tiles per sub-row owned by a wavefront in pass 2
-    extern __shared__ f32x4 xch[];  // [W sub-rows][8 tiles][2 halves][64 lanes]
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t w = threadIdx.x >> 6;
+    extern __shared__ f32x4 xch[];
     const uint64_t row = blockIdx.x;
     if (row >= rows) return;
     const uint64_t total = rows << (12 + LW);
-    const uint64_t tile0 = row * (8u * W);
 
     TileOperands<typename IO::T16> ops;
     make_tile_operands<typename IO::T16, IO::ESIZE>(12 + LW, ops, exp2);
-
-    {
-        typename IO::In tin[8];
-#pragma unroll
-        for (int c = 0; c < 8; ++c) tin[c] = IO::template load<false>(in, tile0 + w * 8u + c, total);
-        f32x4 acc[8][2];
-#pragma unroll
-        for (int c = 0; c < 8; ++c) IO::transform(tin[c], ops, acc[c]);
-        cross_tile_butterflies<8, 3>(acc);
-#pragma unroll
-        for (int c = 0; c < 8; ++c)
-#pragma unroll
-            for (int t = 0; t < 2; ++t) xch[((w * 8u + c) * 2u + t) * 64u + lane] = acc[c][t];
-    }
-    __syncthreads();
-
-    f32x4 g[W * OWN][2];  // index s * OWN + c'
-#pragma unroll
-    for (int s = 0; s < W; ++s)
-#pragma unroll
-        for (int cc = 0; cc < OWN; ++cc)
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-                g[s * OWN + cc][t] = xch[((s * 8u + w * OWN + cc) * 2u + t) * 64u + lane];
-
-    // butterflies over the sub-row index s (element bits 12 .. 12+LW-1)
-#pragma unroll
-    for (int b = 0; b < LW; ++b)
-#pragma unroll
-        for (int s = 0; s < W; ++s) {
-            if (s & (1 << b)) continue;
-#pragma unroll
-            for (int cc = 0; cc < OWN; ++cc)
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    const f32x4 x = g[s * OWN + cc][t], y = g[(s | (1 << b)) * OWN + cc][t];
-                    g[s * OWN + cc][t] = x + y;
-                    g[(s | (1 << b)) * OWN + cc][t] = x - y;
-                }
-        }
-
-#pragma unroll
-    for (int s = 0; s < W; ++s)
-#pragma unroll
-        for (int cc = 0; cc < OWN; ++cc)
-            IO::template store<false, MUL>(out, tile0 + s * 8u + w * OWN + cc, total,
-                                           g[s * OWN + cc], mult);
+    block_fwht_row<IO, LW, MUL>(in, out, row * (8u << LW), total, xch, ops, mult);
 }
 
 // ---- host dispatch --------------------------------------------------------------------------------

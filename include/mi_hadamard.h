@@ -142,6 +142,17 @@ int mi_debug_mfma_16x16(int kind, const void* A, const void* B, float* D, void* 
  */
 int mi_debug_convert(int kind, const float* in, void* out, uint64_t count, void* stream);
 
+/*
+ * Same contract as mi_fwht, but computed by a minimal kernel written against the device-side
+ * embedding API (csrc/hadamard_device.hpp: HadamardTransformDevice<IO, LOG_N>), one call of
+ * hadamard_transform_device per workgroup.  Exists so the embedding API -- the counterpart of the
+ * reference's  HadamardTransform<dtype,N>::hadamard_transform_device  (csrc/hada_handler.cuh:
+ * 227-264, thin caller csrc/main.cu:42-53) -- is tested for every length and element type.
+ *   rows must be a multiple of the API's N_ROWS (512 / n for n <= 512, else 1): MI_ERR_SHAPE.
+ */
+int mi_debug_device_fwht(const void* in, void* out, uint64_t rows, uint32_t n, int dtype,
+                         float scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
