@@ -4,15 +4,18 @@
 // benchmark configuration).
 //
 // Workgroup tile 256 x 256, four wavefronts of 128 x 128, K walked in steps of 128 bytes with
-// v_mfma_f32_16x16x128_f8f6f4 (unscaled form).  Both operand tiles go global -> registers (eight
-// lanes per 128-byte row segment, so the L1 coalesces) -> LDS, double buffered: the loads of
-// step s+1 are in flight while step s is multiplied.  LDS tiles are [256 rows][8 chunks of 16 B]
+// v_mfma_f32_16x16x128_f8f6f4 (unscaled form).  Both operand tiles go global -> LDS directly (eight
+// lanes per 128-byte row segment, so the L1 coalesces), double buffered: the loads of step s+1
+// are in flight while step s is multiplied, and the first fragments of step s+1 are read from
+// LDS behind the last MFMAs of step s.  LDS tiles are [256 rows][8 chunks of 16 B]
 // with chunk c of LDS row r stored at c ^ (r & 7); a lane of K-group hi reads chunks hi and hi + 4
 // of its row (any K assignment works as long as both operands use the same one).  Both the staging
 // writes and these fragment reads measured bank-conflict free; chunks 2*hi, 2*hi + 1 did not.
 // qb rows are the MFMA A operand and are stored in LDS in the order that lets a lane own 32
 // consecutive output columns; the result is staged through LDS once more so that C rows are
 // written as whole 512-byte runs.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace mi {
@@ -83,15 +86,17 @@ fp8_gemm_rowscale_kernel(const uint8_t* __restrict__ qa, const float* __restrict
     }
     typedef __attribute__((address_space(1))) const void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
-    auto stage = [&](uint32_t buf, uint32_t k0) {
+    // instruction pair i (of 8) of the transfer of K step k0 / 128 into LDS buffer `buf`
+    auto stage_part = [&](uint32_t buf, uint32_t k0, int i) {
         unsigned char* A = lds + buf * (2u * kTileBytes);
         unsigned char* B = A + kTileBytes;
+        const uint32_t run = (32u * i + 8u * wave) * 128u;  // wavefront-uniform
+        __builtin_amdgcn_global_load_lds((gptr_t)(qb + (ob[i] + k0)), (lptr_t)(B + run), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(qa + (oa[i] + k0)), (lptr_t)(A + run), 16, 0, 0);
+    };
+    auto stage = [&](uint32_t buf, uint32_t k0) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t run = (32u * i + 8u * wave) * 128u;  // wavefront-uniform
-            __builtin_amdgcn_global_load_lds((gptr_t)(qb + (ob[i] + k0)), (lptr_t)(B + run), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((gptr_t)(qa + (oa[i] + k0)), (lptr_t)(A + run), 16, 0, 0);
-        }
+        for (int i = 0; i < 8; ++i) stage_part(buf, k0, i);
     };
 
     f32x4 acc[8][8];  // [nb][ti]
@@ -101,47 +106,85 @@ fp8_gemm_rowscale_kernel(const uint8_t* __restrict__ qa, const float* __restrict
         for (int ti = 0; ti < 8; ++ti) acc[nb][ti] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     const uint32_t ksteps = K / kStepBytes;
-    // Pipeline: the operands of step ks+1 stream into the other LDS buffer while step ks is
-    // multiplied; every wavefront waits for its own transfers before the barrier that ends the step.
-    stage(0, 0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+    auto frag = [&](const unsigned char* tile, uint32_t r) {
+        const u32x4 x0 = *reinterpret_cast<const u32x4*>(tile + tile_off(r, hi));
+        const u32x4 x1 = *reinterpret_cast<const u32x4*>(tile + tile_off(r, hi + 4u));
+        return i32x8{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3],
+                     (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
+    };
+    const uint32_t ra0 = 128u * wn + lo;  // first LDS row of this lane's qb fragments (MFMA A)
+    const uint32_t rb0 = 128u * wt + lo;  // first LDS row of its qa fragments (MFMA B)
 
+    // Two LDS buffers, transfers running two steps ahead of the multiplication.  The barrier of
+    // step ks sits after the sixth of its eight fragment columns: by then every LDS read of the
+    // current buffer has been issued and waited for, and the transfer of step ks+1 (started two
+    // steps earlier) has landed.  Behind the barrier the current buffer is refilled with step ks+2
+    // (half of the transfer instructions in the shadow of the last sixteen MFMAs, the other half
+    // behind the first sixteen of the next step), and the fragments step ks+1 starts with are
+    // read, each qb fragment right after its last use.
+    stage(0, 0);
+    {
+        const uint32_t k1 = ksteps > 1 ? 1u : 0u;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) stage_part(1, k1 * kStepBytes, i);
+    }
+    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");  // the 16 transfers of step 0 are the oldest
+    __syncthreads();
+    i32x8 af[8], b0, b1;
+#pragma unroll
+    for (int nb = 0; nb < 8; ++nb) af[nb] = frag(lds + kTileBytes, ra0 + 16u * nb);
+    b0 = frag(lds, rb0);
+    b1 = frag(lds, rb0 + 16u);
+    // The body is branch-free: the last two steps of a tile repeat transfers of earlier K steps
+    // (valid addresses, results never read) and read fragments nobody uses, which is cheaper than
+    // conditional code on the matrix-core critical path.  Those stray transfers are drained before
+    // the epilogue reuses LDS.
+#pragma unroll 1
     for (uint32_t ks = 0; ks < ksteps; ++ks) {
         const uint32_t buf = ks & 1u;
-        if (ks + 1 < ksteps) stage(buf ^ 1u, (ks + 1) * kStepBytes);
+        const uint32_t k1 = ks + 1 < ksteps ? ks + 1 : 0u;                          // step after this one
+        const uint32_t k2 = ks + 2 < ksteps ? ks + 2 : 0u;  // and the next
         const unsigned char* A = lds + buf * (2u * kTileBytes);  // qa tile
-        const unsigned char* B = A + kTileBytes;                  // qb tile
-
-        i32x8 af[8];  // MFMA A operand fragments: qb rows, block nb
+        const unsigned char* An = lds + (buf ^ 1u) * (2u * kTileBytes);
+        i32x8 bfr[8];
+        bfr[0] = b0;
+        bfr[1] = b1;
 #pragma unroll
-        for (int nb = 0; nb < 8; ++nb) {
-            const uint32_t r = 128u * wn + 16u * nb + lo;
-            const u32x4 x0 = *reinterpret_cast<const u32x4*>(B + tile_off(r, hi));
-            const u32x4 x1 = *reinterpret_cast<const u32x4*>(B + tile_off(r, hi + 4u));
-            af[nb] = i32x8{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3],
-                           (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
-        }
-        auto read_b = [&](int ti) {
-            const uint32_t r = 128u * wt + 16u * ti + lo;
-            const u32x4 x0 = *reinterpret_cast<const u32x4*>(A + tile_off(r, hi));
-            const u32x4 x1 = *reinterpret_cast<const u32x4*>(A + tile_off(r, hi + 4u));
-            return i32x8{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3],
-                         (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
-        };
-        i32x8 bf_nx = read_b(0);
+        for (int ti = 0; ti < 6; ++ti) {
 #pragma unroll
-        for (int ti = 0; ti < 8; ++ti) {
-            const i32x8 bf = bf_nx;
-            if (ti + 1 < 8) bf_nx = read_b(ti + 1);
-#pragma unroll
-            for (int nb = 0; nb < 8; ++nb)
-                acc[nb][ti] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[nb], bf, acc[nb][ti],
-                                                                              0, 0, 0, 0, 0, 0);
+            for (int nb = 0; nb < 8; ++nb) {
+                acc[nb][ti] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                    af[nb], bfr[ti], acc[nb][ti], 0, 0, 0, 0, 0, 0);
+                if (nb == 0) bfr[ti + 2] = frag(A, rb0 + 16u * (ti + 2));
+                if (ti < 2 && (nb & 3) == 1)
+                    stage_part(buf ^ 1u, k1 * kStepBytes, 4 + 2 * ti + (nb >> 2));
+            }
+            // keep the scheduler from hoisting later fragment reads up here: with all 512
+            // registers in use, longer live ranges turn into accumulator shuffling
+            __builtin_amdgcn_sched_barrier(0);
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
+#pragma unroll
+        for (int nb = 0; nb < 8; ++nb) {
+            if (nb == 0) b0 = frag(An, rb0);
+            if (nb == 1) b1 = frag(An, rb0 + 16u);
+            acc[nb][6] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                af[nb], bfr[6], acc[nb][6], 0, 0, 0, 0, 0, 0);
+            if ((nb & 3) == 2) stage_part(buf, k2 * kStepBytes, nb >> 2);
+            if ((nb & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int nb = 0; nb < 8; ++nb) {
+            acc[nb][7] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                af[nb], bfr[7], acc[nb][7], 0, 0, 0, 0, 0, 0);
+            af[nb] = frag(An + kTileBytes, ra0 + 16u * nb);
+            if ((nb & 3) == 2) stage_part(buf, k2 * kStepBytes, 2 + (nb >> 2));
+            if (nb & 1) __builtin_amdgcn_sched_barrier(0);
+        }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
 
     // ---- epilogue: scale, narrow, stage through LDS, store whole rows ---------------------------
     // D[m'][n']: n' = lo -> qa row t0 + 128*wt + 16*ti + lo; m' = 4*hi + r -> column
@@ -188,7 +231,9 @@ fp8_gemm_rowscale_kernel(const uint8_t* __restrict__ qa, const float* __restrict
         if (t < T && col < N) {
             __bf16* dst = out + (uint64_t)t * N + col;
             if (vec_ok && col + 8u <= N) {
-                *reinterpret_cast<bf16x8v*>(dst) = o;
+                // streaming store: the result is not read again here, and keeping it out of the
+                // caches leaves them to the operand panels that the following tiles re-read
+                __builtin_nontemporal_store(o, reinterpret_cast<bf16x8v*>(dst));
             } else {
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
