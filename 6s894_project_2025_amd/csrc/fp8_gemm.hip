@@ -28,6 +28,17 @@ constexpr int kStepBytes = 128;      // K bytes per step
 constexpr int kTileBytes = kTile * kStepBytes;  // 32 KB
 constexpr int kThreads = 256;
 
+// acc += A(16 x 128, E4M3FN) * B(128 x 16, E4M3FN) with the accumulator tied in place in the AGPR
+// file.  Written as inline assembly because, with all 256 AGPRs holding accumulators, the
+// compiler's own MFMA selection kept shuffling accumulators between register files inside the K
+// loop.  Hazards the compiler can no longer see: the operands come from LDS reads (ordinary
+// register dependencies, which it still tracks), the two idle cycles cover a VALU-written operand,
+// and the accumulators are first read after the drain at the end of the K loop.
+__device__ __forceinline__ void mfma_fp8(f32x4& c, const i32x8& a, const i32x8& b)
+{
+    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+
 __device__ __forceinline__ uint32_t tile_off(uint32_t row, uint32_t chunk)
 {
     return (row * 8u + (chunk ^ (row & 7u))) << 4;
@@ -47,7 +58,9 @@ fp8_gemm_rowscale_kernel(const uint8_t* __restrict__ qa, const float* __restrict
                          uint32_t tiles_t, uint32_t tiles_n)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // 2 x (A tile + B tile)
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    // wavefront index as a scalar, so LDS bases of the direct transfers (M0) are scalar arithmetic
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t lo = lane & 15u, hi = lane >> 4;
     const uint32_t wt = wave >> 1, wn = wave & 1u;
 
@@ -153,8 +166,7 @@ fp8_gemm_rowscale_kernel(const uint8_t* __restrict__ qa, const float* __restrict
         for (int ti = 0; ti < 6; ++ti) {
 #pragma unroll
             for (int nb = 0; nb < 8; ++nb) {
-                acc[nb][ti] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                    af[nb], bfr[ti], acc[nb][ti], 0, 0, 0, 0, 0, 0);
+                mfma_fp8(acc[nb][ti], af[nb], bfr[ti]);
                 if (nb == 0) bfr[ti + 2] = frag(A, rb0 + 16u * (ti + 2));
                 if (ti < 2 && (nb & 3) == 1)
                     stage_part(buf ^ 1u, k1 * kStepBytes, 4 + 2 * ti + (nb >> 2));
@@ -169,21 +181,20 @@ fp8_gemm_rowscale_kernel(const uint8_t* __restrict__ qa, const float* __restrict
         for (int nb = 0; nb < 8; ++nb) {
             if (nb == 0) b0 = frag(An, rb0);
             if (nb == 1) b1 = frag(An, rb0 + 16u);
-            acc[nb][6] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                af[nb], bfr[6], acc[nb][6], 0, 0, 0, 0, 0, 0);
+            mfma_fp8(acc[nb][6], af[nb], bfr[6]);
             if ((nb & 3) == 2) stage_part(buf, k2 * kStepBytes, nb >> 2);
             if ((nb & 3) == 3) __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
         for (int nb = 0; nb < 8; ++nb) {
-            acc[nb][7] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                af[nb], bfr[7], acc[nb][7], 0, 0, 0, 0, 0, 0);
+            mfma_fp8(acc[nb][7], af[nb], bfr[7]);
             af[nb] = frag(An + kTileBytes, ra0 + 16u * nb);
             if ((nb & 3) == 2) stage_part(buf, k2 * kStepBytes, 2 + (nb >> 2));
             if (nb & 1) __builtin_amdgcn_sched_barrier(0);
         }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // drain: stray transfers, and the matrix-core pipeline before the accumulators are read
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
     // ---- epilogue: scale, narrow, stage through LDS, store whole rows ---------------------------
