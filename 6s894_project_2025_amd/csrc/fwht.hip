@@ -91,7 +91,7 @@ int launch_lds(const void* in, void* out, uint64_t rows, OutputScale os, hipStre
 {
     if (rows == 0) return MI_OK;
     if (rows > 0x7fffffffull) return MI_ERR_SHAPE;
-    constexpr size_t lds = sizeof(f32x4) * 64u * 16u * (1u << LW);
+    constexpr size_t lds = sizeof(f32x4) * 64u * 8u * (1u << LW);
     const bool mul = os.mult != 1.0f;
     auto kern = mul ? fwht_lds_kernel<IO, LW, true> : fwht_lds_kernel<IO, LW, false>;
     if (lds > 64u * 1024u) {

@@ -166,7 +166,7 @@ __device__ __forceinline__ void wave_fwht_step(const void* in, void* out, uint64
 // Pass 1: wavefront w transforms elements [4096w, 4096w+4096) (12 bits).  Exchange: every
 // accumulator quad goes to LDS once; wavefront w then gathers, from all W sub-rows, the 8/W tiles
 // it owns, runs the LW remaining butterflies in registers and stores.  `xch` holds
-// 16 * 64 * 16 * W bytes; all 64*W threads must call (one __syncthreads inside).
+// 16 * 64 * 8 * W bytes; all 64*W threads must call (__syncthreads inside).
 template <class IO, int LW, bool MUL>
 __device__ __forceinline__ void block_fwht_row(const void* in, void* out, uint64_t tile0,
                                                uint64_t total, f32x4* xch,
@@ -176,30 +176,30 @@ __device__ __forceinline__ void block_fwht_row(const void* in, void* out, uint64
     constexpr int OWN = 8 / W;  // tiles per sub-row owned by a wavefront in pass 2
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t w = threadIdx.x >> 6;
-    // xch layout: [W sub-rows][8 tiles][2 halves][64 lanes]
+    // xch layout: [W sub-rows][8 tiles][64 lanes], used twice (once per accumulator half), which
+    // halves the LDS footprint and lets two workgroups share a compute unit at W = 8
+    f32x4 acc[8][2];
     {
         typename IO::In tin[8];
 #pragma unroll
         for (int c = 0; c < 8; ++c) tin[c] = IO::template load<false>(in, tile0 + w * 8u + c, total);
-        f32x4 acc[8][2];
 #pragma unroll
         for (int c = 0; c < 8; ++c) IO::transform(tin[c], ops, acc[c]);
         cross_tile_butterflies<8, 3>(acc);
-#pragma unroll
-        for (int c = 0; c < 8; ++c)
-#pragma unroll
-            for (int t = 0; t < 2; ++t) xch[((w * 8u + c) * 2u + t) * 64u + lane] = acc[c][t];
     }
-    __syncthreads();
-
     f32x4 g[W * OWN][2];  // index s * OWN + c'
 #pragma unroll
-    for (int s = 0; s < W; ++s)
+    for (int t = 0; t < 2; ++t) {
+        if (t) __syncthreads();  // every wavefront has read the first half
 #pragma unroll
-        for (int cc = 0; cc < OWN; ++cc)
+        for (int c = 0; c < 8; ++c) xch[(w * 8u + c) * 64u + lane] = acc[c][t];
+        __syncthreads();
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
-                g[s * OWN + cc][t] = xch[((s * 8u + w * OWN + cc) * 2u + t) * 64u + lane];
+        for (int s = 0; s < W; ++s)
+#pragma unroll
+            for (int cc = 0; cc < OWN; ++cc)
+                g[s * OWN + cc][t] = xch[(s * 8u + w * OWN + cc) * 64u + lane];
+    }
 
     // butterflies over the sub-row index s (element bits 12 .. 12+LW-1)
 #pragma unroll
@@ -242,7 +242,7 @@ struct HadamardTransformDevice {
     static constexpr int LW = LOG_N > 12 ? LOG_N - 12 : 0;
     static constexpr int THREADS = 64 << LW;
     static constexpr int N_ROWS = LOG_N <= 9 ? (512 >> LOG_N) : 1;
-    static constexpr int LDS_BYTES = LOG_N > 12 ? (int)sizeof(f32x4) * 64 * 16 * (1 << LW) : 0;
+    static constexpr int LDS_BYTES = LOG_N > 12 ? (int)sizeof(f32x4) * 64 * 8 * (1 << LW) : 0;
 
     static __device__ __forceinline__ Operands prepare(OutputScale os)
     {
