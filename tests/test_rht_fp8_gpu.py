@@ -67,7 +67,8 @@ def test_quant_full_size_config(pkg, oracle):
     assert not ((codes & 0x7F) == 0x7F).any()
 
 
-@pytest.mark.parametrize("T,N,K", [(16, 16, 128), (100, 70, 256), (256, 384, 512), (130, 129, 1024)])
+@pytest.mark.parametrize("T,N,K", [(16, 16, 128), (100, 70, 256), (256, 384, 512), (130, 129, 1024),
+                                   (16, 16, 384), (600, 520, 640)])
 def test_fp8_gemm_against_dequantised_product(pkg, oracle, T, N, K):
     g = torch.Generator().manual_seed(5)
     a = torch.randn(T, K, generator=g)
@@ -83,6 +84,29 @@ def test_fp8_gemm_against_dequantised_product(pkg, oracle, T, N, K):
     db = oracle.e4m3fn_decode(qb).astype(np.float64) * sb[:, None].astype(np.float64)
     want = da @ db.T
     assert oracle.rel_err(out.cpu().double().numpy(), want) <= 2e-2
+
+
+def test_fp8_gemm_full_size_sampled_rows(pkg, oracle):
+    # the benchmark shape (T = 8192, N = 14336, K = 4096): 48 sampled rows of the output against
+    # the oracle's dequantised fp64 product; every tile row and every column tile is touched
+    T, N, K = 8192, 14336, 4096
+    g = torch.Generator().manual_seed(9)
+    qa = torch.randint(0, 0x7E, (T, K), generator=g, dtype=torch.uint8)
+    qa |= (torch.randint(0, 2, (T, K), generator=g, dtype=torch.uint8) << 7)
+    qb = torch.randint(0, 0x7E, (N, K), generator=g, dtype=torch.uint8)
+    qb |= (torch.randint(0, 2, (N, K), generator=g, dtype=torch.uint8) << 7)
+    sa = torch.rand(T, generator=g) * 1e-2 + 1e-3
+    sb = torch.rand(N, generator=g) * 1e-2 + 1e-3
+    out = pkg.fp8_gemm_rowscale(qa.cuda().view(torch.float8_e4m3fn), sa.cuda(),
+                                qb.cuda().view(torch.float8_e4m3fn), sb.cuda())
+    torch.cuda.synchronize()
+    rows = torch.cat([torch.arange(0, T, 256) + torch.randint(0, 256, (T // 256,), generator=g),
+                      torch.tensor([0, 255, 256, T - 1]), torch.randint(0, T, (12,), generator=g)])
+    da = oracle.e4m3fn_decode(qa[rows].numpy()).astype(np.float64) * sa[rows, None].double().numpy()
+    db = oracle.e4m3fn_decode(qb.numpy()).astype(np.float64) * sb[:, None].double().numpy()
+    want = da @ db.T
+    got = out[rows.cuda()].cpu().double().numpy()
+    assert oracle.rel_err(got, want) <= 2e-2
 
 
 def test_rht_fp8_linear_end_to_end(pkg, oracle):
