@@ -90,6 +90,8 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-fwht", action="store_true", help="headline kernel only (profiling)")
     ap.add_argument("--only-gemm", action="store_true", help="fused GEMM only (profiling)")
+    ap.add_argument("--only-rht", action="store_true",
+                    help="RHT + FP8 quantize and FP8 GEMM only (profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.stderr.write("bench.py: this build runs on exactly one GPU; --gpus must be 1 "
@@ -111,7 +113,7 @@ def main() -> int:
     g = torch.Generator().manual_seed(0)
     x_cpu = torch.randn(rows, n, generator=g, dtype=torch.float32).to(torch.bfloat16)
     result = {}
-    if not args.only_gemm:
+    if not (args.only_gemm or args.only_rht):
         x = x_cpu.to(dev)
         ms, wall_ms = _events_ms(torch, lambda: hada.hadamard_transform(x, inplace=True), steps, warmup)
         alg_bytes = 2 * rows * n * 2
@@ -149,7 +151,7 @@ def main() -> int:
     K = 1024
     gsteps = max(10, min(steps, 200))
     others = {}
-    for name, dt in (("bf16", torch.bfloat16), ("f32", torch.float32)):
+    for name, dt in (() if args.only_rht else (("bf16", torch.bfloat16), ("f32", torch.float32))):
         W = torch.randn(M, K, generator=torch.Generator().manual_seed(1)).to(dt).to(dev)
         Xt = torch.randn(N, K, generator=torch.Generator().manual_seed(0)).to(dt).to(dev)
         C = hada.fused_ht_gemm(W, Xt)
@@ -175,7 +177,8 @@ def main() -> int:
         del W, Xt, C
 
     # ---- remaining configurations --------------------------------------------------------------------
-    for (m, nn, b) in ((256, 256, 512), (1024, 1024, 8), (1024, 1024, 64), (1024, 1024, 512)):
+    for (m, nn, b) in (() if args.only_rht else
+                       ((256, 256, 512), (1024, 1024, 8), (1024, 1024, 64), (1024, 1024, 512))):
         W = torch.randn(m, nn, device=dev) / math.sqrt(nn)
         X = torch.randn(nn, b, device=dev)
         ms, _ = _events_ms(torch, lambda: hada.fused_ht_gemv(W, X), 50, 3)
@@ -186,7 +189,10 @@ def main() -> int:
             "GB/s": round(4 * (m * nn + nn * b + m * b) / ms / 1e6, 1),
             "TFLOP/s": round((2 * m * nn * b + nn * math.log2(nn) * b) / ms / 1e9, 3)}
     T, nq, Nw = 8192, 4096, 14336
-    xa = torch.randn(T, nq, device=dev).to(torch.bfloat16)
+    xa = torch.randn(T, nq, generator=torch.Generator().manual_seed(0))
+    outl = torch.randperm(nq, generator=torch.Generator().manual_seed(3))[:41]  # 1 % outlier channels
+    xa[:, outl] *= 50.0
+    xa = xa.to(torch.bfloat16).to(dev)
     sign = (1 - 2 * torch.randint(0, 2, (nq,), generator=torch.Generator().manual_seed(2))).to(torch.int8).to(dev)
     ms, _ = _events_ms(torch, lambda: hada.rht_quant_fp8(xa, sign), 50, 3)
     qbytes = T * nq * 3 + T * 4
@@ -204,8 +210,11 @@ def main() -> int:
         "us": round(ms * 1e3, 1), "algorithmic_flops": fl, "TFLOP/s": round(fl / ms / 1e9, 1),
         "roofline": {"bound": "mfma", "achieved": round(fl / ms / 1e9, 1), "peak": PEAK_TFLOPS["fp8"],
                      "unit": "TFLOP/s", "frac": round(fl / ms / 1e9 / PEAK_TFLOPS["fp8"], 4),
-                     "traffic": None}}
+                     "traffic": traffic.get("fp8_gemm_8192x14336x4096_l2_fill_plus_write")}}
     del xa, w, qx, qw
+    if args.only_rht:
+        print(json.dumps(others))
+        return 0
 
     if args.sweep:
         sweep = {}
