@@ -300,7 +300,7 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
                         if (m < m_end && col < N) {
                             E* dst = static_cast<E*>(C) + (uint64_t)m * N + col;
                             if (vec_ok && col + 8u <= N) {
-                                *reinterpret_cast<V8*>(dst) = o;
+                                __builtin_nontemporal_store(o, reinterpret_cast<V8*>(dst));
                             } else {
 #pragma unroll
                                 for (int j = 0; j < 8; ++j)
@@ -331,7 +331,7 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
                         if (m < m_end && col < N) {
                             float* dst = static_cast<float*>(C) + (uint64_t)m * N + col;
                             if (vec_ok && col + 4u <= N) {
-                                *reinterpret_cast<f32x4*>(dst) = o;
+                                __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(dst));
                             } else {
 #pragma unroll
                                 for (int j = 0; j < 4; ++j)

@@ -161,7 +161,7 @@ rht_quant_fp8_kernel(const __bf16* __restrict__ x, const int8_t* __restrict__ si
                 pk = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], pk, true);
                 codes[w] = (uint32_t)pk;
             }
-            *reinterpret_cast<u32x2*>(q + off) = codes;
+            __builtin_nontemporal_store(codes, reinterpret_cast<u32x2*>(q + off));  // streaming output
             if (y_out) *reinterpret_cast<bf16x8*>(y_out + off) = y[c];
         }
     }
