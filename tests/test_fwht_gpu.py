@@ -169,9 +169,6 @@ def test_involution_at_full_size(pkg, dt):
     nx = x.float().norm(dim=1)
     ny = y.float().norm(dim=1)
     assert ((ny - nx).abs() / nx).max().item() <= (1e-5 if dt == torch.float32 else 5e-3)
-    # first 64 rows against the oracle would need /root/reference-free fp64 math: done on device
-    H = None
-    del H
 
 
 def test_full_size_rows_against_oracle(pkg, oracle):
@@ -183,3 +180,38 @@ def test_full_size_rows_against_oracle(pkg, oracle):
     idx = [0, 1, 2, 3, 4095, 8191, 8192, 16383]
     y64 = oracle.fwht_f64(x[idx].to(torch.float64).numpy())
     assert oracle.rel_err(xd[idx].cpu().to(torch.float64).numpy(), y64) <= 2e-2
+
+
+def test_more_than_2_to_32_elements(pkg, oracle):
+    # the reference's seam counts elements in a u32 (csrc/main.cuh:5-6); rows is 64-bit here.
+    # 2^20 + 3 rows of 4096 bf16 = 4.29e9 elements (8.6 GB), in place; rows on both sides of the
+    # 2^32-element boundary and the ragged tail are compared with the fp64 oracle.
+    rows, n = (1 << 20) + 3, 4096
+    g = torch.Generator(device="cuda").manual_seed(11)
+    x = torch.empty(rows, n, dtype=torch.bfloat16, device="cuda")
+    for r0 in range(0, rows, 1 << 17):
+        x[r0:r0 + (1 << 17)] = torch.randn(min(1 << 17, rows - r0), n, generator=g, device="cuda")
+    idx = torch.tensor([0, 1, (1 << 19), (1 << 20) - 1, (1 << 20), (1 << 20) + 1, rows - 1])
+    before = x[idx.cuda()].cpu()
+    pkg.hadamard_transform(x, inplace=True)
+    torch.cuda.synchronize()
+    y64 = oracle.fwht_f64(before.to(torch.float64).numpy())
+    assert oracle.rel_err(x[idx.cuda()].cpu().to(torch.float64).numpy(), y64) <= 2e-2
+    del x
+
+
+def test_runs_on_the_callers_stream(pkg, oracle):
+    # asynchronous launch on torch's current stream (csrc/hadamard_transform.cpp:46-47): work queued
+    # on a side stream before the call is seen by it, work queued after sees its result
+    x_cpu = oracle.inputs_fwht(2048, 1024, torch.bfloat16)
+    side = torch.cuda.Stream()
+    x = x_cpu.cuda()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        t = x * 2                                   # producer on the side stream
+        y = pkg.hadamard_transform(t)               # must run after it, on the same stream
+        z = y.float().sum(dim=1)                    # consumer on the same stream
+    side.synchronize()
+    y64 = oracle.fwht_f64((x_cpu.float() * 2).to(torch.bfloat16).to(torch.float64).numpy())
+    assert oracle.rel_err(y.cpu().to(torch.float64).numpy(), y64) <= 2e-2
+    assert torch.allclose(z.cpu(), y.float().sum(dim=1).cpu(), rtol=1e-3, atol=1e-2)
