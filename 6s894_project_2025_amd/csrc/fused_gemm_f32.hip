@@ -4,8 +4,9 @@
 // the bf16 matrix cores with exact three-piece operands (tile_transform_f32), and the
 // contraction uses the fp32 matrix-core instruction v_mfma_f32_16x16x4_f32, so every product
 // and sum is fp32 (there is no reduced-precision shortcut on this hardware).
-// One 16-byte load per lane supplies four consecutive K for four MFMAs: lane (lo, hi) of K-step
-// kk holds k = 16*kk + 4*hi + s, s = 0..3, for both operands.
+// One 16-byte fragment per lane supplies four consecutive K for four MFMAs: lane (lo, hi) of K-step
+// kk holds k = 16*kk + 4*hi + s, s = 0..3, for both operands.  W reaches that order through a
+// wavefront-private LDS staging area (coalescable loads in, operand-order reads out).
 #include "fwht_device.hpp"
 
 namespace mi {
@@ -13,6 +14,7 @@ namespace {
 
 constexpr int kThreads = 512;
 constexpr int kWaves = kThreads / 64;
+constexpr int kStageBytes = 64 * 64;  // per wavefront: 64 rows x 16 K x 4 B
 
 template <int LOG_NB>
 __device__ __forceinline__ uint32_t y_off(uint32_t n, uint32_t q, uint32_t col_bytes,
@@ -74,6 +76,12 @@ fused_ht_gemm_f32_kernel(const float* __restrict__ W, const float* __restrict__ 
     }
     __syncthreads();
 
+    // staging layout: row r (64 bytes), 16-byte chunk c stored at position c ^ ((r >> 1) & 3)
+    // (conflict-free for both the writer's and the reader's lane order)
+    unsigned char* stage = ylds + (size_t)BN * K * 4u + wave * kStageBytes;
+    const uint32_t wr_off = (lane >> 2) * 64u + (((lane & 3u) ^ ((lane >> 3) & 3u)) << 4);
+    const uint32_t rd_off = lo * 64u + ((hi ^ ((lo >> 1) & 3u)) << 4);
+
     const uint32_t m_begin = blockIdx.y * m_per_block;
     const uint32_t m_end = min(M, m_begin + m_per_block);
     const uint32_t ksteps = K >> 4;
@@ -84,37 +92,60 @@ fused_ht_gemm_f32_kernel(const float* __restrict__ W, const float* __restrict__ 
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
             for (int mi = 0; mi < 4; ++mi) acc[nb][mi] = f32x4{0.f, 0.f, 0.f, 0.f};
-        const float* wrow[4];
+        // W goes global -> registers with four adjacent lanes on the 64 contiguous bytes a row
+        // contributes to a K step (the pattern the L1 coalesces; one lane per row, which is what
+        // the MFMA operand wants, runs at a third of the rate), then through a wavefront-private
+        // 4 KB LDS area into operand order.  Piece mi of the wavefront holds rows 16 mi + lane/4,
+        // 16-byte chunk lane%4; reader lane (hi, lo) takes row 16 mi + lo, chunk hi.  LDS
+        // operations of one wavefront complete in order, so no barrier is needed.
+        const float* wsrc[4];
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
-            const uint32_t m = min(mb + 16u * mi + lo, M - 1u);
-            wrow[mi] = W + (uint64_t)m * K + 4u * hi;
+            const uint32_t m = min(mb + 16u * mi + (lane >> 2), M - 1u);
+            wsrc[mi] = W + (uint64_t)m * K + 4u * (lane & 3u);
         }
-        f32x4 bcur[4], bnext[4];
+        // Software pipeline: while step kk is multiplied, the fragments of step kk+1 are already
+        // on their way out of LDS and the W pieces of step kk+2 are in flight from memory.
+        f32x4 wreg[4];   // W pieces of the step after the one whose fragments are being fetched
+        f32x4 a_nx[NB], b_nx[4];
+        auto fetch = [&](uint32_t kk) {  // wreg (step kk) -> staging -> fragments of step kk
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) bcur[mi] = *reinterpret_cast<const f32x4*>(wrow[mi]);
-
-        for (uint32_t kk = 0; kk < ksteps; ++kk) {
-            if (kk + 1 < ksteps) {
-#pragma unroll
-                for (int mi = 0; mi < 4; ++mi)
-                    bnext[mi] = *reinterpret_cast<const f32x4*>(wrow[mi] + 16u * (kk + 1));
-            }
-            f32x4 a[NB];
+            for (int mi = 0; mi < 4; ++mi)
+                *reinterpret_cast<f32x4*>(stage + mi * 1024u + wr_off) = wreg[mi];
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb)
-                a[nb] = *reinterpret_cast<const f32x4*>(
+                a_nx[nb] = *reinterpret_cast<const f32x4*>(
                     ylds + y_off<LOG_NB>(NB * lo + nb, 4u * kk + hi, col_bytes, swz_mask));
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi)
+                b_nx[mi] = *reinterpret_cast<const f32x4*>(stage + mi * 1024u + rd_off);
+        };
+        auto gload = [&](uint32_t kk) {
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi)
+                wreg[mi] = *reinterpret_cast<const f32x4*>(wsrc[mi] + 16u * kk);
+        };
+        gload(0);
+        fetch(0);
+        gload(1);  // K >= 32: at least two steps
+        for (uint32_t kk = 0; kk < ksteps; ++kk) {
+            f32x4 a[NB], b[4];
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) a[nb] = a_nx[nb];
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi) b[mi] = b_nx[mi];
+            if (kk + 1 < ksteps) {
+                fetch(kk + 1);
+                if (kk + 2 < ksteps) gload(kk + 2);
+            }
 #pragma unroll
             for (int s = 0; s < 4; ++s)
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
                     for (int mi = 0; mi < 4; ++mi)
-                        acc[nb][mi] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[nb][s], bcur[mi][s],
+                        acc[nb][mi] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[nb][s], b[mi][s],
                                                                            acc[nb][mi], 0, 0, 0);
-#pragma unroll
-            for (int mi = 0; mi < 4; ++mi) bcur[mi] = bnext[mi];
         }
 
 #pragma unroll
@@ -143,12 +174,13 @@ int launch(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, ui
     const float fscale = (float)((double)scale * (double)(1u << shift));
     const uint32_t n_tiles = (N + BN - 1) / BN;
     const uint32_t row_blocks = (M + 511u) / 512u;
-    uint32_t msplit = (512u + n_tiles - 1u) / n_tiles;
+    // one workgroup per compute unit fits (LDS): aim at one round of 256 workgroups
+    uint32_t msplit = (256u + n_tiles - 1u) / n_tiles;
     if (msplit < 1u) msplit = 1u;
     if (msplit > row_blocks) msplit = row_blocks;
     const uint32_t m_per_block = ((row_blocks + msplit - 1u) / msplit) * 512u;
     msplit = (M + m_per_block - 1u) / m_per_block;
-    const size_t lds = (size_t)BN * K * 4u;
+    const size_t lds = (size_t)BN * K * 4u + (size_t)kWaves * kStageBytes;
     auto kern = fused_ht_gemm_f32_kernel<BN, XB>;
     if (lds > 64u * 1024u) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
