@@ -95,7 +95,7 @@ def main() -> int:
     args = ap.parse_args()
     if args.gpus != 1:
         sys.stderr.write("bench.py: this build runs on exactly one GPU; --gpus must be 1 "
-                         "(rows shard across GPUs with no exchange, see DESIGN.md)\n")
+                         "(rows are independent, so several GPUs would each take a row slab with no exchange)\n")
         return 2
 
     import torch
