@@ -36,6 +36,22 @@ fwht_reg_kernel(const void* in, void* out, uint64_t total, uint64_t num_steps, u
     TileOperands<typename IO::T16> ops;
     make_tile_operands<typename IO::T16, IO::ESIZE>(p, ops, exp2);
 
+    if constexpr (XB > 0 && IO::ESIZE == 2) {
+        // whole rows, 16-bit elements: software pipeline, the loads of the wavefront's next row
+        // are in flight while this one is transformed and stored (`in` may equal `out`: the next
+        // row is a different row)
+        typename IO::In cur[NT], nxt[NT];
+        wave_fwht_load<IO, NT, false>(in, first, total, cur);
+        for (uint64_t step = first; step < num_steps; step += stride) {
+            if (step + stride < num_steps) wave_fwht_load<IO, NT, false>(in, step + stride, total, nxt);
+            __builtin_amdgcn_sched_barrier(0);
+            wave_fwht_finish<IO, NT, XB, false, MUL>(cur, out, step, total, ops, mult);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int c = 0; c < NT; ++c) cur[c] = nxt[c];
+        }
+        return;
+    }
     // Unguarded when every tile of the step lies inside the buffer (always, except for the last
     // step of a ragged n <= 512 problem): no bounds code on the hot path.
     for (uint64_t step = first; step < num_steps; step += stride) {

@@ -140,17 +140,20 @@ struct Io32 {
 // One step = tiles [step*NT, step*NT + NT) of the buffer = one row when XB > 0, several short rows
 // otherwise.  `in` may equal `out`: the wavefront reads all tiles of the step before it writes any.
 // GUARD = true bounds-checks every access against `total` elements (ragged last step only).
-template <class IO, int NT, int XB, bool GUARD, bool MUL>
-__device__ __forceinline__ void wave_fwht_step(const void* in, void* out, uint64_t step,
-                                               uint64_t total,
-                                               const TileOperands<typename IO::T16>& ops, float mult)
+template <class IO, int NT, bool GUARD>
+__device__ __forceinline__ void wave_fwht_load(const void* in, uint64_t step, uint64_t total,
+                                               typename IO::In (&tin)[NT])
 {
-    typename IO::In tin[NT];
 #pragma unroll
     for (int c = 0; c < NT; ++c) tin[c] = IO::template load<GUARD>(in, step * NT + c, total);
-    // keep every load of the step in flight before any arithmetic is scheduled
-    __builtin_amdgcn_sched_barrier(0);
+}
 
+template <class IO, int NT, int XB, bool GUARD, bool MUL>
+__device__ __forceinline__ void wave_fwht_finish(const typename IO::In (&tin)[NT], void* out,
+                                                 uint64_t step, uint64_t total,
+                                                 const TileOperands<typename IO::T16>& ops,
+                                                 float mult)
+{
     f32x4 acc[NT][2];
 #pragma unroll
     for (int c = 0; c < NT; ++c) IO::transform(tin[c], ops, acc[c]);
@@ -160,6 +163,18 @@ __device__ __forceinline__ void wave_fwht_step(const void* in, void* out, uint64
 #pragma unroll
     for (int c = 0; c < NT; ++c)
         IO::template store<GUARD, MUL>(out, step * NT + c, total, acc[c], mult);
+}
+
+template <class IO, int NT, int XB, bool GUARD, bool MUL>
+__device__ __forceinline__ void wave_fwht_step(const void* in, void* out, uint64_t step,
+                                               uint64_t total,
+                                               const TileOperands<typename IO::T16>& ops, float mult)
+{
+    typename IO::In tin[NT];
+    wave_fwht_load<IO, NT, GUARD>(in, step, total, tin);
+    // keep every load of the step in flight before any arithmetic is scheduled
+    __builtin_amdgcn_sched_barrier(0);
+    wave_fwht_finish<IO, NT, XB, GUARD, MUL>(tin, out, step, total, ops, mult);
 }
 
 // ---- workgroup level: W = 2^LW wavefronts transform one row of n = 4096 * W -----------------------
