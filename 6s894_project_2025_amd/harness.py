@@ -3,7 +3,8 @@
 Two sub-commands (run from the repository root)::
 
     python -m 6s894_project_2025_amd.harness fwht  [--check] [--runs-per-size 400] [--sizes ...]
-    python -m 6s894_project_2025_amd.harness fused [--dtype bf16|f32] [--runs 8]
+    python -m 6s894_project_2025_amd.harness fused [--dtype bf16|f32] [--runs 8] [--out-prefix P]
+    python -m 6s894_project_2025_amd.harness plot P.csv [--out-dir plots]
 
 ``fwht`` keeps the structure of the reference's bench/bench.py: a registry of in-place cases
 (three AddOne roofline proxies around the transform, :96-103), a correctness pass of every case
@@ -227,6 +228,46 @@ def run_fused(dtype: torch.dtype, runs: int = 8, configs=None, out_prefix: str |
     return rows
 
 
+def plot_fused(csv_path: str, out_dir: str = "plots") -> list[str]:
+    """Figures from the sweep CSV, the counterpart of fused_ht/plot_results.py: speed-up of the fused
+    kernel over the unfused baseline against K for every N = M, and achieved TFLOP/s of both."""
+    import os
+
+    import matplotlib
+    matplotlib.use("Agg")
+    import matplotlib.pyplot as plt
+
+    with open(csv_path, newline="") as f:
+        rows = [{k: (v if k == "dtype" else float(v)) for k, v in r.items()} for r in csv.DictReader(f)]
+    os.makedirs(out_dir, exist_ok=True)
+    sizes = sorted({int(r["ndim"]) for r in rows})
+    written = []
+    for key, ylabel, name in (("speedup", "fused / unfused speed-up", "speedup_vs_k.png"),
+                              ("fused_gflops", "TFLOP/s", "tflops_vs_k.png")):
+        fig, ax = plt.subplots(figsize=(7, 4.5))
+        for n in sizes:
+            sub = sorted((r for r in rows if int(r["ndim"]) == n), key=lambda r: r["kdim"])
+            ks = [r["kdim"] for r in sub]
+            if key == "speedup":
+                ax.plot(ks, [r[key] for r in sub], "o-", label=f"N=M={n}")
+            else:
+                ax.plot(ks, [r["fused_gflops"] / 1e3 for r in sub], "o-", label=f"fused N=M={n}")
+                ax.plot(ks, [r["baseline_gflops"] / 1e3 for r in sub], "s--", label=f"unfused N=M={n}")
+        if key == "speedup":
+            ax.axhline(1.0, color="gray", linewidth=0.8)
+        ax.set_xscale("log", base=2)
+        ax.set_xlabel("K")
+        ax.set_ylabel(ylabel)
+        ax.grid(True, alpha=0.3)
+        ax.legend(fontsize=8)
+        path = os.path.join(out_dir, name)
+        fig.tight_layout()
+        fig.savefig(path, dpi=120)
+        plt.close(fig)
+        written.append(path)
+    return written
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="harness")
     sub = ap.add_subparsers(dest="cmd", required=True)
@@ -242,7 +283,14 @@ def main(argv=None) -> int:
     p2.add_argument("--dtype", default="bf16", choices=list(DTYPES))
     p2.add_argument("--runs", type=int, default=8)
     p2.add_argument("--out-prefix", default=None)
+    p3 = sub.add_parser("plot")
+    p3.add_argument("csv")
+    p3.add_argument("--out-dir", default="plots")
     args = ap.parse_args(argv)
+    if args.cmd == "plot":
+        for path in plot_fused(args.csv, args.out_dir):
+            print("wrote", path)
+        return 0
     if not torch.cuda.is_available():
         sys.stderr.write("harness: no GPU visible\n")
         return 2

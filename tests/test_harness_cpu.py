@@ -47,3 +47,23 @@ def test_cli_without_gpu_exits_nonzero(harness):
     if torch.cuda.is_available():
         pytest.skip("GPU present")
     assert harness.main(["fwht", "--check"]) == 2
+
+
+def test_plot_from_sweep_csv(harness, tmp_path):
+    import csv
+    rows = []
+    for k in (256, 1024, 4096):
+        for n in (1024, 4096):
+            rows.append({"kdim": k, "ndim": n, "mdim": n, "dtype": "bfloat16", "baseline_ms": 0.05,
+                         "fused_ms": 0.04, "speedup": 1.25, "fused_gflops": 5e5, "baseline_gflops": 4e5,
+                         "fused_bandwidth_gbps": 100.0, "max_error": 0.1, "max_abs_reference": 30.0})
+    path = tmp_path / "s.csv"
+    with open(path, "w", newline="") as f:
+        w = csv.DictWriter(f, fieldnames=list(rows[0]))
+        w.writeheader()
+        w.writerows(rows)
+    out = harness.plot_fused(str(path), str(tmp_path / "plots"))
+    assert len(out) == 2
+    for p in out:
+        assert (tmp_path / "plots" / p.split("/")[-1]).stat().st_size > 1000
+    assert harness.main(["plot", str(path), "--out-dir", str(tmp_path / "p2")]) == 0
