@@ -67,7 +67,7 @@ fwht_reg_kernel(const void* in, void* out, uint64_t total, uint64_t num_steps, u
 }
 
 // ---- LDS kernel: one workgroup of W = 2^LW wavefronts per row of n = 4096 * W ----------------
-template <class IO, int LW, bool MUL>
+template <class IO, int LW, bool MUL, bool TWO_PHASE>
 __global__ void __launch_bounds__(64 << LW)
 fwht_lds_kernel(const void* in, void* out, uint64_t rows, int exp2, float mult)
 {
@@ -78,7 +78,7 @@ fwht_lds_kernel(const void* in, void* out, uint64_t rows, int exp2, float mult)
 
     TileOperands<typename IO::T16> ops;
     make_tile_operands<typename IO::T16, IO::ESIZE>(12 + LW, ops, exp2);
-    block_fwht_row<IO, LW, MUL>(in, out, row * (8u << LW), total, xch, ops, mult);
+    block_fwht_row<IO, LW, MUL, TWO_PHASE>(in, out, row * (8u << LW), total, xch, ops, mult);
 }
 
 // ---- host dispatch --------------------------------------------------------------------------------
@@ -87,10 +87,16 @@ int launch_reg(const void* in, void* out, uint64_t total, uint64_t num_steps, ui
                OutputScale os, hipStream_t s)
 {
     if (num_steps == 0) return MI_OK;
-    // up to four steps per wavefront once every compute unit has a full set of wavefronts
+    // Up to four steps per wavefront once every compute unit has a full set of wavefronts: the
+    // operand set-up is paid once and the next row's loads overlap the current row's arithmetic.
+    // Beyond the 256 MiB Infinity Cache the transform is DRAM-bound, and there one step per
+    // (short-lived) wavefront measured 2 - 4 % faster: the sweep through memory stays in order.
     uint64_t waves = num_steps;
     const uint64_t resident = 256u * 16u;
-    if (waves > resident) waves = (num_steps + 3u) / 4u > resident ? (num_steps + 3u) / 4u : resident;
+    const uint64_t per_wave = total * (uint64_t)IO::ESIZE > (256ull << 20) ? 1u : 4u;
+    if (waves > resident)
+        waves = (num_steps + per_wave - 1u) / per_wave > resident ? (num_steps + per_wave - 1u) / per_wave
+                                                                  : resident;
     const uint64_t blocks = (waves + 3u) / 4u;
     if (blocks > 0x7fffffffull) return MI_ERR_SHAPE;
     if (os.mult == 1.0f)
@@ -102,14 +108,12 @@ int launch_reg(const void* in, void* out, uint64_t total, uint64_t num_steps, ui
     return launch_status();
 }
 
-template <class IO, int LW>
-int launch_lds(const void* in, void* out, uint64_t rows, OutputScale os, hipStream_t s)
+template <class IO, int LW, bool TWO_PHASE>
+int launch_lds_as(const void* in, void* out, uint64_t rows, OutputScale os, hipStream_t s)
 {
-    if (rows == 0) return MI_OK;
-    if (rows > 0x7fffffffull) return MI_ERR_SHAPE;
-    constexpr size_t lds = sizeof(f32x4) * 64u * 8u * (1u << LW);
+    constexpr size_t lds = sizeof(f32x4) * 64u * (TWO_PHASE ? 8u : 16u) * (1u << LW);
     const bool mul = os.mult != 1.0f;
-    auto kern = mul ? fwht_lds_kernel<IO, LW, true> : fwht_lds_kernel<IO, LW, false>;
+    auto kern = mul ? fwht_lds_kernel<IO, LW, true, TWO_PHASE> : fwht_lds_kernel<IO, LW, false, TWO_PHASE>;
     if (lds > 64u * 1024u) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -118,6 +122,19 @@ int launch_lds(const void* in, void* out, uint64_t rows, OutputScale os, hipStre
     hipLaunchKernelGGL(kern, dim3((uint32_t)rows), dim3(64u << LW), lds, s, in, out, rows, os.exp2,
                        os.mult);
     return launch_status();
+}
+
+template <class IO, int LW>
+int launch_lds(const void* in, void* out, uint64_t rows, OutputScale os, hipStream_t s)
+{
+    if (rows == 0) return MI_OK;
+    if (rows > 0x7fffffffull) return MI_ERR_SHAPE;
+    // While the tensor fits the 256 MiB Infinity Cache, occupancy decides (exchange in two
+    // phases, half the LDS); once it is DRAM-bound, the single exchange with fewer resident
+    // workgroups measured 3 - 5 % faster.
+    const uint64_t bytes = (rows << (12 + LW)) * (uint64_t)IO::ESIZE;
+    if (bytes > (256ull << 20)) return launch_lds_as<IO, LW, false>(in, out, rows, os, s);
+    return launch_lds_as<IO, LW, true>(in, out, rows, os, s);
 }
 
 template <class IO>

@@ -181,8 +181,9 @@ __device__ __forceinline__ void wave_fwht_step(const void* in, void* out, uint64
 // Pass 1: wavefront w transforms elements [4096w, 4096w+4096) (12 bits).  Exchange: every
 // accumulator quad goes to LDS once; wavefront w then gathers, from all W sub-rows, the 8/W tiles
 // it owns, runs the LW remaining butterflies in registers and stores.  `xch` holds
-// 16 * 64 * 8 * W bytes; all 64*W threads must call (__syncthreads inside).
-template <class IO, int LW, bool MUL>
+// 16 * 64 * 8 * W bytes (TWO_PHASE: the two accumulator halves take turns) or twice that (one
+// exchange); all 64*W threads must call (__syncthreads inside).
+template <class IO, int LW, bool MUL, bool TWO_PHASE = true>
 __device__ __forceinline__ void block_fwht_row(const void* in, void* out, uint64_t tile0,
                                                uint64_t total, f32x4* xch,
                                                const TileOperands<typename IO::T16>& ops, float mult)
@@ -191,8 +192,6 @@ __device__ __forceinline__ void block_fwht_row(const void* in, void* out, uint64
     constexpr int OWN = 8 / W;  // tiles per sub-row owned by a wavefront in pass 2
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t w = threadIdx.x >> 6;
-    // xch layout: [W sub-rows][8 tiles][64 lanes], used twice (once per accumulator half), which
-    // halves the LDS footprint and lets two workgroups share a compute unit at W = 8
     f32x4 acc[8][2];
     {
         typename IO::In tin[8];
@@ -203,17 +202,35 @@ __device__ __forceinline__ void block_fwht_row(const void* in, void* out, uint64
         cross_tile_butterflies<8, 3>(acc);
     }
     f32x4 g[W * OWN][2];  // index s * OWN + c'
+    if constexpr (TWO_PHASE) {
+        // xch layout: [W sub-rows][8 tiles][64 lanes], used twice (once per accumulator half):
+        // half the LDS footprint, so two workgroups share a compute unit at W = 8
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        if (t) __syncthreads();  // every wavefront has read the first half
+        for (int t = 0; t < 2; ++t) {
+            if (t) __syncthreads();  // every wavefront has read the first half
 #pragma unroll
-        for (int c = 0; c < 8; ++c) xch[(w * 8u + c) * 64u + lane] = acc[c][t];
+            for (int c = 0; c < 8; ++c) xch[(w * 8u + c) * 64u + lane] = acc[c][t];
+            __syncthreads();
+#pragma unroll
+            for (int s = 0; s < W; ++s)
+#pragma unroll
+                for (int cc = 0; cc < OWN; ++cc)
+                    g[s * OWN + cc][t] = xch[(s * 8u + w * OWN + cc) * 64u + lane];
+        }
+    } else {
+        // xch layout: [W sub-rows][8 tiles][2 halves][64 lanes], one exchange with one barrier
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+#pragma unroll
+            for (int t = 0; t < 2; ++t) xch[((w * 8u + c) * 2u + t) * 64u + lane] = acc[c][t];
         __syncthreads();
 #pragma unroll
         for (int s = 0; s < W; ++s)
 #pragma unroll
             for (int cc = 0; cc < OWN; ++cc)
-                g[s * OWN + cc][t] = xch[(s * 8u + w * OWN + cc) * 64u + lane];
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    g[s * OWN + cc][t] = xch[((s * 8u + w * OWN + cc) * 2u + t) * 64u + lane];
     }
 
     // butterflies over the sub-row index s (element bits 12 .. 12+LW-1)
