@@ -3,7 +3,6 @@
 Tolerances (metric max|y - y64| / max|y64|): fp32 <= 1e-5, bf16/fp16 <= 2e-2 (build contract);
 plus the reference's own absolute bars against the matrix product in the tensor's dtype,
 allclose(atol=1e-2 fp16 / 5e-2 bf16, rtol=0), HadaCore/test.py:91,97."""
-import math
 
 import numpy as np
 import pytest

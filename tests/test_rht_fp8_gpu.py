@@ -4,7 +4,6 @@ The reference has no FP8 path, so parity here is against the oracle's stated con
 codes and scales are bit-exact given identical pre-quant values (the kernel's own bf16 y, which
 is itself checked against the fp64 oracle at the bf16 tolerance and against the stand-alone
 transform bit for bit)."""
-import math
 
 import numpy as np
 import pytest
