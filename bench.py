@@ -168,6 +168,12 @@ def main() -> int:
         if name == "bf16":
             mm_ms, _ = _steady_ms(torch, lambda: torch.matmul(W, Xt.t()), gsteps)
             entry["library_gemm_without_transform_tflops"] = round(flops / mm_ms / 1e9, 1)
+            # the reference's "Baseline (Unfused)" (fusion_pipelined.cu:640-656): transform kernel,
+            # H(X) through HBM, then the vendor GEMM
+            un_ms, _ = _steady_ms(
+                torch, lambda: torch.matmul(W, hada.hadamard_transform(Xt).t()), gsteps)
+            entry["unfused_transform_then_library_gemm_ms"] = round(un_ms, 6)
+            entry["fused_over_unfused_speedup"] = round(un_ms / ms, 3)
             result["fused_ht_gemm"] = entry
             if args.only_gemm:
                 print(json.dumps(entry))
