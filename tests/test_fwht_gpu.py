@@ -214,3 +214,29 @@ def test_runs_on_the_callers_stream(pkg, oracle):
     y64 = oracle.fwht_f64((x_cpu.float() * 2).to(torch.bfloat16).to(torch.float64).numpy())
     assert oracle.rel_err(y.cpu().to(torch.float64).numpy(), y64) <= 2e-2
     assert torch.allclose(z.cpu(), y.float().sum(dim=1).cpu(), rtol=1e-3, atol=1e-2)
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("p", range(1, 16))
+def test_reference_sweep_against_matrix_product(pkg, p, dt):
+    # the reference's own test, HadaCore/test.py:71-97: for every n = 2 .. 32768 and element counts
+    # 2^9 .. 2^25, the in-place op against  a @ (hadamard(n) * n^-1/2).to(dtype)  with
+    # allclose(atol=1e-2 fp16 / 5e-2 bf16, rtol=0).  The matrix is built on the device from
+    # H[i][j] = (-1)^popcount(i & j) (= scipy.linalg.hadamard, pinned on the CPU in test_oracle.py).
+    n = 1 << p
+    idx = torch.arange(n, device="cuda")
+    bits = idx[:, None] & idx[None, :]
+    par = torch.zeros_like(bits)
+    for b in range(p):
+        par ^= (bits >> b) & 1
+    H = ((1.0 - 2.0 * par.float()) * n ** -0.5).to(dt)
+    del bits, par
+    g = torch.Generator(device="cuda").manual_seed(0)
+    for numel in (1 << 9, 1 << 15, 1 << 21, 1 << 25):
+        if numel < n:
+            continue
+        a = torch.randn(numel // n, n, generator=g, device="cuda").to(dt)
+        want = a @ H
+        got = pkg.hadamard_transform(a, inplace=True)
+        assert got.data_ptr() == a.data_ptr()
+        assert torch.allclose(want, got, atol=ATOL_REF[dt], rtol=0), (n, numel, dt)
