@@ -31,7 +31,7 @@ __device__ __forceinline__ uint32_t prow(uint32_t r)
 }
 
 template <int WBITS>
-__device__ __forceinline__ void butterfly_regs(float (&v)[16])
+__device__ __forceinline__ void butterfly_regs(float (&v)[32])
 {
 #pragma unroll
     for (int b = 0; b < WBITS; ++b)
@@ -52,14 +52,14 @@ __device__ __forceinline__ void pass(const float* __restrict__ X, float* tile, u
                                      uint32_t B, uint32_t b0, uint32_t shift, float mul)
 {
     constexpr int R = 1 << WBITS;
-    constexpr int SETS = FROM_GLOBAL ? 4 : 2;
+    constexpr int SETS = (FROM_GLOBAL ? 4 : 2) / (WBITS == 5 ? 2 : 1);
     const uint32_t c = threadIdx.x & 15u, g = threadIdx.x >> 4;
     const uint32_t stride = 1u << shift;
     const uint32_t sets = N >> WBITS;
     const bool col_ok = b0 + c < B;
     constexpr uint32_t G = kThreads / 16;
     for (uint32_t s0 = g; s0 < sets; s0 += G * SETS) {
-        float v[SETS][16];
+        float v[SETS][32];
         uint32_t base[SETS];
 #pragma unroll
         for (int u = 0; u < SETS; ++u) {
@@ -100,7 +100,8 @@ __device__ __forceinline__ void pass_w(int wbits, const float* __restrict__ X, f
         case 1: pass<1, FROM_GLOBAL>(X, tile, N, B, b0, shift, mul); break;
         case 2: pass<2, FROM_GLOBAL>(X, tile, N, B, b0, shift, mul); break;
         case 3: pass<3, FROM_GLOBAL>(X, tile, N, B, b0, shift, mul); break;
-        default: pass<4, FROM_GLOBAL>(X, tile, N, B, b0, shift, mul); break;
+        case 4: pass<4, FROM_GLOBAL>(X, tile, N, B, b0, shift, mul); break;
+        default: pass<5, FROM_GLOBAL>(X, tile, N, B, b0, shift, mul); break;
     }
 }
 
@@ -148,8 +149,10 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
     {
         uint32_t done = 0;
         bool first = true;
+        uint32_t passes_left = (logN + 4u) / 5u;  // fewest radix-32 passes, bits spread evenly
         while (done < logN) {
-            const int wbits = (int)min(4u, logN - done);
+            const int wbits = (int)((logN - done + passes_left - 1u) / passes_left);
+            --passes_left;
             const float mul = (done + wbits == logN) ? scale : 1.0f;
             if (first)
                 pass_w<true>(wbits, X, tile, N, B, b0, done, mul);
