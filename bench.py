@@ -260,13 +260,25 @@ def main() -> int:
         for _ in range(reps):
             xs @ H
         dt_s = (time.perf_counter() - t0) / reps
+        # the C restatement's O(n log n) butterfly on one core, over the whole batch (under a second)
+        bsample = rows
+        xb = x_cpu[:bsample].float().numpy()
+        oracle.fwht_f32(xb[:64])
+        t0 = time.perf_counter()
+        oracle.fwht_f32(xb)
+        bdt = time.perf_counter() - t0
+        butterfly = {"value": round(2 * bsample * n * 2 / bdt / 1e9, 4), "unit": "GB/s", "cores": 1,
+                     "sample": f"oracle_fwht_f32 (plain C butterfly, fp32) on all {bsample} rows; "
+                               "bytes counted at the workload's 2 B per element",
+                     "ms_for_sample": round(bdt * 1e3, 3)}
         result["cpu_baseline"] = {
             "value": round(2 * sample * n * 2 / dt_s / 1e9, 4), "unit": "GB/s", "cores": nthreads,
             "kind": "port",
             "sample": f"torch CPU x @ (hadamard(4096)/64).to(bf16) on the first {sample} of 16384 rows "
                       f"(matrix built once, untimed), mean of {reps} calls; os.cpu_count()={os.cpu_count()}",
             "ms_for_sample": round(dt_s * 1e3, 3),
-            "ms_extrapolated_full_batch": round(dt_s * 1e3 * rows / sample, 1)}
+            "ms_extrapolated_full_batch": round(dt_s * 1e3 * rows / sample, 1),
+            "butterfly_port": butterfly}
 
     print(json.dumps(result))
     return 0
