@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep] [--no-cpu]
 
 A *step* is one pass of the stand-alone transform over one batch: the in-place normalised FWHT of
-a bf16 X[16384, 4096] (BASELINE config 2), inputs resident in HBM before timing starts.  The
+a bf16 X[16384, 4096] (the headline benchmark configuration), inputs resident in HBM before timing starts.  The
 protocol is the reference's (bench/bench.py:112-127): warm-up launches, then K back-to-back
 launches on the same buffer inside one event window on the launch stream.  One JSON line is
 printed; besides the headline it carries

@@ -117,7 +117,7 @@ def test_gemm_reference_self_check_shape(pkg, oracle):
 
 @pytest.mark.parametrize("dt,tol", [(torch.bfloat16, 2e-2), (torch.float32, 1e-5)], ids=["bf16", "f32"])
 def test_gemm_full_size_config(pkg, oracle, dt, tol):
-    # BASELINE config 4: W [4096,1024], Xt [4096,1024], scale 1/32; checked on sampled rows/cols
+    # benchmark configuration 4: W [4096,1024], Xt [4096,1024], scale 1/32; checked on sampled rows/cols
     W, Xt = oracle.inputs_gemm(4096, 4096, 1024, dt)
     C = pkg.fused_ht_gemm(W.cuda(), Xt.cuda(), out_dtype=torch.float32)
     torch.cuda.synchronize()

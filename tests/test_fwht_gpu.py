@@ -155,7 +155,7 @@ def test_errors(pkg):
 
 @pytest.mark.parametrize("dt", DTYPES, ids=str)
 def test_involution_at_full_size(pkg, dt):
-    # BASELINE config 2 shape: [16384, 4096]; the normalised transform is its own inverse and
+    # benchmark configuration 2 shape: [16384, 4096]; the normalised transform is its own inverse and
     # preserves the row norms (size-independent properties, checked on the device)
     g = torch.Generator().manual_seed(0)
     x = torch.randn(16384, 4096, generator=g, dtype=torch.float32).to(dt).cuda()

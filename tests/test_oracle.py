@@ -75,7 +75,7 @@ def test_fp32_port_close_to_fp64(oracle):
 
 
 def test_matrix_truth_path_config1(oracle):
-    # BASELINE config 1: fp32 [512,256], scale 1/16, x @ H in torch on the CPU
+    # benchmark configuration 1: fp32 [512,256], scale 1/16, x @ H in torch on the CPU
     x = oracle.inputs_fwht(512, 256, torch.float32)
     y = oracle.hadamard_matrix_ref(x).numpy()
     assert oracle.rel_err(y, oracle.fwht_f64(x.numpy())) < 1e-5

@@ -50,7 +50,7 @@ def test_quant_zero_row_and_outliers(pkg, oracle):
 
 
 def test_quant_full_size_config(pkg, oracle):
-    # BASELINE config 5 activations [8192, 4096]; property checks on the device + sampled rows
+    # benchmark configuration 5 activations [8192, 4096]; property checks on the device + sampled rows
     x, sign = oracle.inputs_rht(8192, 4096)
     q, rs, y = pkg.rht_quant_fp8(x.cuda(), sign, return_prequant=True)
     torch.cuda.synchronize()
