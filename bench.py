@@ -217,6 +217,13 @@ def main() -> int:
         "roofline": {"bound": "mfma", "achieved": round(fl / ms / 1e9, 1), "peak": PEAK_TFLOPS["fp8"],
                      "unit": "TFLOP/s", "frac": round(fl / ms / 1e9 / PEAK_TFLOPS["fp8"], 4),
                      "traffic": traffic.get("fp8_gemm_8192x14336x4096_l2_fill_plus_write")}}
+    try:  # the vendor library's row-scaled FP8 GEMM on the same operands, for comparison only
+        lib_ms, _ = _steady_ms(torch, lambda: torch._scaled_mm(
+            qx, qw.t(), scale_a=sx.view(-1, 1), scale_b=sw.view(1, -1), out_dtype=torch.bfloat16), 20)
+        others["fp8_gemm_8192x14336x4096"]["library_scaled_mm_rowwise_us"] = round(lib_ms * 1e3, 1)
+        others["fp8_gemm_8192x14336x4096"]["library_scaled_mm_rowwise_tflops"] = round(fl / lib_ms / 1e9, 1)
+    except Exception as ex:  # not every torch build exposes it
+        others["fp8_gemm_8192x14336x4096"]["library_scaled_mm_rowwise_us"] = f"unavailable: {str(ex)[:80]}"
     del xa, w, qx, qw
     if args.only_rht:
         print(json.dumps(others))
