@@ -6,13 +6,14 @@ Two sub-commands (run from the repository root)::
     python -m 6s894_project_2025_amd.harness fused [--dtype bf16|f32] [--runs 8] [--out-prefix P]
     python -m 6s894_project_2025_amd.harness plot P.csv [--out-dir plots]
 
-``fwht`` keeps the structure of the reference's bench/bench.py: a registry of in-place cases
-(three AddOne roofline proxies around the transform, :96-103), a correctness pass of every case
-against its ``call_ref`` with ``allclose(atol=1e-2 fp16 / 5e-2 bf16, rtol=0)`` (:159-203), the
-timing protocol "3 warm-up calls, then N back-to-back calls on the same buffer inside one event
-window" (:112-127), and a JSON dump with the same fields (:226-237, :291-300).  The reference
-checks its own kernel against HadaCore; here ``call_ref`` is the matrix truth path
-``t @ (hadamard(n) * n**-0.5)`` evaluated with torch on the GPU (bench/bench.py:49-59).
+``fwht`` follows the protocol of the reference's bench/bench.py: a registry of in-place cases
+(add-one roofline proxies around the transform, :96-103), a correctness pass of every case with
+``allclose(atol=1e-2 fp16 / 5e-2 bf16, rtol=0)`` (:159-203), timing as "3 warm-up calls, then N
+back-to-back calls on the same buffer inside one event window" (:112-127), and a JSON dump with
+the same fields (:226-237, :291-300).  The reference checks its own kernel against HadaCore; here
+the truth is the matrix path ``t @ (hadamard(n) * n**-0.5)`` evaluated with torch on the GPU
+(bench/bench.py:49-59).  The check runs each case on the full-size buffer, because the launcher
+picks its kernel variant by tensor size, and compares row slices of the result.
 
 ``fused`` covers the 15 (K, N, M) shapes of fused_ht/benchmark_sweep.py:20-45 with its FLOP and
 byte models (:123-140), but with run-time shapes (no regex edit + recompile), and times the
@@ -36,66 +37,45 @@ from typing import Any, Callable
 import torch
 
 from .ops import fused_ht_gemm, hadamard_transform
+from .timing import best_single_call_ms, event_window_ms
 
 ATOL = {torch.float16: 1e-2, torch.bfloat16: 5e-2, torch.float32: 1e-4}
 DTYPES = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}
 
 
-def get_scale(size: int) -> float:
-    return math.sqrt(1.0 / size)
-
-
 @functools.lru_cache(maxsize=None)
-def _hadamard_cache(size: int) -> torch.Tensor:
-    """Sylvester matrix times n**-0.5 on the GPU, H[i][j] = (-1)**popcount(i & j)."""
-    idx = torch.arange(size, device="cuda")
+def _normalised_sylvester(n: int) -> torch.Tensor:
+    """H_n / sqrt(n) on the GPU in fp32, H[i][j] = (-1)**popcount(i & j)."""
+    idx = torch.arange(n, device="cuda")
     bits = idx[:, None] & idx[None, :]
-    par = torch.zeros_like(bits)
-    for b in range(max(1, size.bit_length())):
-        par ^= (bits >> b) & 1
-    return (1.0 - 2.0 * par.to(torch.float32)) * get_scale(size)
+    parity = torch.zeros_like(bits)
+    for b in range(max(1, n.bit_length())):
+        parity ^= (bits >> b) & 1
+    return (1.0 - 2.0 * parity.to(torch.float32)) / math.sqrt(n)
 
 
-def hadamard_ref(t: torch.Tensor) -> None:
-    m = int(t.shape[-1])
-    t.copy_(t @ _hadamard_cache(m).to(t.dtype))
+@dataclass(frozen=True)
+class Case:
+    """One in-place benchmark case: ``run`` is what gets timed, ``truth`` returns what ``run``
+    must leave in a buffer that held ``t``.  The registry below keeps the reference's order
+    (bench/bench.py:96-103): add-one roofline proxies before and after the transform."""
+    run: Callable[[torch.Tensor], Any]
+    truth: Callable[[torch.Tensor], torch.Tensor]
 
 
-class AddOne:
-    """In-place add: the achieved-bandwidth proxy (bench/bench.py:88-93)."""
-
-    def call(self, t: torch.Tensor) -> None:
-        t.add_(1)
-
-    def call_ref(self, t: torch.Tensor) -> None:
-        t.add_(1)
+def _matrix_truth(t: torch.Tensor) -> torch.Tensor:
+    # the reference's definition of correct: t @ (hadamard(n) * n**-0.5) in t's dtype
+    # (HadaCore/test.py:27,40; bench/bench.py:49-59)
+    return t @ _normalised_sylvester(int(t.shape[-1])).to(t.dtype)
 
 
-class Ours:
-    def call(self, t: torch.Tensor) -> None:
-        hadamard_transform(t, inplace=True)
-
-    def call_ref(self, t: torch.Tensor) -> None:
-        hadamard_ref(t)
-
-
-CASES: dict[str, Any] = {"AddOne1": AddOne(), "AddOne2": AddOne(), "Ours": Ours(), "AddOne3": AddOne()}
-
-
-def _bench_many(fn: Callable[[], None], iters: int, warmup: int = 3) -> dict[str, float]:
-    torch.cuda.synchronize()
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()
-    start = torch.cuda.Event(enable_timing=True)
-    end = torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(iters):
-        fn()
-    end.record()
-    end.synchronize()
-    total_ms = float(start.elapsed_time(end))
-    return {"total_ms": total_ms, "per_iter_ms": total_ms / max(iters, 1)}
+_ADD_ONE = Case(run=lambda t: t.add_(1), truth=lambda t: t + 1)
+CASES: dict[str, Case] = {
+    "AddOne1": _ADD_ONE,
+    "AddOne2": _ADD_ONE,
+    "Ours": Case(run=lambda t: hadamard_transform(t, inplace=True), truth=_matrix_truth),
+    "AddOne3": _ADD_ONE,
+}
 
 
 @dataclass
@@ -109,6 +89,24 @@ class TestConfig:
     dtypes: tuple[torch.dtype, ...] = (torch.float16, torch.bfloat16)
 
 
+def _check_case(name: str, case: Case, full: torch.Tensor) -> None:
+    """Runs the case on the *full-size* buffer (so the launch path that gets timed is the one that
+    gets checked) and compares bounded row slices of the result with the truth path, which costs
+    O(rows * n^2) and is therefore evaluated on slices only.  Restores the buffer afterwards."""
+    rows, n = full.shape
+    take = min(rows, max(1, (1 << 21) // n))
+    starts = sorted({0, max(0, rows // 2 - take // 2), rows - take})
+    before = [full[s:s + take].clone() for s in starts]
+    case.run(full)
+    for s, src in zip(starts, before):
+        got, want = full[s:s + take], case.truth(src)
+        if not torch.allclose(want, got, atol=ATOL.get(full.dtype, 1e-2), rtol=0):
+            worst = (want.float() - got.float()).abs().max().item()
+            print(f"Failed test: {name} {n}x{rows} {full.dtype} rows {s}..{s + take}; max diff {worst}")
+            raise SystemExit(1)
+        got.copy_(src)
+
+
 def run_fwht(cfg: TestConfig) -> list[dict[str, Any]]:
     print("test_sizes_m: ", cfg.test_sizes)
     print("test_elem_counts: ", cfg.elem_counts)
@@ -119,39 +117,29 @@ def run_fwht(cfg: TestConfig) -> list[dict[str, Any]]:
     results: list[dict[str, Any]] = []
     for m in cfg.test_sizes:
         for elem_c in cfg.elem_counts:
-            n = elem_c // m
             if elem_c < m:
                 continue
-            print(f"Testing size {m}x{n}")
-            a = torch.randn((n, m), device="cuda", dtype=torch.float32)
-            for case_name in cfg.benchmark_cases:
-                target = CASES[case_name]
-                # correctness on a bounded slice (the matrix truth path is O(rows * m^2))
-                rows_chk = min(n, max(1, (1 << 22) // m))
-                for dtype in cfg.dtypes:
-                    got = a[:rows_chk].clone().to(dtype)
-                    want = a[:rows_chk].clone().to(dtype)
-                    target.call(got)
-                    target.call_ref(want)
-                    if not torch.allclose(want, got, atol=ATOL.get(dtype, 1e-2), rtol=0):
-                        diff = (want.float() - got.float()).abs()
-                        print(f"Failed test: {case_name} {m}x{n} {dtype}; max diff {diff.max().item()}")
-                        raise SystemExit(1)
-                if cfg.check:
-                    continue
-                for dtype in cfg.dtypes:
-                    a_run = a.to(dtype).contiguous()
-                    stats = _bench_many(lambda: target.call(a_run), cfg.runs_per_size)
-                    gbs = 2 * a_run.numel() * a_run.element_size() / stats["per_iter_ms"] / 1e6
-                    print(f"{case_name} m={m} n={n} {str(dtype).replace('torch.', '')} | "
-                          f"{stats['per_iter_ms']:.4f} ms/iter over {cfg.runs_per_size} iters "
-                          f"({gbs:.0f} GB/s)")
-                    results.append({"device": device_name, "case": case_name, "m": m, "n": n,
-                                    "dtype": str(dtype).replace("torch.", ""),
-                                    "runs": cfg.runs_per_size, "per_iter_ms": stats["per_iter_ms"],
-                                    "total_ms": stats["total_ms"], "GB/s": gbs})
-                    del a_run
-            del a
+            rows = elem_c // m
+            print(f"Testing size {m}x{rows}")
+            base = torch.randn((rows, m), device="cuda", dtype=torch.float32)
+            for dtype in cfg.dtypes:
+                buf = base.to(dtype).contiguous()
+                dname = str(dtype).replace("torch.", "")
+                for name in cfg.benchmark_cases:
+                    case = CASES[name]
+                    _check_case(name, case, buf)
+                    if cfg.check:
+                        continue
+                    ms, _ = event_window_ms(lambda: case.run(buf), cfg.runs_per_size)
+                    gbs = 2 * buf.numel() * buf.element_size() / ms / 1e6
+                    print(f"{name} m={m} n={rows} {dname} | {ms:.4f} ms/iter over "
+                          f"{cfg.runs_per_size} iters ({gbs:.0f} GB/s)")
+                    results.append({"device": device_name, "case": name, "m": m, "n": rows,
+                                    "dtype": dname, "runs": cfg.runs_per_size, "per_iter_ms": ms,
+                                    "total_ms": ms * cfg.runs_per_size, "GB/s": gbs})
+                    buf.copy_(base)  # add-one and repeated transforms drift; start each case alike
+                del buf
+            del base
     if not cfg.check and cfg.json_output_file:
         with open(cfg.json_output_file, "w") as f:
             json.dump({"device": device_name, "cases": cfg.benchmark_cases,
@@ -164,29 +152,14 @@ def run_fwht(cfg: TestConfig) -> list[dict[str, Any]]:
 FUSED_CONFIGS = [(k, s, s) for k in (256, 512, 1024, 2048, 4096) for s in (1024, 2048, 4096)]
 
 
-def compute_metrics(kdim: int, ndim: int, mdim: int, time_ms: float, esize: int = 4):
-    """GFLOPS and GB/s under the reference's model (benchmark_sweep.py:123-140)."""
-    ht_flops = kdim * (kdim.bit_length() - 1) * ndim * 2
-    gemm_flops = 2 * mdim * ndim * kdim
-    gflops = (ht_flops + gemm_flops) / 1e9 / (time_ms / 1e3)
-    bytes_rw = (kdim * ndim + mdim * kdim + mdim * ndim) * esize
-    return gflops, bytes_rw / 1e9 / (time_ms / 1e3)
-
-
-def _min_time_ms(fn: Callable[[], None], runs: int, warmup: int = 2) -> float:
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()
-    best = float("inf")
-    for _ in range(runs):
-        s = torch.cuda.Event(enable_timing=True)
-        e = torch.cuda.Event(enable_timing=True)
-        s.record()
-        fn()
-        e.record()
-        e.synchronize()
-        best = min(best, float(s.elapsed_time(e)))
-    return best
+def sweep_metrics(K: int, N: int, M: int, ms: float, esize: int = 4) -> tuple[float, float]:
+    """(GFLOP/s, GB/s) of one (K, N, M) shape under the reference's accounting
+    (fused_ht/benchmark_sweep.py:123-140): two flops per butterfly output and per multiply-add,
+    each of X, W and C moved once."""
+    seconds = ms / 1e3
+    flops = 2 * K * (K.bit_length() - 1) * N + 2 * M * N * K
+    moved = esize * (K * N + M * K + M * N)
+    return flops / 1e9 / seconds, moved / 1e9 / seconds
 
 
 def run_fused(dtype: torch.dtype, runs: int = 8, configs=None, out_prefix: str | None = None):
@@ -201,13 +174,13 @@ def run_fused(dtype: torch.dtype, runs: int = 8, configs=None, out_prefix: str |
         scale = 1.0 / math.sqrt(K)
         fused = lambda: fused_ht_gemm(W, Xt, scale)
         unfused = lambda: torch.matmul(W, hadamard_transform(Xt, scale).t())
-        t_f = _min_time_ms(fused, runs)
-        t_u = _min_time_ms(unfused, runs)
+        t_f = best_single_call_ms(fused, runs)
+        t_u = best_single_call_ms(unfused, runs)
         diff = (fused().float() - unfused().float()).abs().max().item()
         ref_scale = unfused().float().abs().max().item()
         esize = W.element_size()
-        gf, bw = compute_metrics(K, N, M, t_f, esize)
-        gu, _ = compute_metrics(K, N, M, t_u, esize)
+        gf, bw = sweep_metrics(K, N, M, t_f, esize)
+        gu, _ = sweep_metrics(K, N, M, t_u, esize)
         print(f"K={K:5d} N={N:5d} M={M:5d} {str(dtype).replace('torch.', ''):9s} "
               f"unfused {t_u * 1e3:9.1f} us ({gu / 1e3:7.1f} TFLOP/s)  fused {t_f * 1e3:9.1f} us "
               f"({gf / 1e3:7.1f} TFLOP/s)  speedup {t_u / t_f:5.2f}x  max|diff| {diff:.3e} "

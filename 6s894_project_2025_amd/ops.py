@@ -15,6 +15,9 @@ from . import _lib
 
 _DTYPE_CODE = {torch.float32: _lib.MI_F32, torch.bfloat16: _lib.MI_BF16, torch.float16: _lib.MI_F16}
 MAX_LOG_N = 15
+# ranges of the C ABI (include/mi_hadamard.h); the wrappers reject the same values it does
+GEMV_MAX_N = 2048
+GEMM_MIN_K, GEMM_MAX_K = 32, 4096
 
 
 def _is_pow2(n: int) -> bool:
@@ -94,8 +97,8 @@ def fused_ht_gemv(W: torch.Tensor, X: torch.Tensor, scale: float | None = None) 
         raise RuntimeError(f"shape mismatch: W {tuple(W.shape)} X {tuple(X.shape)}")
     M, N = W.shape
     B = X.size(1)
-    if not _is_pow2(N) or N < 2 or N > 4096:
-        raise RuntimeError(f"N must be a power of two in [2, 4096], got {N}")
+    if not _is_pow2(N) or N < 2 or N > GEMV_MAX_N:
+        raise RuntimeError(f"N must be a power of two in [2, {GEMV_MAX_N}], got {N}")
     s = 1.0 / math.sqrt(N) if scale is None else float(scale)
     Y = torch.empty((M, B), dtype=torch.float32, device=W.device)
     if M == 0 or B == 0:
@@ -125,8 +128,8 @@ def fused_ht_gemm(W: torch.Tensor, Xt: torch.Tensor, scale: float | None = None,
         raise RuntimeError(f"shape mismatch: W {tuple(W.shape)} Xt {tuple(Xt.shape)}")
     M, K = W.shape
     N = Xt.size(0)
-    if not _is_pow2(K) or K < 16 or K > 4096:
-        raise RuntimeError(f"K must be a power of two in [16, 4096], got {K}")
+    if not _is_pow2(K) or K < GEMM_MIN_K or K > GEMM_MAX_K:
+        raise RuntimeError(f"K must be a power of two in [{GEMM_MIN_K}, {GEMM_MAX_K}], got {K}")
     od = W.dtype if out_dtype is None else out_dtype
     if od not in (torch.float32, W.dtype):
         raise RuntimeError("out_dtype must be fp32 or the input dtype")
@@ -184,17 +187,24 @@ def fp8_gemm_rowscale(qa: torch.Tensor, sa: torch.Tensor, qb: torch.Tensor, sb: 
     _require_cuda(qb, "qb")
     if qa.dim() != 2 or qb.dim() != 2 or qa.size(1) != qb.size(1):
         raise RuntimeError("shape mismatch")
+    if qa.element_size() != 1 or qb.element_size() != 1:
+        raise RuntimeError(f"qa and qb must hold one-byte E4M3FN codes (got {qa.dtype}, {qb.dtype})")
+    if qb.device != qa.device:
+        raise RuntimeError("qa and qb must be on the same device")
     T, K = qa.shape
     N = qb.size(0)
     if K % 128 != 0:
         raise RuntimeError("K must be a multiple of 128")
+    if sa.numel() != T or sb.numel() != N:
+        raise RuntimeError(f"scale lengths {sa.numel()}, {sb.numel()} do not match T={T}, N={N}")
     out = torch.empty((T, N), dtype=torch.bfloat16, device=qa.device)
     if T == 0 or N == 0:
         return out
     a = _dense16(qa.view(torch.uint8))
     b = _dense16(qb.view(torch.uint8))
-    sa = sa.to(torch.float32).contiguous()
-    sb = sb.to(torch.float32).contiguous()
+    # the kernel dereferences the scales on the device: bring them there like `sign` above
+    sa = sa.to(device=qa.device, dtype=torch.float32).contiguous().view(-1)
+    sb = sb.to(device=qa.device, dtype=torch.float32).contiguous().view(-1)
     lib = _lib.load()
     with torch.cuda.device(qa.device):
         st = lib.mi_fp8_gemm_rowscale(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(),

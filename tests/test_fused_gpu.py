@@ -45,6 +45,32 @@ def test_gemv_reference_self_check(pkg, oracle, M, N, B):
     assert np.abs(fused.cpu().double().numpy() - want).max() < 1e-3
 
 
+# Launch paths that only larger problems reach: the 64-row workgroup variant (column groups x
+# 64-row blocks >= 256; the benchmark's M=N=1024 with B=256 and B=512, the shapes of
+# fused_ht/fwht_gemv_fusion.cu:643-653) and a workgroup that walks several row blocks with one
+# transformed tile (more row blocks than workgroup rows in the grid).
+@pytest.mark.parametrize("M,N,B", [(1024, 1024, 256), (1024, 1024, 512), (1024, 1024, 128),
+                                   (4096, 256, 4096), (2000, 64, 1000), (4100, 2048, 130)])
+def test_gemv_large_launch_paths(pkg, oracle, M, N, B):
+    W, X = oracle.inputs_gemv(M, N, B)
+    Y = pkg.fused_ht_gemv(W.cuda(), X.cuda())
+    torch.cuda.synchronize()
+    assert Y.shape == (M, B)
+    # every row block boundary of the 64-row variant, first/last rows, and a random sample
+    g = torch.Generator().manual_seed(7)
+    rows = torch.unique(torch.cat([torch.tensor([0, 1, 63, 64, 65, 127, 128, M // 2, M - 65, M - 64,
+                                                 M - 2, M - 1]).clamp(0, M - 1),
+                                   torch.randint(0, M, (52,), generator=g)]))
+    want = oracle.fused_ht_gemv_f64_blas(W[rows].double().numpy(), X.double().numpy(),
+                                         1.0 / math.sqrt(N))
+    assert _rel(oracle, Y[rows.cuda()], want) <= 1e-5, (M, N, B)
+    # size-independent: column sums of Y equal (column sums of W) . H(X)
+    colsum = oracle.fused_ht_gemv_f64_blas(W.double().sum(0, keepdim=True).numpy(),
+                                           X.double().numpy(), 1.0 / math.sqrt(N))
+    got = Y.double().sum(0, keepdim=True).cpu().numpy()
+    assert np.abs(got - colsum).max() / np.abs(colsum).max() <= 1e-5
+
+
 def test_gemv_identity_reduces_to_transform(pkg, oracle):
     N, B = 256, 48
     _, X = oracle.inputs_gemv(N, N, B)
@@ -124,6 +150,27 @@ def test_gemm_full_size_config(pkg, oracle, dt, tol):
     rows = torch.tensor([0, 1, 63, 64, 511, 512, 2047, 2048, 4095])
     want = oracle.fused_ht_gemm_f64_blas(W[rows].double().numpy(), Xt.double().numpy(), 1.0 / 32.0)
     assert oracle.rel_err(C[rows.cuda()].cpu().double().numpy(), want) <= tol
+
+
+def test_fused_size_limits_match_the_c_abi(pkg, oracle):
+    # boundary values of the documented ranges: GEMV N in [2, 2048], GEMM K in [32, 4096]
+    for N in (2, 2048):
+        W, X = oracle.inputs_gemv(8, N, 5)
+        Y = pkg.fused_ht_gemv(W.cuda(), X.cuda())
+        want = oracle.fused_ht_gemv_f64_blas(W.double().numpy(), X.double().numpy(), N ** -0.5)
+        assert _rel(oracle, Y, want) <= 1e-5
+    for N in (1, 4096):
+        with pytest.raises(RuntimeError, match="power of two in"):
+            pkg.fused_ht_gemv(torch.zeros(8, N, device="cuda"), torch.zeros(N, 5, device="cuda"))
+    for K in (32, 4096):
+        W, Xt = oracle.inputs_gemm(8, 5, K, torch.bfloat16)
+        C = pkg.fused_ht_gemm(W.cuda(), Xt.cuda(), out_dtype=torch.float32)
+        want = oracle.fused_ht_gemm_f64_blas(W.double().numpy(), Xt.double().numpy(), K ** -0.5)
+        assert _rel(oracle, C, want) <= 2e-2
+    for K in (16, 8192):
+        with pytest.raises(RuntimeError, match="power of two in"):
+            pkg.fused_ht_gemm(torch.zeros(8, K, device="cuda", dtype=torch.bfloat16),
+                              torch.zeros(5, K, device="cuda", dtype=torch.bfloat16))
 
 
 def test_fused_errors(pkg):

@@ -20,14 +20,14 @@ def test_fused_shape_list(harness):
     assert [k for k, _, _ in cfgs] == sorted(k for k, _, _ in cfgs)
 
 
-def test_compute_metrics_known_values(harness):
+def test_sweep_metrics_known_values(harness):
     # K=1024, N=M=4096, 1 ms: transform 1024*10*4096*2 flops + GEMM 2*4096*4096*1024 flops;
     # bytes (K*N + M*K + M*N) * 4.  Numbers written out by hand, not recomputed from the formula.
-    gflops, gbps = harness.compute_metrics(1024, 4096, 4096, 1.0)
+    gflops, gbps = harness.sweep_metrics(1024, 4096, 4096, 1.0)
     assert gflops == pytest.approx((83_886_080 + 34_359_738_368) / 1e9 / 1e-3)
     assert gbps == pytest.approx(100_663_296 / 1e9 / 1e-3)
     # halving the time doubles both; 2-byte elements halve the bytes only
-    g2, b2 = harness.compute_metrics(1024, 4096, 4096, 0.5, esize=2)
+    g2, b2 = harness.sweep_metrics(1024, 4096, 4096, 0.5, esize=2)
     assert g2 == pytest.approx(2 * gflops) and b2 == pytest.approx(gbps)
 
 
@@ -39,7 +39,8 @@ def test_case_registry_and_tolerances(harness):
     assert cfg.test_sizes == [256, 512, 1024, 2048, 4096, 8192, 16384, 32768]
     assert cfg.elem_counts == [1 << 30]
     t = torch.zeros(4, 8)
-    harness.CASES["AddOne1"].call(t)
+    assert torch.equal(harness.CASES["AddOne1"].truth(t), torch.ones(4, 8))
+    harness.CASES["AddOne1"].run(t)
     assert torch.equal(t, torch.ones(4, 8))
 
 

@@ -21,20 +21,32 @@ def test_check_mode_all_cases(harness):
 
 
 def test_check_mode_detects_a_wrong_case(harness):
-    class Wrong:
-        def call(self, t):
-            t.add_(1)
-
-        def call_ref(self, t):
-            t.add_(2)
-
-    harness.CASES["Wrong"] = Wrong()
+    harness.CASES["Wrong"] = harness.Case(run=lambda t: t.add_(1), truth=lambda t: t + 2)
     try:
         with pytest.raises(SystemExit):
             harness.run_fwht(harness.TestConfig(check=True, benchmark_cases=["Wrong"],
                                                 test_sizes=[256], elem_counts=[1 << 16]))
     finally:
         del harness.CASES["Wrong"]
+
+
+def test_check_mode_runs_the_full_size_buffer(harness, pkg, monkeypatch):
+    # the transform must be called on the whole buffer (the launch path that is timed is chosen by
+    # tensor size), not on a cloned slice
+    seen = []
+    real = harness.hadamard_transform
+
+    def spy(t, *a, **k):
+        seen.append(tuple(t.shape))
+        return real(t, *a, **k)
+
+    monkeypatch.setattr(harness, "hadamard_transform", spy)
+    monkeypatch.setitem(harness.CASES, "Ours",
+                        harness.Case(run=lambda t: spy(t, inplace=True), truth=harness.CASES["Ours"].truth))
+    cfg = harness.TestConfig(check=True, benchmark_cases=["Ours"], test_sizes=[8192],
+                             elem_counts=[1 << 24], dtypes=(torch.bfloat16,))
+    assert harness.run_fwht(cfg) == []
+    assert seen == [(2048, 8192)]
 
 
 def test_timed_run_json(harness, tmp_path):

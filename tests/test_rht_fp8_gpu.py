@@ -121,3 +121,20 @@ def test_rht_fp8_linear_end_to_end(pkg, oracle):
     want = x.double() @ w.double().t()
     err = (out.cpu().double() - want).abs().max().item() / want.abs().max().item()
     assert err < 0.1
+
+
+def test_fp8_gemm_wrapper_validates_operands(pkg):
+    qa = torch.zeros(16, 128, dtype=torch.uint8, device="cuda")
+    qb = torch.zeros(24, 128, dtype=torch.uint8, device="cuda")
+    sa = torch.ones(16, device="cuda")
+    sb = torch.ones(24, device="cuda")
+    with pytest.raises(RuntimeError, match="scale lengths"):
+        pkg.fp8_gemm_rowscale(qa, sa[:15], qb, sb)
+    with pytest.raises(RuntimeError, match="scale lengths"):
+        pkg.fp8_gemm_rowscale(qa, sa, qb, sb[:1])
+    with pytest.raises(RuntimeError, match="one-byte"):
+        pkg.fp8_gemm_rowscale(qa.to(torch.int16), sa, qb, sb)
+    # scales handed over on the host are moved to the device, not dereferenced there
+    out = pkg.fp8_gemm_rowscale(qa, sa.cpu(), qb, sb.cpu().view(1, -1))
+    torch.cuda.synchronize()
+    assert out.shape == (16, 24) and out.abs().max().item() == 0.0
