@@ -33,6 +33,8 @@ HIPCC_FLAGS = [
 PER_FILE_FLAGS = {
     "fwht.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "rht_fp8.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    # the prologue's MFMA results feed VALU conversions; the main loop's MFMAs are inline assembly
+    "fused_gemm_xreg.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
 }
 
 

@@ -24,6 +24,7 @@ constexpr int kWave = 64;
 // 16-bit storage types the matrix cores take directly.  `E` is the element type, `V8`/`V4` the
 // 8- and 4-wide MFMA operand vectors.
 struct BF16 {
+    static constexpr int kCode = MI_BF16;
     using E = __bf16;
     using V8 = bf16x8;
     using V4 = bf16x4;
@@ -39,6 +40,7 @@ struct BF16 {
 };
 
 struct F16 {
+    static constexpr int kCode = MI_F16;
     using E = _Float16;
     using V8 = f16x8;
     using V4 = f16x4;

@@ -1,6 +1,10 @@
 // Fused Hadamard -> GEMM (mi_fused_ht_gemm), gfx950:  C[M,N] = W[M,K] * (scale * H_K * X[K,N]),
 // X given as Xt[N,K].  The transformed operand lives only in LDS.
 //
+// This file: the dispatcher and the LDS-resident variant, used for K = 32 .. 512, 2048 and 4096.
+// K = 1024 goes to the register-resident variant in fused_gemm_xreg.hip, which holds twice as many
+// columns per compute unit.
+//
 // Structure ("X-stationary"): a workgroup owns BN columns of X for the whole K extent.
 //   prologue : its wavefronts transform those BN rows of Xt on the matrix cores (tile_transform,
 //              the stand-alone kernel's building block), round to the 16-bit type and park
@@ -26,6 +30,11 @@
 #include "fwht_device.hpp"
 
 namespace mi {
+
+// K = 1024 with the transformed operand in registers: fused_gemm_xreg.hip
+int fused_gemm16_xreg(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, int in_dtype,
+                      int out_f32, float scale, hipStream_t s);
+
 namespace {
 
 constexpr int kGemmThreads = 512;
@@ -405,7 +414,7 @@ int dispatch_gemm16(const void* W, const void* Xt, void* C, uint32_t M, uint32_t
         case 128:
         case 256:
         case 512: return launch_gemm16<T16, 64, 0, 0>(W, Xt, C, M, N, K, out_f32, scale, s);
-        case 1024: return launch_gemm16<T16, 64, 1, 1024>(W, Xt, C, M, N, K, out_f32, scale, s);
+        case 1024: return fused_gemm16_xreg(W, Xt, C, M, N, T16::kCode, out_f32, scale, s);
         case 2048: return launch_gemm16<T16, 32, 2, 0>(W, Xt, C, M, N, K, out_f32, scale, s);
         case 4096: return launch_gemm16<T16, 16, 3, 0>(W, Xt, C, M, N, K, out_f32, scale, s);
         default: return MI_ERR_SIZE;

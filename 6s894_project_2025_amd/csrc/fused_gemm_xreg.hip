@@ -1,0 +1,547 @@
+// Fused Hadamard -> GEMM with the transformed operand held in registers, gfx950, 16-bit inputs:
+//     C[M,N] = W[M,K] * (scale * H_K * X[K,N]),  X given as Xt[N,K],  K = 1024.
+//
+// One workgroup = four wavefronts, one per SIMD, each with the whole 512-register budget.
+//   prologue : wavefront w transforms 32 columns of X on the matrix cores (coalesced 16-byte
+//              loads, the two-stage tile transform of fwht_device.hpp with the last butterfly
+//              folded into the second stage), passes them once through a wavefront-private LDS
+//              area to get from "a lane owns 8 consecutive k of one column" to MFMA operand order
+//              "lane (hi, lo) owns 8 consecutive k of column lo", and keeps all K x 32 values in
+//              the 256 accumulation registers for the rest of the kernel.  The workgroup
+//              therefore owns 128 columns, twice what fits in LDS.
+//   main loop: the workgroup walks its M range in 64-row blocks.  W is the only operand that
+//              moves: global -> LDS directly (no register hop), each wavefront fetching a quarter
+//              of a 64-row x 256-K stage as whole 512-byte row segments into a ring of four
+//              stage buffers, three stages ahead; every wavefront then reads all of it back as
+//              MFMA A fragments (LDS is the broadcast medium: a W fragment serves the four
+//              wavefronts' different columns).  One workgroup barrier per stage, placed after
+//              the stage's last fragment read has been issued, so the first fragments of the next
+//              stage are read behind the stage's last sixteen MFMAs.  With one wavefront per SIMD
+//              nothing hides an instruction that waits, so every memory instruction is issued in
+//              the shadow of a running MFMA.
+//   epilogue : D[row 4*hi + r][column lo] of the two column fragments is packed into pairs of
+//              adjacent columns and stored straight from registers, two stores per K step of the
+//              *next* row block (two accumulator sets take turns).
+// Per compute unit the kernel reads 128 columns of X once and a 1/msplit share of W once; the
+// register file, not LDS, decides how many columns a compute unit can keep.
+//
+// Behaviour replaced: fused_ht_gemm_pipelined, fused_ht/fusion_pipelined.cu:306-563; its
+// "Load(t+1) || GEMM(t)" pipeline with asynchronous 16-byte copies (:247-268, :468-543) is the W
+// stream here.
+#include <type_traits>
+
+#include "fwht_device.hpp"
+
+namespace mi {
+namespace xreg {
+
+constexpr int kThreads = 256;
+constexpr int kCols = 128;                        // columns of X per workgroup
+constexpr int kRows = 64;                         // rows of W per row block
+constexpr int kStageK = 256;                      // K extent of one W stage
+constexpr int kStageBytes = kRows * kStageK * 2;  // 32 KB
+constexpr int kSlots = 4;                         // ring of stage buffers
+constexpr int kStepsPerStage = kStageK / 32;      // 8 MFMA K steps
+constexpr int kAreaBytes = 16 * 512 * 2;          // per wavefront: 16 columns x 512 k
+// stage buffers 0..3 at [0, 128K); the wavefront areas of the prologue at [96K, 160K), i.e.
+// on top of stage buffer 3, which is first filled after the prologue
+constexpr int kAreaBase = 3 * kStageBytes;
+constexpr int kLdsBytes = kAreaBase + 4 * kAreaBytes;
+
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+// acc (+)= A(16 x 32) * B(32 x 16) with B read straight from the accumulation-register file, where
+// the transformed operand lives for the whole kernel, and the accumulator in ordinary registers.
+// Inline assembly because the compiler, left to itself, copies register-file-resident operands
+// into ordinary registers before every use (v_accvgpr_read, four per fragment), and those copies
+// wait for the matrix-core pipeline.  What the compiler no longer sees: the result is written when
+// the instruction retires, not when it issues; readers of `c` other than the next accumulate must
+// come at least one more MFMA (or drain_mfma()) later.
+template <class T16>
+struct XMfma;
+template <>
+struct XMfma<BF16> {
+    static __device__ __forceinline__ void first(f32x4& c, bf16x8 a, bf16x8 b)
+    {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "a"(b));
+    }
+    static __device__ __forceinline__ void next(f32x4& c, bf16x8 a, bf16x8 b)
+    {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+    }
+};
+template <>
+struct XMfma<F16> {
+    static __device__ __forceinline__ void first(f32x4& c, f16x8 a, f16x8 b)
+    {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "a"(b));
+    }
+    static __device__ __forceinline__ void next(f32x4& c, f16x8 a, f16x8 b)
+    {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+    }
+};
+
+// Waits out the matrix-core pipeline before `acc` is read by anything but an MFMA.  The
+// accumulators pass through the statement, so that the compiler cannot move a read of them (a
+// register copy, say) above the wait.
+__device__ __forceinline__ void drain_mfma(f32x4 (&acc)[4][2])
+{
+    asm volatile("s_nop 15\n\ts_nop 7"
+                 : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[1][0]), "+v"(acc[1][1]),
+                   "+v"(acc[2][0]), "+v"(acc[2][1]), "+v"(acc[3][0]), "+v"(acc[3][1]));
+}
+
+// A column = two 512-element tiles.  Stage 1 as in tile_transform; stage 2 contracts the two
+// tiles' stage-1 results together (K = 32: 16 stage-2 inputs of each tile) against [G2; +G2] and
+// [G2; -G2], which yields the transform of the first and of the second half of the column (the
+// butterfly over element bit 9) without any vector arithmetic.
+template <class T16>
+struct PairOperands {
+    typename T16::V8 g1[2];
+    typename T16::V8 g2s, g2d;
+};
+
+template <class T16>
+__device__ __forceinline__ void make_pair_operands(PairOperands<T16>& po, int exp2)
+{
+    TileOperands<T16> ops;
+    make_tile_operands<T16, 2>(10, ops, exp2);
+    po.g1[0] = ops.g1[0];
+    po.g1[1] = ops.g1[1];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        po.g2s[j] = ops.g2[j];
+        po.g2s[4 + j] = ops.g2[j];
+        po.g2d[j] = ops.g2[j];
+        po.g2d[4 + j] = -ops.g2[j];
+    }
+}
+
+// lo_half / hi_half: lane l's elements 8l .. 8l+7 of H_1024 (x) restricted to k < 512 / k >= 512
+template <class T16>
+__device__ __forceinline__ void column_transform(typename T16::V8 t0, typename T16::V8 t1,
+                                                 const PairOperands<T16>& po,
+                                                 typename T16::V8& lo_half, typename T16::V8& hi_half)
+{
+    using E = typename T16::E;
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const f32x4 d0 = T16::mfma32(t0, po.g1[h], zero);
+        const f32x4 d1 = T16::mfma32(t1, po.g1[h], zero);
+        typename T16::V8 a2;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            a2[r] = (E)d0[r];
+            a2[4 + r] = (E)d1[r];
+        }
+        const f32x4 s = T16::mfma32(a2, po.g2s, zero);
+        const f32x4 d = T16::mfma32(a2, po.g2d, zero);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            lo_half[4 * h + r] = (E)s[r];
+            hi_half[4 * h + r] = (E)d[r];
+        }
+    }
+}
+
+__device__ __forceinline__ void wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+// at most N vector memory operations of this wavefront still outstanding (they complete in order)
+// (`n` folds to a constant once the loops around the call are unrolled)
+__device__ __forceinline__ void wait_vm(int n)
+{
+    switch (n) {
+        case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+        case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+        case 16: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
+        default: break;  // nothing to wait for
+    }
+}
+
+// 16 bytes per lane from global memory straight into LDS: lane l's bytes land at lds_base + 16 l.
+// Scalar base + 32-bit lane offset form, so that no vector arithmetic is spent on addresses.
+// (M0 carries the LDS base of the transfer; nothing else in this kernel uses it.)
+__device__ __forceinline__ void global_to_lds16(uint32_t lane_off, const void* base, uint32_t lds_base)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(lane_off), "s"(base), "s"(lds_base) : "memory");
+}
+// streaming (non-temporal) stores, scalar base + 32-bit lane offset
+__device__ __forceinline__ void stream_store4(uint32_t lane_off, uint32_t v, void* base)
+{
+    asm volatile("global_store_dword %0, %1, %2 nt" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
+}
+__device__ __forceinline__ void stream_store8(uint32_t lane_off, u32x2 v, void* base)
+{
+    asm volatile("global_store_dwordx2 %0, %1, %2 nt" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
+}
+
+template <class T16, int K, bool OUT_F32>
+__global__ void __launch_bounds__(kThreads)
+fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
+                          const typename T16::E* __restrict__ Xt, void* __restrict__ C, uint32_t M,
+                          uint32_t N, uint32_t m_per_block, uint32_t msplit, uint32_t mpx,
+                          int exp2, float mult)
+{
+    using E = typename T16::E;
+    using V8 = typename T16::V8;
+    typedef E V2 __attribute__((ext_vector_type(2)));
+    static_assert(K == 1024, "register budget: 32 columns x K / 128 = 256 registers per lane");
+    constexpr int KSTEPS = K / 32;
+    constexpr int SPB = K / kStageK;  // stages per row block
+    static_assert(SPB == kSlots, "the stage buffer of a stage is its K quarter");
+    constexpr uint32_t ROW_BYTES = K * 2u;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t lo = lane & 15u, hi = lane >> 4;
+
+    // ---- which tile: consecutive workgroup ids go to different XCDs (id % 8).  `mpx` = M slices
+    // handled inside one XCD: 1 keeps one slice of W per XCD L2 (and makes every XCD read all of
+    // X), larger values trade W locality for fewer redundant X reads per XCD.
+    uint32_t cg, ms;
+    {
+        const uint32_t id = blockIdx.x;
+        const uint32_t ngroups = gridDim.x / msplit;
+        if (msplit == 8u && (ngroups % mpx) == 0u && mpx <= 8u) {
+            const uint32_t x = id & 7u, j = id >> 3;  // XCD, index inside the XCD
+            const uint32_t sets = 8u / mpx;           // distinct slice sets
+            const uint32_t ss = x % sets, part = x / sets;
+            ms = ss * mpx + j % mpx;
+            cg = part * (ngroups / mpx) + j / mpx;
+        } else {
+            ms = id % msplit;
+            cg = id / msplit;
+        }
+    }
+    const uint32_t n0 = cg * kCols;
+    const uint32_t m_begin = ms * m_per_block;
+    if (m_begin >= M || n0 >= N) return;  // workgroup-uniform, before any barrier
+    const uint32_t m_end = min(M, m_begin + m_per_block);
+    const uint32_t nrb = (m_end - m_begin + kRows - 1u) / kRows;
+    // workgroups that share a slice of W start at different row blocks, so that they do not all
+    // ask the L2 for the same lines at the same moment
+    // (a slice whose last block is partial keeps its order, so that the partial block comes last)
+    const uint32_t rb0 = (m_end - m_begin) % kRows ? 0u : cg % nrb;
+    auto row_block = [&](uint32_t rbi) __attribute__((always_inline)) {  // the rbi-th row block this workgroup visits
+        uint32_t rb = rb0 + rbi;  // rbi <= nrb, rb0 < nrb
+        if (rb >= nrb) rb -= nrb;
+        if (rb >= nrb) rb -= nrb;
+        return rb;
+    };
+
+    // ---- W stream -------------------------------------------------------------------------------
+    // Stage g = (row block g / 4, K quarter g % 4) lives in stage buffer g % 4.  Wavefront w moves
+    // rows 16w .. 16w+15 of the block in eight pieces; piece i = rows 2i, 2i+1: lane l fetches row
+    // 2i + l/32 and lands at byte 16 l of the piece's 1 KB of LDS (the transfer's fixed lane order).
+    // LDS stage image: [64 rows][512 B] with 16-byte chunk q of row r stored at q ^ (r & 15), so
+    // the lane asks for chunk (l % 32) ^ (r & 15): a half-wavefront still covers one contiguous
+    // 512-byte row segment (four adjacent lanes one aligned 64-byte run), and a fragment read
+    // (lane (hi, lo): row 16 mb + lo, chunk 4 ks + hi) hits 16 different 16-byte bank groups.
+    const unsigned char* Wb = reinterpret_cast<const unsigned char*>(W);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;  // LDS byte address of the array
+    const uint32_t lrow = lane >> 5, lq = lane & 31u;
+    uint32_t voff[8];  // byte offset of this lane's 16 bytes of piece i, K quarter 0, in W
+    auto set_voff = [&](uint32_t rbi) __attribute__((always_inline)) {
+        const uint32_t r0 = m_begin + row_block(rbi) * kRows + 16u * wave + lrow;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            voff[i] = min(r0 + 2u * i, M - 1u) * ROW_BYTES + ((lq ^ (2u * i + lrow)) << 4);
+    };
+    auto w_issue = [&](uint32_t kq, uint32_t slot, int i) __attribute__((always_inline)) {
+        global_to_lds16(voff[i], Wb + kq * (kStageK * 2u),
+                        lds_base + slot * kStageBytes + (16u * wave + 2u * i) * 512u);
+    };
+    set_voff(0);
+
+    // ---- prologue: Y fragments of this wavefront's 32 columns ------------------------------------
+    // Column of fragment nb, fragment column j (= MFMA B column = lane lo): n0 + 32w + 2j + nb, so
+    // that a lane ends up with pairs of adjacent output columns.
+    V8 yf[2][KSTEPS];
+    {
+        PairOperands<T16> po;
+        make_pair_operands<T16>(po, exp2);
+        unsigned char* area = lds + kAreaBase + wave * kAreaBytes;
+        // the 32 tiles of a round are all in flight at once (128 registers); the tiles of the
+        // second round are requested as the first round's are consumed
+        V8 in[16][2];
+        auto load_col = [&](int nb, int j) {
+            const uint32_t col = min(n0 + 32u * wave + 2u * j + nb, N - 1u);
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+                in[j][t] = *reinterpret_cast<const V8*>(Xt + ((uint64_t)col * K + 512u * t + 8u * lane));
+        };
+#pragma unroll
+        for (int j = 0; j < 16; ++j) load_col(0, j);
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+            V8 hold[16];  // second halves (k >= 512) wait here while the first go through LDS
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                V8 first_half;
+                column_transform<T16>(in[j][0], in[j][1], po, first_half, hold[j]);
+                if (nb == 0) load_col(1, j);
+                // The first three W stages are requested behind the last X tile (vector memory
+                // operations complete in order, so anything issued earlier would hold the tiles
+                // back), two pieces per column of the second round, while its tiles arrive.
+                if (nb == 1 && j >= 2 && j < 14) {
+                    const int p = 2 * (j - 2);
+                    w_issue(p >> 3, p >> 3, p & 7);
+                    w_issue((p + 1) >> 3, (p + 1) >> 3, (p + 1) & 7);
+                }
+                // area: [16 columns][64 chunks of 16 B], chunk q of column j stored at q ^ j
+                *reinterpret_cast<V8*>(area + j * 1024u + ((lane ^ j) << 4)) = first_half;
+            }
+            // LDS operations of one wavefront complete in order: no barrier between its own
+            // writes and reads
+#pragma unroll
+            for (int s = 0; s < KSTEPS / 2; ++s)
+                yf[nb][s] = *reinterpret_cast<const V8*>(area + lo * 1024u + (((4u * s + hi) ^ lo) << 4));
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+                *reinterpret_cast<V8*>(area + j * 1024u + ((lane ^ j) << 4)) = hold[j];
+#pragma unroll
+            for (int s = 0; s < KSTEPS / 2; ++s)
+                yf[nb][KSTEPS / 2 + s] =
+                    *reinterpret_cast<const V8*>(area + lo * 1024u + (((4u * s + hi) ^ lo) << 4));
+        }
+    }
+
+    // Every wavefront has finished with its area (stage buffer 3 may be filled from now on), and
+    // its pieces of stage 0 have landed (the 16 pieces of stages 1 and 2 may still be in flight).
+    asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+
+    auto frag = [&](uint32_t slot, int mb, int ks) __attribute__((always_inline)) -> V8 {
+        return *reinterpret_cast<const V8*>(lds + slot * kStageBytes + (16u * mb + lo) * 512u +
+                                            (((4u * ks + hi) ^ lo) << 4));
+    };
+    V8 fr[4][4];  // [K step % 4][mb]
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) {
+        fr[0][mb] = frag(0, mb, 0);
+        fr[1][mb] = frag(0, mb, 1);
+    }
+
+    // ---- output addressing ------------------------------------------------------------------------
+    // lane (hi, lo) of a row block owns rows 16 mb + 4 hi + r and the column pair 2 lo, 2 lo + 1 of
+    // its wavefront's 32 columns
+    constexpr uint32_t esize = OUT_F32 ? 4u : 2u;
+    const uint32_t col = n0 + 32u * wave + 2u * lo;
+    const uint32_t lane_off = (4u * hi * N + col) * esize;  // inside the row block, < 2^32
+    unsigned char* const Cb = static_cast<unsigned char*>(C);
+    // `mult` is the part of the scale that is not a power of two: 1 for the usual scales, and only
+    // then do row blocks take the interleaved store path
+    const bool cols_full = n0 + kCols <= N && (N & 1u) == 0 && mult == 1.0f;
+
+    // one store of the interleaved epilogue: rows 16 mb + 4 hi + r of a full row block
+    auto store_pair = [&](const f32x4 (&acc)[4][2], uint64_t block_base, int mb, int r)
+        __attribute__((always_inline)) {
+        const float v0 = acc[mb][0][r], v1 = acc[mb][1][r];
+        // streaming stores: C is not read again, and keeping it out of the L2 leaves the cache to
+        // the operands
+        unsigned char* row_ptr = Cb + (block_base + (uint64_t)((16u * mb + r) * N) * esize);  // scalar
+        if (OUT_F32)
+            stream_store8(lane_off, u32x2{__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1)}, row_ptr);
+        else
+            stream_store4(lane_off, __builtin_bit_cast(uint32_t, V2{(E)v0, (E)v1}), row_ptr);
+    };
+    // the same for a row block at the edge of the matrix (masked, element by element)
+    auto store_edge = [&](const f32x4 (&acc)[4][2], uint32_t row_base) __attribute__((always_inline)) {
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t row = row_base + 16u * mb + 4u * hi + r;
+                if (row >= m_end) continue;
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb) {
+                    if (col + nb >= N) continue;
+                    const float v = acc[mb][nb][r] * mult;
+                    const uint64_t at = (uint64_t)row * N + col + nb;
+                    if (OUT_F32)
+                        static_cast<float*>(C)[at] = v;
+                    else
+                        static_cast<E*>(C)[at] = (E)v;
+                }
+            }
+    };
+
+    // ---- one row block: 32 K steps into `acc`, while `prev` (the previous row block's result, when
+    // the tag says there is one) is stored two pieces per K step of the first stage ----------------
+    auto row_block_body = [&](auto prev_tag, f32x4 (&acc)[4][2], const f32x4 (&prev)[4][2],
+                              uint64_t prev_base, uint32_t rbi) __attribute__((always_inline)) {
+        constexpr bool prev_full = decltype(prev_tag)::value;
+        // the last row block requests only its own fourth stage: nothing follows it
+        const bool last = rbi + 1u == nrb;
+#pragma unroll
+        for (int kq = 0; kq < SPB; ++kq) {
+            // pieces of stage g+3 issued during K step ks of this stage
+            constexpr int kPieceAt[7] = {0, 2, 4, 5, 6, 7, 8};
+#pragma unroll
+            for (int ks = 0; ks < kStepsPerStage; ++ks) {
+                if (kq == 1 && ks == 0 && !last) set_voff(rbi + 1u);  // stages g+3: the next block's
+                const int kk = kq * kStepsPerStage + ks;
+#pragma unroll
+                for (int m = 0; m < 8; ++m) {
+                    const int mb = m >> 1, nb = m & 1;
+                    if (kk == 0)
+                        XMfma<T16>::first(acc[mb][nb], fr[ks & 3][mb], yf[nb][0]);
+                    else
+                        XMfma<T16>::next(acc[mb][nb], fr[ks & 3][mb], yf[nb][kk]);
+                    // one memory instruction in the shadow of each MFMA
+                    if (m < 4) {
+                        // fragments two K steps ahead; the last two steps of a stage read the
+                        // first two of the next stage, behind the barrier
+                        fr[(ks + 2) & 3][m] = ks < 6 ? frag(kq, m, ks + 2) : frag((kq + 1) & 3, m, ks - 6);
+                    } else if (m < 6) {
+                        if (ks < 6 && (kq == 0 || !last)) {
+                            const int i = kPieceAt[ks] + (m - 4);
+                            if (i < kPieceAt[ks + 1]) w_issue((kq + 3) & 3, (kq + 3) & 3, i);
+                        }
+                    }
+                    // the previous block's sixteen stores, one behind each MFMA of the two K steps
+                    // that follow the first stage's barrier: they then have a whole stage to
+                    // complete before the next barrier counts outstanding memory operations
+                    if (prev_full && kq == 0 && ks >= 6) {
+                        const int e = 8 * (ks - 6) + m;
+                        store_pair(prev, prev_base, e >> 2, e & 3);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                // The matrix core reads its 128-bit A operand over several cycles after issue, and
+                // the compiler, which sees an opaque statement, would hand a fragment register to a
+                // temporary right behind the last MFMA that uses it (observed: a v_mov one
+                // instruction later corrupted the product).  Naming the previous step's fragments
+                // here keeps all four fragment sets allocated for the whole loop.
+                asm volatile("" ::"v"(fr[(ks + 3) & 3][0]), "v"(fr[(ks + 3) & 3][1]),
+                             "v"(fr[(ks + 3) & 3][2]), "v"(fr[(ks + 3) & 3][3]));
+                if (ks == 5) {
+                    // Own pieces of stage g+1 have landed.  Loads complete in order among
+                    // themselves, but not relative to stores, so the count allowed to remain
+                    // outstanding is the number of *loads* requested after those pieces (8 of
+                    // stage g+2, 8 of stage g+3; fewer at the end of the last row block): pending
+                    // stores can only make this wait longer, never shorter.
+                    constexpr int kAfterLast[4] = {16, 8, 0, -1};
+                    if (last)
+                        wait_vm(kAfterLast[kq]);
+                    else
+                        wait_vm(16);
+                    wait_lds();
+                    __builtin_amdgcn_s_barrier();
+                }
+            }
+        }
+    };
+
+    f32x4 accA[4][2], accB[4][2];
+    bool pend = false;        // accB holds a finished full row block that is not stored yet
+    uint64_t pend_base = 0;
+    auto run = [&](bool prev_full, f32x4 (&acc)[4][2], const f32x4 (&prev)[4][2], uint64_t prev_base,
+                   uint32_t rbi) __attribute__((always_inline)) {
+        if (prev_full)
+            row_block_body(std::true_type{}, acc, prev, prev_base, rbi);
+        else
+            row_block_body(std::false_type{}, acc, prev, prev_base, rbi);
+    };
+    auto finish = [&](f32x4 (&acc)[4][2], uint32_t rbi, bool& full, uint64_t& base)
+        __attribute__((always_inline)) {
+        // a full block is stored during the next block; an edge block right away
+        const uint32_t row_base = m_begin + row_block(rbi) * kRows;
+        full = cols_full && row_base + kRows <= m_end;
+        base = (uint64_t)row_base * N * esize;
+        if (!full) {
+            drain_mfma(acc);
+            store_edge(acc, row_base);
+        }
+    };
+#pragma unroll 1
+    for (uint32_t rbi = 0; rbi < nrb; rbi += 2u) {
+        run(pend, accA, accB, pend_base, rbi);
+            bool fullA;
+        uint64_t baseA;
+        finish(accA, rbi, fullA, baseA);
+        if (rbi + 1u < nrb) {
+            run(fullA, accB, accA, baseA, rbi + 1u);
+                    finish(accB, rbi + 1u, pend, pend_base);
+        } else {
+            pend = false;
+            if (fullA) {
+                drain_mfma(accA);
+#pragma unroll
+                for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) store_pair(accA, baseA, mb, r);
+            }
+        }
+    }
+    if (pend) {
+        drain_mfma(accB);
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) store_pair(accB, pend_base, mb, r);
+    }
+    // Every transfer into LDS was waited for at the barrier of the stage before the one that read
+    // it, so none is in flight when the workgroup's LDS is released.
+}
+
+// msplit / m_per_block: about one workgroup per compute unit, every slice a multiple of 64 rows.
+struct Plan {
+    uint32_t ngroups, msplit, m_per_block;
+};
+inline Plan plan(uint32_t M, uint32_t N)
+{
+    Plan p;
+    p.ngroups = (N + kCols - 1u) / kCols;
+    const uint32_t row_blocks = (M + kRows - 1u) / kRows;
+    uint32_t msplit = (256u + p.ngroups - 1u) / p.ngroups;
+    if (msplit > row_blocks) msplit = row_blocks;
+    if (msplit < 1u) msplit = 1u;
+    p.m_per_block = ((row_blocks + msplit - 1u) / msplit) * kRows;
+    p.msplit = (M + p.m_per_block - 1u) / p.m_per_block;
+    return p;
+}
+
+template <class T16, int K, bool OUT_F32>
+int launch_as(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, float scale,
+              uint32_t mpx, hipStream_t s)
+{
+    const OutputScale os = split_output_scale((double)scale, tile_stage_shift<2>(10));
+    const Plan p = plan(M, N);
+    auto kern = fused_ht_gemm_xreg_kernel<T16, K, OUT_F32>;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess)
+        return MI_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(p.ngroups * p.msplit), dim3(kThreads), kLdsBytes, s,
+                       static_cast<const typename T16::E*>(W),
+                       static_cast<const typename T16::E*>(Xt), C, M, N, p.m_per_block, p.msplit, mpx,
+                       os.exp2, os.mult);
+    return launch_status();
+}
+
+template <class T16, int K>
+int launch(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, int out_f32, float scale,
+           uint32_t mpx, hipStream_t s)
+{
+    return out_f32 ? launch_as<T16, K, true>(W, Xt, C, M, N, scale, mpx, s)
+                   : launch_as<T16, K, false>(W, Xt, C, M, N, scale, mpx, s);
+}
+
+}  // namespace xreg
+
+// Called by the dispatcher of mi_fused_ht_gemm for K = 1024 (arguments already validated there).
+int fused_gemm16_xreg(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, int in_dtype,
+                      int out_f32, float scale, hipStream_t s)
+{
+    // W and a row block of C are addressed with 32-bit byte offsets
+    if ((uint64_t)M * 2048u > 0xffffffffull || (uint64_t)N * 4u * 64u > 0xffffffffull)
+        return MI_ERR_SHAPE;
+    if (in_dtype == MI_BF16) return xreg::launch<BF16, 1024>(W, Xt, C, M, N, out_f32, scale, 2u, s);
+    if (in_dtype == MI_F16) return xreg::launch<F16, 1024>(W, Xt, C, M, N, out_f32, scale, 2u, s);
+    return MI_ERR_DTYPE;
+}
+
+}  // namespace mi

@@ -106,6 +106,46 @@ def test_gemm_against_oracle(pkg, oracle, M, N, K, dt, tol):
         assert _rel(oracle, C16, want) <= tol
 
 
+# K = 1024 runs the register-resident kernel: 128-column groups, 64-row blocks, results stored
+# while the next row block is multiplied.  Shapes around every tile boundary, a single row block,
+# odd N (no paired stores), a scale that is not a power of two (separate store path), both 16-bit
+# types and both output types.
+@pytest.mark.parametrize("M,N", [(1, 1), (63, 127), (64, 128), (65, 129), (128, 256), (577, 1333),
+                                 (130, 2000), (4096, 130), (700, 4095)])
+def test_gemm_k1024_tile_boundaries(pkg, oracle, M, N):
+    K = 1024
+    for dt in (torch.bfloat16, torch.float16):
+        W, Xt = oracle.inputs_gemm(M, N, K, dt)
+        for scale, od in ((None, torch.float32), (None, dt), (0.37 / 32.0, torch.float32),
+                          (1.0, torch.float32), (1.0 / 64.0, dt)):
+            if dt == torch.float16 and scale == 1.0:
+                continue  # unnormalised fp16 overflows the storage range by construction
+            s = 1.0 / 32.0 if scale is None else scale
+            C = pkg.fused_ht_gemm(W.cuda(), Xt.cuda(), scale, out_dtype=od)
+            torch.cuda.synchronize()
+            want = oracle.fused_ht_gemm_f64_blas(W.double().numpy(), Xt.double().numpy(), s)
+            assert C.shape == (M, N) and C.dtype == od
+            assert _rel(oracle, C, want) <= 2e-2, (M, N, dt, scale, od)
+
+
+def test_gemm_k1024_every_output_written_once(pkg, oracle):
+    # size-independent check on the full benchmark shape, both output types: C against the
+    # unfused product computed on the device from the library's own transform, every element
+    M = N = 4096
+    K = 1024
+    W, Xt = oracle.inputs_gemm(M, N, K, torch.bfloat16)
+    Wd, Xd = W.cuda(), Xt.cuda()
+    Y = pkg.hadamard_transform(Xd)                      # bf16, same rounding as the fused operand
+    ref = Wd.float() @ Y.float().t()
+    scale = ref.abs().max().item()
+    for od in (torch.bfloat16, torch.float32):
+        for _ in range(3):                               # back-to-back launches reuse LDS and registers
+            C = pkg.fused_ht_gemm(Wd, Xd, out_dtype=od)
+        torch.cuda.synchronize()
+        err = (C.float() - ref).abs().max().item() / scale
+        assert err <= (8e-3 if od == torch.bfloat16 else 2e-3), (od, err)
+
+
 def test_gemm_small_bruteforce(pkg, oracle):
     # triple-loop oracle (no BLAS), fp32
     M, N, K = 16, 20, 64
