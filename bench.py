@@ -2,22 +2,30 @@
 """Benchmark of the Hadamard hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep] [--no-cpu]
+                    [--only-gemm | --only-fwht | --only-rht | --only-gemv | --only-gemm-f32]
 
-A *step* is one pass of the stand-alone transform over one batch: the in-place normalised FWHT of
-a bf16 X[16384, 4096] (the headline benchmark configuration), inputs resident in HBM before timing starts.  The
-protocol is the reference's (bench/bench.py:112-127): warm-up launches, then K back-to-back
-launches on the same buffer inside one event window on the launch stream.  One JSON line is
-printed; besides the headline it carries
-  roofline      - the transform kernel against the 8 TB/s HBM peak,
-  cpu_baseline  - the reference's truth path (x @ Sylvester matrix in torch, on the host cores)
-                  on a bounded row sample of the same workload,
-  fused_ht_gemm - C = W.H(X) at K=1024, M=N=4096 in bf16 against the dense bf16 MFMA peak,
-  others        - the remaining configurations (fp32 fused GEMM, HT+GEMV, RHT+FP8 quantize,
-                  FP8 GEMM), and with --sweep the n = 2^4..2^15 transform sweep.
+The reference's compound metric has two halves and both are printed at the top level of the one
+JSON line:
+
+  value / roofline / cpu_baseline       the fused HT->GEMM  C = W.H(X)/32  at K=1024, M=N=4096 in
+                                        bf16 (fp32 accumulate, C in bf16) against the dense bf16
+                                        MFMA peak.  A *step* is one call of fused_ht_gemm.
+  fwht.value / .roofline / .cpu_baseline  the stand-alone in-place normalised FWHT of a bf16
+                                        X[16384, 4096] against the 8 TB/s HBM peak, plus
+                                        fwht.dram_bound: the same kernel on 2^30 elements (the
+                                        reference harness's size, bench/bench.py:138), which does
+                                        not fit the 256 MiB Infinity Cache.
+
+Timing protocol (the reference's, bench/bench.py:112-127): warm-up launches, then K back-to-back
+launches inside one event window on the launch stream, inputs resident in HBM.  The matrix-core
+bound kernels are warmed for at least 60 ms first (clock ramp).  `others` carries the remaining
+configurations (fp32 fused GEMM, HT+GEMV with its unfused comparator, RHT+FP8 quantize, FP8 GEMM),
+and with --sweep the n = 2^4..2^15 transform sweep.
 """
 from __future__ import annotations
 
 import argparse
+import hashlib
 import importlib
 import json
 import math
@@ -29,56 +37,44 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+PKG = "6s894_project_2025_amd"
 HBM_PEAK_GBS = 8000.0
 PEAK_TFLOPS = {"bf16": 2516.6, "f16": 2516.6, "f32": 157.3, "fp8": 5033.2}
+BASELINE_METRIC = "fused HT+GEMM TFLOP/s (K=1024,M=N=4096) + standalone FWHT HBM GB/s vs peak"
 
 
-def _events_ms(torch, fn, steps, warmup):
-    """Average milliseconds per call: `warmup` untimed calls, then `steps` back-to-back calls
-    bracketed by events on the current stream and full synchronisation on both sides."""
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()
-    t0 = torch.cuda.Event(enable_timing=True)
-    t1 = torch.cuda.Event(enable_timing=True)
-    w0 = time.perf_counter()
-    t0.record()
-    for _ in range(steps):
-        fn()
-    t1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - w0) * 1e3
-    return t0.elapsed_time(t1) / steps, wall_ms / steps
+def kernel_sources_digest() -> str:
+    """sha256 over the HIP sources the timed kernels are built from (names and contents)."""
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, PKG, "csrc")
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".hip", ".hpp")):
+            h.update(name.encode())
+            with open(os.path.join(csrc, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()
 
 
-def _steady_ms(torch, fn, steps, warm_ms=60.0):
-    """Like _events_ms, but the untimed warm-up lasts at least `warm_ms` of GPU time: the
-    matrix-core-bound kernels keep speeding up for the first ~30 ms of sustained load while the
-    clocks ramp, so a three-call warm-up would time the ramp rather than the kernel."""
-    fn()
-    torch.cuda.synchronize()
-    t0 = torch.cuda.Event(enable_timing=True)
-    t1 = torch.cuda.Event(enable_timing=True)
-    spent, batch = 0.0, 4
-    while spent < warm_ms:
-        t0.record()
-        for _ in range(batch):
-            fn()
-        t1.record()
-        torch.cuda.synchronize()
-        spent += t0.elapsed_time(t1)
-        batch = min(batch * 2, 256)
-    return _events_ms(torch, fn, steps, 0)
-
-
-def _load_traffic():
-    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), recorded in
-    profiles/hbm_traffic.json by hand from the committed summaries; None when absent."""
+def load_traffic() -> dict:
+    """HBM bytes per launch recorded from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs
+    (profiles/hbm_traffic.json, figures taken from the summaries beside it).  The file names the
+    digest of the kernel sources it was measured on; when the sources have changed since, every
+    figure is reported as null rather than as a stale number."""
     p = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-    if os.path.exists(p):
-        with open(p) as f:
-            return json.load(f)
-    return {}
+    if not os.path.exists(p):
+        return {}
+    with open(p) as f:
+        rec = json.load(f)
+    if rec.get("kernel_sources_sha256") != kernel_sources_digest():
+        return {}
+    return rec.get("bytes_per_launch", {})
+
+
+def roofline(bound, achieved, peak, unit, traffic, **extra):
+    r = {"bound": bound, "achieved": round(achieved, 1), "peak": peak, "unit": unit,
+         "frac": round(achieved / peak, 4), "traffic": traffic}
+    r.update(extra)
+    return r
 
 
 def main() -> int:
@@ -87,11 +83,11 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--sweep", action="store_true", help="also time n = 2^4..2^15 (128 MiB each)")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only-fwht", action="store_true", help="headline kernel only (profiling)")
-    ap.add_argument("--only-gemm", action="store_true", help="fused GEMM only (profiling)")
-    ap.add_argument("--only-rht", action="store_true",
-                    help="RHT + FP8 quantize and FP8 GEMM only (profiling)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    for flag, what in (("fwht", "stand-alone transform"), ("gemm", "fused bf16 GEMM"),
+                       ("gemm-f32", "fused fp32 GEMM"), ("gemv", "fused HT+GEMV"),
+                       ("rht", "RHT + FP8 quantize and FP8 GEMM")):
+        ap.add_argument(f"--only-{flag}", action="store_true", help=f"{what} only (profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.stderr.write("bench.py: this build runs on exactly one GPU; --gpus must be 1 "
@@ -103,19 +99,66 @@ def main() -> int:
     if not torch.cuda.is_available():
         sys.stderr.write("bench.py: no GPU visible\n")
         return 2
-    hada = importlib.import_module("6s894_project_2025_amd")
+    hada = importlib.import_module(PKG)
+    timing = importlib.import_module(PKG + ".timing")
+    events_ms, steady_ms = timing.event_window_ms, timing.steady_window_ms
     dev = torch.device("cuda:0")
-    traffic = _load_traffic()
+    traffic = load_traffic()
     steps, warmup = args.steps, args.warmup
+    only = [k for k in ("fwht", "gemm", "gemm_f32", "gemv", "rht") if getattr(args, "only_" + k)]
+    want = (lambda k: not only or k in only)
 
-    # ---- headline: config 2 ---------------------------------------------------------------------
+    result: dict = {}
+    others: dict = {}
+
+    # ---- fused HT -> GEMM, bf16 (config 4): the first half of the metric -----------------------------
+    M = N = 4096
+    K = 1024
+    flops = 2 * M * N * K
+    if want("gemm"):
+        W = torch.randn(M, K, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(dev)
+        Xt = torch.randn(N, K, generator=torch.Generator().manual_seed(0)).to(torch.bfloat16).to(dev)
+        C = hada.fused_ht_gemm(W, Xt)
+        # whole-output check against the unfused product of the library's own transform
+        ref = torch.matmul(W.float(), hada.hadamard_transform(Xt).float().t())
+        err = ((C.float() - ref).abs().max() / ref.abs().max()).item()
+        del ref
+        gsteps = max(10, steps)
+        steady_ms(lambda: hada.fused_ht_gemm(W, Xt), 4)  # clock ramp, untimed
+        ms, wall_ms = events_ms(lambda: hada.fused_ht_gemm(W, Xt), gsteps, warmup)
+        tf = flops / ms / 1e9
+        mm_ms, _ = steady_ms(lambda: torch.matmul(W, Xt.t()), gsteps)
+        # the reference's "Baseline (Unfused)" (fusion_pipelined.cu:640-656): transform kernel, H(X)
+        # through HBM, then the GEMM (here the vendor library's)
+        un_ms, _ = steady_ms(lambda: torch.matmul(W, hada.hadamard_transform(Xt).t()), gsteps)
+        result.update({
+            "metric": BASELINE_METRIC,
+            "value": round(tf, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": gsteps, "warmup": warmup,
+            "ms_per_step": round(ms, 6), "wall_ms_per_step": round(wall_ms, 6),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "BASELINE configs[3]: fused C = W.(H_1024 X)/32, W[4096,1024] seed 1, "
+                                   "Xt[4096,1024] seed 0, iid N(0,1), bf16 in, fp32 accumulate, bf16 out; "
+                                   "`value` is this half of the metric, `fwht` the other",
+                       "M": M, "N": N, "K": K, "algorithmic_flops_per_step": flops},
+            "roofline": roofline("mfma", tf, PEAK_TFLOPS["bf16"], "TFLOP/s",
+                                 traffic.get("fused_ht_gemm_bf16"),
+                                 kernel="fused_ht_gemm_xreg_kernel<BF16,1024,false>"),
+            "checks": {"fused_vs_unfused_max_rel_diff": err},
+            "library_gemm_without_transform_tflops": round(flops / mm_ms / 1e9, 1),
+            "unfused_transform_then_library_gemm_ms": round(un_ms, 6),
+            "fused_over_unfused_speedup": round(un_ms / ms, 3),
+        })
+        del W, Xt, C
+
+    # ---- stand-alone FWHT (config 2): the second half ------------------------------------------------
     rows, n = 16384, 4096
-    g = torch.Generator().manual_seed(0)
-    x_cpu = torch.randn(rows, n, generator=g, dtype=torch.float32).to(torch.bfloat16)
-    result = {}
-    if not (args.only_gemm or args.only_rht):
+    x_cpu = None
+    if want("fwht"):
+        g = torch.Generator().manual_seed(0)
+        x_cpu = torch.randn(rows, n, generator=g, dtype=torch.float32).to(torch.bfloat16)
         x = x_cpu.to(dev)
-        ms, wall_ms = _events_ms(torch, lambda: hada.hadamard_transform(x, inplace=True), steps, warmup)
+        ms, wall_ms = events_ms(lambda: hada.hadamard_transform(x, inplace=True), steps, warmup)
         alg_bytes = 2 * rows * n * 2
         gbs = alg_bytes / ms / 1e6
         # size-independent sanity on the timed buffer: an even number of normalised transforms
@@ -123,110 +166,121 @@ def main() -> int:
         if (steps + warmup) % 2 == 1:
             hada.hadamard_transform(x, inplace=True)
         drift = (x.float() - x_cpu.to(dev).float()).abs().max().item()
-        add_ms, _ = _events_ms(torch, lambda: x.add_(1), min(steps, 50), 3)
-        result = {
-            "metric": "standalone FWHT HBM GB/s (bf16 [16384,4096], in place; half of the reference's "
-                      "compound metric, the fused HT+GEMM TFLOP/s half is under fused_ht_gemm)",
-            "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        add_ms, _ = events_ms(lambda: x.add_(1), min(steps, 50), 3)
+        fw = {
+            "metric": "standalone FWHT HBM GB/s (bf16 [16384,4096], in place)",
+            "value": round(gbs, 1), "unit": "GB/s", "steps": steps, "warmup": warmup,
             "ms_per_step": round(ms, 6), "wall_ms_per_step": round(wall_ms, 6),
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-            "dtype": "bf16", "data": "synthetic",
             "config": {"workload": "BASELINE configs[1]: in-place normalised FWHT over the last dim, "
                                    "bf16 X[16384,4096] iid N(0,1) seed 0, scale 1/64",
                        "rows": rows, "n": n, "algorithmic_bytes_per_step": alg_bytes},
-            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
-                         "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
-                         "traffic": traffic.get("fwht_bf16_16384x4096"),
-                         "kernel": "fwht_reg_kernel<Io16<BF16>,8,3>",
-                         "add_one_proxy_gbs": round(alg_bytes / add_ms / 1e6, 1)},
+            "roofline": roofline("hbm", gbs, HBM_PEAK_GBS, "GB/s", traffic.get("fwht_bf16_16384x4096"),
+                                 kernel="fwht_reg_kernel<Io16<BF16>,8,3>",
+                                 add_one_proxy_gbs=round(alg_bytes / add_ms / 1e6, 1),
+                                 note="the 128 MiB buffer is re-run in place and fits the 256 MiB "
+                                      "Infinity Cache: this figure is cache-assisted; dram_bound below "
+                                      "is the same kernel on a tensor that does not fit"),
             "checks": {"max_abs_drift_after_even_number_of_transforms": drift},
         }
         del x
-        if args.only_fwht:
-            print(json.dumps(result))
-            return 0
-
-    # ---- fused HT -> GEMM, config 4 -----------------------------------------------------------------
-    M = N = 4096
-    K = 1024
-    gsteps = max(10, min(steps, 200))
-    others = {}
-    for name, dt in (() if args.only_rht else (("bf16", torch.bfloat16), ("f32", torch.float32))):
-        W = torch.randn(M, K, generator=torch.Generator().manual_seed(1)).to(dt).to(dev)
-        Xt = torch.randn(N, K, generator=torch.Generator().manual_seed(0)).to(dt).to(dev)
-        C = hada.fused_ht_gemm(W, Xt)
-        ms, _ = _steady_ms(torch, lambda: hada.fused_ht_gemm(W, Xt), gsteps)
-        flops = 2 * M * N * K
-        tf = flops / ms / 1e9
-        entry = {"metric": f"fused HT+GEMM TFLOP/s (K=1024, M=N=4096, {name}, fp32 accumulate, "
-                           f"C in {name})",
-                 "value": round(tf, 1), "unit": "TFLOP/s", "ms_per_step": round(ms, 6), "steps": gsteps,
-                 "algorithmic_flops_per_step": flops,
-                 "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_TFLOPS[name],
-                              "unit": "TFLOP/s", "frac": round(tf / PEAK_TFLOPS[name], 4),
-                              "traffic": traffic.get(f"fused_ht_gemm_{name}")}}
-        if name == "bf16":
-            mm_ms, _ = _steady_ms(torch, lambda: torch.matmul(W, Xt.t()), gsteps)
-            entry["library_gemm_without_transform_tflops"] = round(flops / mm_ms / 1e9, 1)
-            # the reference's "Baseline (Unfused)" (fusion_pipelined.cu:640-656): transform kernel,
-            # H(X) through HBM, then the vendor GEMM
-            un_ms, _ = _steady_ms(
-                torch, lambda: torch.matmul(W, hada.hadamard_transform(Xt).t()), gsteps)
-            entry["unfused_transform_then_library_gemm_ms"] = round(un_ms, 6)
-            entry["fused_over_unfused_speedup"] = round(un_ms / ms, 3)
-            result["fused_ht_gemm"] = entry
-            if args.only_gemm:
-                print(json.dumps(entry))
-                return 0
+        # DRAM-bound rows: 2^30 bf16 elements (2 GiB), the reference harness's size
+        dram = {}
+        for nn in (4096, 32768):
+            big = torch.empty((1 << 30) // nn, nn, dtype=torch.bfloat16, device=dev).normal_()
+            bsteps = max(5, min(steps, 20))
+            bms, _ = events_ms(lambda: hada.hadamard_transform(big, inplace=True), bsteps, 2)
+            ams, _ = events_ms(lambda: big.add_(1), bsteps, 2)
+            bb = 2 * big.numel() * 2
+            dram[f"bf16_2^30_elements_n{nn}"] = {
+                "ms_per_step": round(bms, 5), "algorithmic_bytes_per_step": bb,
+                "roofline": roofline("hbm", bb / bms / 1e6, HBM_PEAK_GBS, "GB/s",
+                                     traffic.get(f"fwht_bf16_2^30_n{nn}"),
+                                     add_one_proxy_gbs=round(bb / ams / 1e6, 1))}
+            del big
+        fw["dram_bound"] = dram
+        if result:
+            result["fwht"] = fw
         else:
-            others["fused_ht_gemm_f32"] = entry
-        del W, Xt, C
+            result = fw
+    if only == ["fwht"] or only == ["gemm"]:
+        print(json.dumps(result))
+        return 0
 
-    # ---- remaining configurations --------------------------------------------------------------------
-    for (m, nn, b) in (() if args.only_rht else
-                       ((256, 256, 512), (1024, 1024, 8), (1024, 1024, 64), (1024, 1024, 512))):
-        W = torch.randn(m, nn, device=dev) / math.sqrt(nn)
-        X = torch.randn(nn, b, device=dev)
-        ms, _ = _events_ms(torch, lambda: hada.fused_ht_gemv(W, X), 50, 3)
-        others[f"fused_ht_gemv_M{m}_N{nn}_B{b}"] = {
-            "us": round(ms * 1e3, 2),
-            "algorithmic_bytes": 4 * (m * nn + nn * b + m * b),
-            "algorithmic_flops": 2 * m * nn * b + int(nn * math.log2(nn) * b),
-            "GB/s": round(4 * (m * nn + nn * b + m * b) / ms / 1e6, 1),
-            "TFLOP/s": round((2 * m * nn * b + nn * math.log2(nn) * b) / ms / 1e9, 3)}
-    T, nq, Nw = 8192, 4096, 14336
-    xa = torch.randn(T, nq, generator=torch.Generator().manual_seed(0))
-    outl = torch.randperm(nq, generator=torch.Generator().manual_seed(3))[:41]  # 1 % outlier channels
-    xa[:, outl] *= 50.0
-    xa = xa.to(torch.bfloat16).to(dev)
-    sign = (1 - 2 * torch.randint(0, 2, (nq,), generator=torch.Generator().manual_seed(2))).to(torch.int8).to(dev)
-    ms, _ = _events_ms(torch, lambda: hada.rht_quant_fp8(xa, sign), 50, 3)
-    qbytes = T * nq * 3 + T * 4
-    others["rht_quant_fp8_8192x4096"] = {
-        "us": round(ms * 1e3, 2), "algorithmic_bytes": qbytes, "GB/s": round(qbytes / ms / 1e6, 1),
-        "roofline": {"bound": "hbm", "achieved": round(qbytes / ms / 1e6, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(qbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
-                     "traffic": traffic.get("rht_quant_fp8_8192x4096")}}
-    qx, sx = hada.rht_quant_fp8(xa, sign)
-    w = (torch.randn(Nw, nq, device=dev) * 0.02).to(torch.bfloat16)
-    qw, sw = hada.rht_quant_fp8(w, sign)
-    ms, _ = _steady_ms(torch, lambda: hada.fp8_gemm_rowscale(qx, sx, qw, sw), 20)
-    fl = 2 * T * Nw * nq
-    others["fp8_gemm_8192x14336x4096"] = {
-        "us": round(ms * 1e3, 1), "algorithmic_flops": fl, "TFLOP/s": round(fl / ms / 1e9, 1),
-        "roofline": {"bound": "mfma", "achieved": round(fl / ms / 1e9, 1), "peak": PEAK_TFLOPS["fp8"],
-                     "unit": "TFLOP/s", "frac": round(fl / ms / 1e9 / PEAK_TFLOPS["fp8"], 4),
-                     "traffic": traffic.get("fp8_gemm_8192x14336x4096_l2_fill_plus_write")}}
-    try:  # the vendor library's row-scaled FP8 GEMM on the same operands, for comparison only
-        lib_ms, _ = _steady_ms(torch, lambda: torch._scaled_mm(
-            qx, qw.t(), scale_a=sx.view(-1, 1), scale_b=sw.view(1, -1), out_dtype=torch.bfloat16), 20)
-        others["fp8_gemm_8192x14336x4096"]["library_scaled_mm_rowwise_us"] = round(lib_ms * 1e3, 1)
-        others["fp8_gemm_8192x14336x4096"]["library_scaled_mm_rowwise_tflops"] = round(fl / lib_ms / 1e9, 1)
-    except Exception as ex:  # not every torch build exposes it
-        others["fp8_gemm_8192x14336x4096"]["library_scaled_mm_rowwise_us"] = f"unavailable: {str(ex)[:80]}"
-    del xa, w, qx, qw
-    if args.only_rht:
-        print(json.dumps(others))
+    # ---- fp32 fused GEMM -------------------------------------------------------------------------------
+    if want("gemm_f32"):
+        W = torch.randn(M, K, generator=torch.Generator().manual_seed(1)).to(dev)
+        Xt = torch.randn(N, K, generator=torch.Generator().manual_seed(0)).to(dev)
+        gsteps = max(10, min(steps, 50))
+        ms, _ = steady_ms(lambda: hada.fused_ht_gemm(W, Xt), gsteps)
+        tf = flops / ms / 1e9
+        others["fused_ht_gemm_f32"] = {
+            "metric": "fused HT+GEMM TFLOP/s (K=1024, M=N=4096, f32 in/out, fp32 MFMA)",
+            "value": round(tf, 1), "unit": "TFLOP/s", "ms_per_step": round(ms, 6), "steps": gsteps,
+            "algorithmic_flops_per_step": flops,
+            "roofline": roofline("mfma", tf, PEAK_TFLOPS["f32"], "TFLOP/s",
+                                 traffic.get("fused_ht_gemm_f32"))}
+        del W, Xt
+
+    # ---- fused HT+GEMV and its unfused comparator (fwht_gemv_fusion.cu:323-363) ----------------------
+    if want("gemv"):
+        for (m, nn, b) in ((256, 256, 512), (1024, 1024, 8), (1024, 1024, 64), (1024, 1024, 256),
+                           (1024, 1024, 512)):
+            Wg = torch.randn(m, nn, device=dev) / math.sqrt(nn)
+            X = torch.randn(nn, b, device=dev)
+            Xcols = X.t().contiguous()  # untimed layout change for the unfused leg's transform
+
+            def unfused():
+                return torch.matmul(Wg, hada.hadamard_transform(Xcols).t())
+
+            Y = hada.fused_ht_gemv(Wg, X)
+            ref = unfused()
+            gerr = ((Y - ref).abs().max() / ref.abs().max()).item()
+            ms, _ = events_ms(lambda: hada.fused_ht_gemv(Wg, X), 50, 5)
+            ums, _ = events_ms(unfused, 50, 5)
+            byt = 4 * (m * nn + nn * b + m * b)
+            flo = 2 * m * nn * b + int(nn * math.log2(nn) * b)
+            others[f"fused_ht_gemv_M{m}_N{nn}_B{b}"] = {
+                "us": round(ms * 1e3, 2), "unfused_transform_then_library_gemm_us": round(ums * 1e3, 2),
+                "fused_over_unfused_speedup": round(ums / ms, 2),
+                "fused_vs_unfused_max_rel_diff": gerr,
+                "algorithmic_bytes": byt, "algorithmic_flops": flo,
+                "GB/s": round(byt / ms / 1e6, 1), "TFLOP/s": round(flo / ms / 1e9, 3)}
+            del Wg, X, Xcols
+
+    # ---- RHT + FP8 quantize, FP8 GEMM (config 5) -------------------------------------------------------
+    if want("rht"):
+        T, nq, Nw = 8192, 4096, 14336
+        xa = torch.randn(T, nq, generator=torch.Generator().manual_seed(0))
+        outl = torch.randperm(nq, generator=torch.Generator().manual_seed(3))[:41]  # 1 % outlier channels
+        xa[:, outl] *= 50.0
+        xa = xa.to(torch.bfloat16).to(dev)
+        sign = (1 - 2 * torch.randint(0, 2, (nq,), generator=torch.Generator().manual_seed(2))
+                ).to(torch.int8).to(dev)
+        ms, _ = events_ms(lambda: hada.rht_quant_fp8(xa, sign), 50, 3)
+        qbytes = T * nq * 3 + T * 4
+        others["rht_quant_fp8_8192x4096"] = {
+            "us": round(ms * 1e3, 2), "algorithmic_bytes": qbytes,
+            "roofline": roofline("hbm", qbytes / ms / 1e6, HBM_PEAK_GBS, "GB/s",
+                                 traffic.get("rht_quant_fp8_8192x4096"))}
+        qx, sx = hada.rht_quant_fp8(xa, sign)
+        w = (torch.randn(Nw, nq, device=dev) * 0.02).to(torch.bfloat16)
+        qw, sw = hada.rht_quant_fp8(w, sign)
+        ms, _ = steady_ms(lambda: hada.fp8_gemm_rowscale(qx, sx, qw, sw), 20)
+        fl = 2 * T * Nw * nq
+        entry = {"us": round(ms * 1e3, 1), "algorithmic_flops": fl,
+                 "roofline": roofline("mfma", fl / ms / 1e9, PEAK_TFLOPS["fp8"], "TFLOP/s",
+                                      traffic.get("fp8_gemm_8192x14336x4096_l2_fill_plus_write"))}
+        try:  # the vendor library's row-scaled FP8 GEMM on the same operands, for comparison only
+            lib_ms, _ = steady_ms(lambda: torch._scaled_mm(
+                qx, qw.t(), scale_a=sx.view(-1, 1), scale_b=sw.view(1, -1), out_dtype=torch.bfloat16), 20)
+            entry["library_scaled_mm_rowwise_us"] = round(lib_ms * 1e3, 1)
+            entry["library_scaled_mm_rowwise_tflops"] = round(fl / lib_ms / 1e9, 1)
+        except Exception as ex:  # not every torch build exposes it
+            entry["library_scaled_mm_rowwise_us"] = f"unavailable: {str(ex)[:80]}"
+        others["fp8_gemm_8192x14336x4096"] = entry
+        del xa, w, qx, qw
+    if only:
+        print(json.dumps(result if result else others))
         return 0
 
     if args.sweep:
@@ -236,31 +290,22 @@ def main() -> int:
                 nn = 1 << p
                 numel = (128 << 20) // es
                 t = torch.randn(numel // nn, nn, device=dev).to(dt)
-                ms, _ = _events_ms(torch, lambda: hada.hadamard_transform(t, inplace=True), 50, 3)
+                ms, _ = events_ms(lambda: hada.hadamard_transform(t, inplace=True), 50, 3)
                 sweep[f"{dname}_n{nn}"] = {"us": round(ms * 1e3, 2),
                                            "GB/s": round(2 * numel * es / ms / 1e6, 1)}
                 del t
         others["fwht_sweep_128MiB"] = sweep
     result["others"] = others
 
-    # ---- CPU baseline: the reference's truth path on the host cores ---------------------------------
+    # ---- CPU baselines: the reference's truth path on the host cores ----------------------------------
     if not args.no_cpu:
+        import scipy.linalg
+
         import oracle  # CPU restatement: only this leg uses it
 
         nthreads = torch.get_num_threads()
-        sample = 64
-        xs = x_cpu[:sample].clone()
-        oracle.hadamard_matrix_ref(xs)  # builds the matrix, warms the thread pool
-        t0 = time.perf_counter()
-        oracle.hadamard_matrix_ref(xs)
-        est = time.perf_counter() - t0
-        # grow the sample so that the timed region is roughly 10 s of host work
-        sample = int(max(64, min(rows, 64 * (10.0 / max(est, 1e-3)) / 4)))
-        xs = x_cpu[:sample].clone()
-        import scipy.linalg
 
-        H = (torch.tensor(scipy.linalg.hadamard(n), dtype=torch.float32) / math.sqrt(n)).to(torch.bfloat16)
-        def _cpu_median_s(fn, warm=3, reps=10):
+        def cpu_median_s(fn, warm, reps):
             for _ in range(warm):
                 fn()
             ts = []
@@ -270,41 +315,46 @@ def main() -> int:
                 ts.append(time.perf_counter() - t0)
             return sorted(ts)[len(ts) // 2]
 
-        reps = 10
-        dt_s = _cpu_median_s(lambda: xs @ H)
-        # the fused configuration's truth path on the host: W @ (H_K @ X) in fp32
-        Mc = Nc = 4096
-        Kc = 1024
-        Wc = torch.randn(Mc, Kc, generator=torch.Generator().manual_seed(1))
-        Xc = torch.randn(Nc, Kc, generator=torch.Generator().manual_seed(0)).t().contiguous()
-        Hk = torch.tensor(scipy.linalg.hadamard(Kc), dtype=torch.float32) / math.sqrt(Kc)
-        fdt = _cpu_median_s(lambda: Wc @ (Hk @ Xc), warm=2, reps=5)
-        if "fused_ht_gemm" in result:
-            result["fused_ht_gemm"]["cpu_baseline"] = {
-                "value": round(2 * Mc * Nc * Kc / fdt / 1e12, 4), "unit": "TFLOP/s", "cores": nthreads,
-                "kind": "port", "ms": round(fdt * 1e3, 2),
-                "sample": "torch CPU fp32 W @ (H_1024 @ X), whole configuration, matrices built once "
-                          "(untimed), median of 5 after 2 warm-up calls; flops counted as 2MNK"}
+        # fused configuration: W @ (H_K @ X) in fp32, whole configuration
+        Wc = torch.randn(M, K, generator=torch.Generator().manual_seed(1))
+        Xc = torch.randn(N, K, generator=torch.Generator().manual_seed(0)).t().contiguous()
+        Hk = torch.tensor(scipy.linalg.hadamard(K), dtype=torch.float32) / math.sqrt(K)
+        fdt = cpu_median_s(lambda: Wc @ (Hk @ Xc), 2, 5)
+        result["cpu_baseline"] = {
+            "value": round(flops / fdt / 1e12, 4), "unit": "TFLOP/s", "cores": nthreads, "kind": "port",
+            "ms": round(fdt * 1e3, 2),
+            "sample": "torch CPU fp32 W @ (H_1024 @ X), whole configuration, matrices built once "
+                      f"(untimed), median of 5 after 2 warm-up calls; flops counted as 2MNK; os.cpu_count()={os.cpu_count()}"}
         del Wc, Xc, Hk
+
+        # transform: x @ (hadamard(4096)/64) in bf16 on a bounded row sample (~10 s of host work)
+        sample = 64
+        xs = x_cpu[:sample].clone()
+        oracle.hadamard_matrix_ref(xs)  # builds the matrix, warms the thread pool
+        t0 = time.perf_counter()
+        oracle.hadamard_matrix_ref(xs)
+        est = time.perf_counter() - t0
+        sample = int(max(64, min(rows, 64 * (10.0 / max(est, 1e-3)) / 13)))
+        xs = x_cpu[:sample].clone()
+        H = (torch.tensor(scipy.linalg.hadamard(n), dtype=torch.float32) / math.sqrt(n)).to(torch.bfloat16)
+        dt_s = cpu_median_s(lambda: xs @ H, 3, 10)
         # the C restatement's O(n log n) butterfly on one core, over the whole batch (under a second)
-        bsample = rows
-        xb = x_cpu[:bsample].float().numpy()
+        xb = x_cpu.float().numpy()
         oracle.fwht_f32(xb[:64])
         t0 = time.perf_counter()
         oracle.fwht_f32(xb)
         bdt = time.perf_counter() - t0
-        butterfly = {"value": round(2 * bsample * n * 2 / bdt / 1e9, 4), "unit": "GB/s", "cores": 1,
-                     "sample": f"oracle_fwht_f32 (plain C butterfly, fp32) on all {bsample} rows; "
-                               "bytes counted at the workload's 2 B per element",
-                     "ms_for_sample": round(bdt * 1e3, 3)}
-        result["cpu_baseline"] = {
+        result["fwht"]["cpu_baseline"] = {
             "value": round(2 * sample * n * 2 / dt_s / 1e9, 4), "unit": "GB/s", "cores": nthreads,
             "kind": "port",
             "sample": f"torch CPU x @ (hadamard(4096)/64).to(bf16) on the first {sample} of 16384 rows "
-                      f"(matrix built once, untimed), median of {reps} calls after 3 warm-up calls; os.cpu_count()={os.cpu_count()}",
+                      "(matrix built once, untimed), median of 10 calls after 3 warm-up calls",
             "ms_for_sample": round(dt_s * 1e3, 3),
             "ms_extrapolated_full_batch": round(dt_s * 1e3 * rows / sample, 1),
-            "butterfly_port": butterfly}
+            "butterfly_port": {"value": round(2 * rows * n * 2 / bdt / 1e9, 4), "unit": "GB/s", "cores": 1,
+                               "sample": f"oracle_fwht_f32 (plain C butterfly, fp32) on all {rows} rows; "
+                                         "bytes counted at the workload's 2 B per element",
+                               "ms_for_sample": round(bdt * 1e3, 3)}}
 
     print(json.dumps(result))
     return 0
