@@ -379,7 +379,7 @@ int launch_gemm16(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N
                   int out_f32, float scale, hipStream_t s)
 {
     const uint32_t logK = ilog2(K);
-    const int shift = tile_stage_shift<2>(logK);
+    const int shift = tile_stage_shift<2>(logK, kNarrowRange<T16>);
     const float fscale = (float)((double)scale * (double)(1u << shift));
     const uint32_t n_tiles = (N + BN - 1) / BN;
     // split M so that about one workgroup per compute unit exists; each covers a multiple of

@@ -170,7 +170,7 @@ int launch(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, ui
            float scale, hipStream_t s)
 {
     const uint32_t logK = ilog2(K);
-    const int shift = tile_stage_shift<4>(logK);
+    const int shift = tile_stage_shift<4>(logK, false);
     const float fscale = (float)((double)scale * (double)(1u << shift));
     const uint32_t n_tiles = (N + BN - 1) / BN;
     const uint32_t row_blocks = (M + 511u) / 512u;

@@ -509,7 +509,7 @@ template <class T16, int K, bool OUT_F32>
 int launch_as(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, float scale,
               uint32_t mpx, hipStream_t s)
 {
-    const OutputScale os = split_output_scale((double)scale, tile_stage_shift<2>(10));
+    const OutputScale os = split_output_scale((double)scale, tile_stage_shift<2>(10, kNarrowRange<T16>));
     const Plan p = plan(M, N);
     auto kern = fused_ht_gemm_xreg_kernel<T16, K, OUT_F32>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),

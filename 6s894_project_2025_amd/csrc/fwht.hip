@@ -67,6 +67,8 @@ fwht_reg_kernel(const void* in, void* out, uint64_t total, uint64_t num_steps, u
 }
 
 // ---- LDS kernel: one workgroup of W = 2^LW wavefronts per row of n = 4096 * W ----------------
+// (Persistent workgroups that prefetch their next row before the exchange were measured slower
+// than one short-lived workgroup per row on tensors beyond the last-level cache.)
 template <class IO, int LW, bool MUL, bool TWO_PHASE>
 __global__ void __launch_bounds__(64 << LW)
 fwht_lds_kernel(const void* in, void* out, uint64_t rows, int exp2, float mult)
@@ -90,7 +92,9 @@ int launch_reg(const void* in, void* out, uint64_t total, uint64_t num_steps, ui
     // Up to four steps per wavefront once every compute unit has a full set of wavefronts: the
     // operand set-up is paid once and the next row's loads overlap the current row's arithmetic.
     // Beyond the 256 MiB Infinity Cache the transform is DRAM-bound, and there one step per
-    // (short-lived) wavefront measured 2 - 4 % faster: the sweep through memory stays in order.
+    // (short-lived) wavefront measured 2 - 4 % faster (the sweep through memory stays in order)
+    // and non-temporal loads and stores another 5 - 13 % (lines that are never touched again
+    // stay out of the caches).
     uint64_t waves = num_steps;
     const uint64_t resident = 256u * 16u;
     const uint64_t per_wave = total * (uint64_t)IO::ESIZE > (256ull << 20) ? 1u : 4u;
@@ -99,12 +103,12 @@ int launch_reg(const void* in, void* out, uint64_t total, uint64_t num_steps, ui
                                                                   : resident;
     const uint64_t blocks = (waves + 3u) / 4u;
     if (blocks > 0x7fffffffull) return MI_ERR_SHAPE;
-    if (os.mult == 1.0f)
-        hipLaunchKernelGGL((fwht_reg_kernel<IO, NT, XB, false>), dim3((uint32_t)blocks), dim3(256), 0,
-                           s, in, out, total, num_steps, p, os.exp2, os.mult);
-    else
-        hipLaunchKernelGGL((fwht_reg_kernel<IO, NT, XB, true>), dim3((uint32_t)blocks), dim3(256), 0,
-                           s, in, out, total, num_steps, p, os.exp2, os.mult);
+    using IOB = typename IO::Streaming;
+    const bool big = total * (uint64_t)IO::ESIZE > (256ull << 20);
+    auto kern = big ? (os.mult == 1.0f ? fwht_reg_kernel<IOB, NT, XB, false> : fwht_reg_kernel<IOB, NT, XB, true>)
+                    : (os.mult == 1.0f ? fwht_reg_kernel<IO, NT, XB, false> : fwht_reg_kernel<IO, NT, XB, true>);
+    hipLaunchKernelGGL(kern, dim3((uint32_t)blocks), dim3(256), 0, s, in, out, total, num_steps, p,
+                       os.exp2, os.mult);
     return launch_status();
 }
 
@@ -130,10 +134,13 @@ int launch_lds(const void* in, void* out, uint64_t rows, OutputScale os, hipStre
     if (rows == 0) return MI_OK;
     if (rows > 0x7fffffffull) return MI_ERR_SHAPE;
     // While the tensor fits the 256 MiB Infinity Cache, occupancy decides (exchange in two
-    // phases, half the LDS); once it is DRAM-bound, the single exchange with fewer resident
-    // workgroups measured 3 - 5 % faster.
+    // phases, half the LDS).  Once it is DRAM-bound, non-temporal accesses gain 5 - 10 %; with
+    // them the single exchange is the faster one for n = 8192 and 16384, the two-phase exchange
+    // (two workgroups per compute unit) for n = 32768, where a single-exchange workgroup fills
+    // the LDS alone and streaming loads then measured slower than ordinary ones.
     const uint64_t bytes = (rows << (12 + LW)) * (uint64_t)IO::ESIZE;
-    if (bytes > (256ull << 20)) return launch_lds_as<IO, LW, false>(in, out, rows, os, s);
+    if (bytes > (256ull << 20))
+        return launch_lds_as<typename IO::Streaming, LW, LW == 3>(in, out, rows, os, s);
     return launch_lds_as<IO, LW, true>(in, out, rows, os, s);
 }
 
@@ -142,7 +149,7 @@ int dispatch(const void* in, void* out, uint64_t rows, uint32_t n, float scale, 
 {
     const uint32_t p = ilog2(n);
     const uint64_t total = rows * (uint64_t)n;
-    const OutputScale os = split_output_scale((double)scale, tile_stage_shift<IO::ESIZE>(p));
+    const OutputScale os = split_output_scale((double)scale, tile_stage_shift<IO::ESIZE>(p, kNarrowRange<typename IO::T16>));
     if (p <= 9) {
         const uint64_t tiles = (total + 511u) / 512u;
         // several independent tiles per step once there is enough work to fill the chip

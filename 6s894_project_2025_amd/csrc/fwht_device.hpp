@@ -24,6 +24,8 @@
 // caller folds the inverse into its output scale (tile_stage_shift, split_output_scale).
 #pragma once
 
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace mi {
@@ -83,14 +85,27 @@ inline OutputScale split_output_scale(double scale, int stage_shift)
     return r;
 }
 
+// log2 of the attenuation of stage 1 over k index bits.  bf16 operands: 2^-(k/2), the square root
+// of the stage's gain.  fp16 operands (`narrow_range`): 2^-(k-1), so that the 16-bit value between
+// the stages, a sum of 2^k inputs, never exceeds twice the largest input; with the square-root
+// factor an input pattern that the full transform spreads out could already overflow fp16 there
+// (partial sums up to 8x the largest input at k = 5).
+__host__ __device__ inline int stage1_shift(int k, bool narrow_range)
+{
+    return narrow_range && k > 1 ? k - 1 : k >> 1;
+}
+
 // log2 of the (power-of-two) attenuation the two MFMA stages apply for a transform of length 2^p.
+// `narrow_range`: the matrix-core operand type is fp16 (see stage1_shift).
 template <int ESIZE>
-__host__ __device__ inline int tile_stage_shift(uint32_t p)
+__host__ __device__ inline int tile_stage_shift(uint32_t p, bool narrow_range)
 {
     uint32_t m1, m2;
     tile_masks<ESIZE>(p, m1, m2);
-    return (__builtin_popcount(m1) >> 1) + (__builtin_popcount(m2) >> 1);
+    return stage1_shift(__builtin_popcount(m1), narrow_range) + (__builtin_popcount(m2) >> 1);
 }
+template <class T16>
+constexpr bool kNarrowRange = std::is_same<T16, F16>::value;
 
 // Per-lane Hadamard operands for the two stages.
 template <class T16>
@@ -109,7 +124,7 @@ __device__ __forceinline__ void make_tile_operands(uint32_t p, TileOperands<T16>
     const uint32_t lo = lane & 15u, hi = lane >> 4;
     uint32_t mask1, mask2;
     tile_masks<ESIZE>(p, mask1, mask2);
-    const float c1 = __builtin_ldexpf(1.0f, -(__popc(mask1) >> 1));
+    const float c1 = __builtin_ldexpf(1.0f, -stage1_shift(__popc(mask1), kNarrowRange<T16>));
     const float c2 = __builtin_ldexpf(1.0f, exp2 - (__popc(mask2) >> 1));
 #pragma unroll
     for (int t = 0; t < 2; ++t) {

@@ -30,8 +30,11 @@ namespace mi {
 // Each IO policy loads a lane's share of one tile into MFMA input form and stores two f32x4
 // accumulators back, both guarded against the end of the buffer (`total` elements).
 
-template <class T16_>
+// STREAM = true marks every access non-temporal: for tensors that do not fit the last-level
+// cache, where keeping lines that are never touched again only costs bandwidth.
+template <class T16_, bool STREAM = false>
 struct Io16 {
+    using Streaming = Io16<T16_, true>;
     using T16 = T16_;
     using E = typename T16::E;
     using Elem = E;
@@ -47,7 +50,10 @@ struct Io16 {
         const uint64_t off = tile * 512u + 8u * (threadIdx.x & 63u);
         In in;
         if (!GUARD || off + 8u <= total) {
-            in.a = *reinterpret_cast<const typename T16::V8*>(p + off);
+            if (STREAM)
+                in.a = __builtin_nontemporal_load(reinterpret_cast<const typename T16::V8*>(p + off));
+            else
+                in.a = *reinterpret_cast<const typename T16::V8*>(p + off);
         } else {
 #pragma unroll
             for (int j = 0; j < 8; ++j) in.a[j] = (off + j < total) ? p[off + j] : (E)0.0f;
@@ -73,7 +79,10 @@ struct Io16 {
 #pragma unroll
             for (int r = 0; r < 4; ++r) o[4 * t + r] = (E)(MUL ? acc[t][r] * s : acc[t][r]);
         if (!GUARD || off + 8u <= total) {
-            *reinterpret_cast<typename T16::V8*>(p + off) = o;
+            if (STREAM)
+                __builtin_nontemporal_store(o, reinterpret_cast<typename T16::V8*>(p + off));
+            else
+                *reinterpret_cast<typename T16::V8*>(p + off) = o;
         } else {
 #pragma unroll
             for (int j = 0; j < 8; ++j)
@@ -82,7 +91,9 @@ struct Io16 {
     }
 };
 
-struct Io32 {
+template <bool STREAM = false>
+struct Io32T {
+    using Streaming = Io32T<true>;
     using T16 = BF16;  // matrix-core type used for the three-piece products
     using Elem = float;
     static constexpr int ESIZE = 4;
@@ -99,7 +110,8 @@ struct Io32 {
         for (int t = 0; t < 2; ++t) {
             const uint64_t off = tile * 512u + 256u * t + 4u * (threadIdx.x & 63u);
             if (!GUARD || off + 4u <= total) {
-                const f32x4 q = *reinterpret_cast<const f32x4*>(p + off);
+                const f32x4 q = STREAM ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p + off))
+                                       : *reinterpret_cast<const f32x4*>(p + off);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) in.v[4 * t + r] = q[r];
             } else {
@@ -126,7 +138,10 @@ struct Io32 {
             const uint64_t off = tile * 512u + 256u * t + 4u * (threadIdx.x & 63u);
             const f32x4 o = MUL ? acc[t] * s : acc[t];
             if (!GUARD || off + 4u <= total) {
-                *reinterpret_cast<f32x4*>(p + off) = o;
+                if (STREAM)
+                    __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(p + off));
+                else
+                    *reinterpret_cast<f32x4*>(p + off) = o;
             } else {
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
@@ -135,6 +150,8 @@ struct Io32 {
         }
     }
 };
+
+using Io32 = Io32T<false>;
 
 // ---- wavefront level: NT tiles of 512 elements, XB cross-tile bits ---------------------------------
 // One step = tiles [step*NT, step*NT + NT) of the buffer = one row when XB > 0, several short rows
@@ -183,24 +200,28 @@ __device__ __forceinline__ void wave_fwht_step(const void* in, void* out, uint64
 // it owns, runs the LW remaining butterflies in registers and stores.  `xch` holds
 // 16 * 64 * 8 * W bytes (TWO_PHASE: the two accumulator halves take turns) or twice that (one
 // exchange); all 64*W threads must call (__syncthreads inside).
+template <class IO>
+__device__ __forceinline__ void block_fwht_load(const void* in, uint64_t tile0, uint64_t total,
+                                                typename IO::In (&tin)[8])
+{
+    const uint32_t w = threadIdx.x >> 6;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) tin[c] = IO::template load<false>(in, tile0 + w * 8u + c, total);
+}
+
 template <class IO, int LW, bool MUL, bool TWO_PHASE = true>
-__device__ __forceinline__ void block_fwht_row(const void* in, void* out, uint64_t tile0,
-                                               uint64_t total, f32x4* xch,
-                                               const TileOperands<typename IO::T16>& ops, float mult)
+__device__ __forceinline__ void block_fwht_finish(const typename IO::In (&tin)[8], void* out,
+                                                  uint64_t tile0, uint64_t total, f32x4* xch,
+                                                  const TileOperands<typename IO::T16>& ops, float mult)
 {
     constexpr int W = 1 << LW;
     constexpr int OWN = 8 / W;  // tiles per sub-row owned by a wavefront in pass 2
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t w = threadIdx.x >> 6;
     f32x4 acc[8][2];
-    {
-        typename IO::In tin[8];
 #pragma unroll
-        for (int c = 0; c < 8; ++c) tin[c] = IO::template load<false>(in, tile0 + w * 8u + c, total);
-#pragma unroll
-        for (int c = 0; c < 8; ++c) IO::transform(tin[c], ops, acc[c]);
-        cross_tile_butterflies<8, 3>(acc);
-    }
+    for (int c = 0; c < 8; ++c) IO::transform(tin[c], ops, acc[c]);
+    cross_tile_butterflies<8, 3>(acc);
     f32x4 g[W * OWN][2];  // index s * OWN + c'
     if constexpr (TWO_PHASE) {
         // xch layout: [W sub-rows][8 tiles][64 lanes], used twice (once per accumulator half):
@@ -257,11 +278,21 @@ __device__ __forceinline__ void block_fwht_row(const void* in, void* out, uint64
                                            g[s * OWN + cc], mult);
 }
 
+template <class IO, int LW, bool MUL, bool TWO_PHASE = true>
+__device__ __forceinline__ void block_fwht_row(const void* in, void* out, uint64_t tile0,
+                                               uint64_t total, f32x4* xch,
+                                               const TileOperands<typename IO::T16>& ops, float mult)
+{
+    typename IO::In tin[8];
+    block_fwht_load<IO>(in, tile0, total, tin);
+    block_fwht_finish<IO, LW, MUL, TWO_PHASE>(tin, out, tile0, total, xch, ops, mult);
+}
+
 // Host side: the (exp2, mult) pair for a transform of length 2^LOG_N with output factor `scale`.
 template <class IO, int LOG_N>
 inline OutputScale output_scale(double scale)
 {
-    return split_output_scale(scale, tile_stage_shift<IO::ESIZE>(LOG_N));
+    return split_output_scale(scale, tile_stage_shift<IO::ESIZE>(LOG_N, kNarrowRange<typename IO::T16>));
 }
 
 template <class IO_, int LOG_N>

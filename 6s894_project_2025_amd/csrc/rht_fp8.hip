@@ -204,7 +204,7 @@ extern "C" int mi_rht_quant_fp8(const void* x, const int8_t* sign, void* q, floa
         return MI_ERR_ALIGN;
     const uint32_t p = ilog2(n);
     const uint64_t total = T * (uint64_t)n;
-    const OutputScale os = split_output_scale((double)scale, tile_stage_shift<2>(p));
+    const OutputScale os = split_output_scale((double)scale, tile_stage_shift<2>(p, false));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (p <= 9) {
         const uint64_t tiles = (total + 511u) / 512u;

@@ -271,3 +271,33 @@ def test_beyond_infinity_cache_variants(pkg, oracle, n, dt):
     torch.cuda.synchronize()
     tol_abs = 1e-4 if dt == torch.float32 else (0.1 if dt == torch.bfloat16 else 2e-2)
     assert (z.float() - x.float()).abs().max().item() <= tol_abs
+
+
+def test_fp16_large_inputs_do_not_overflow_between_stages(pkg, oracle):
+    # 32 equal inputs of 2e4 on exactly the index bits the first matrix-core stage sums over
+    # (element bits 0, 1, 2, 7, 8): the 16-bit value between the stages is 32 x 2e4 x (stage-1
+    # factor).  With a square-root factor (1/4) that is 1.6e5, beyond fp16; the transform keeps it
+    # within twice the largest input.  The normalised result, +-1e4 on 128 outputs, is representable.
+    n = 4096
+    rows = 6
+    x = torch.zeros(rows, n, dtype=torch.float16)
+    group = [b0 + 2 * b1 + 4 * b2 + 128 * b7 + 256 * b8
+             for b0 in (0, 1) for b1 in (0, 1) for b2 in (0, 1) for b7 in (0, 1) for b8 in (0, 1)]
+    g = torch.Generator().manual_seed(5)
+    for r in range(rows):
+        base = int(torch.randint(0, 16, (1,), generator=g)) * 8 + int(torch.randint(0, 8, (1,), generator=g)) * 512
+        sign = 1.0 if r % 2 == 0 else -1.0
+        x[r, [base + e for e in group]] = sign * 2.0e4
+    x[rows - 1] += (torch.randn(n, generator=g) * 100).to(torch.float16)  # plus ordinary data
+    y = pkg.hadamard_transform(x.cuda())
+    torch.cuda.synchronize()
+    assert torch.isfinite(y).all()
+    want = oracle.fwht_f64(x.double().numpy())
+    assert np.abs(want).max() < 6.0e4
+    assert oracle.rel_err(y.cpu().double().numpy(), want) <= 2e-2
+    # the same guarantee for every length with a full first stage, and for tiny inputs the
+    # stronger factor must not cost accuracy
+    for nn in (32, 256, 1024, 32768):
+        small = (torch.randn(8, nn, generator=g) * 1e-3).to(torch.float16)
+        ys = pkg.hadamard_transform(small.cuda())
+        assert oracle.rel_err(ys.cpu().double().numpy(), oracle.fwht_f64(small.double().numpy())) <= 2e-2
