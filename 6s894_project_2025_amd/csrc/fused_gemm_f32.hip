@@ -23,12 +23,18 @@ __device__ __forceinline__ uint32_t y_off(uint32_t n, uint32_t q, uint32_t col_b
     return (n * (col_bytes >> 4) + (q ^ ((n >> LOG_NB) & swz_mask))) << 4;
 }
 
-template <int BN, int XB>
+// HALVES = 2 (K = 4096, whose fp32 tile does not fit in LDS): H_K = [[H, H], [H, -H]] with
+// H = H_{K/2}, so the kernel runs twice over half the K range, first with
+// Y = H (X_lo + X_hi) against W[:, :K/2], then with Y = H (X_lo - X_hi) against W[:, K/2:], the
+// accumulators staying in registers in between.  Each wavefront then owns exactly one 64-row
+// block (the launcher gives such workgroups 512 rows).
+template <int BN, int XB, int HALVES>
 __global__ void __launch_bounds__(kThreads)
 fused_ht_gemm_f32_kernel(const float* __restrict__ W, const float* __restrict__ Xt,
-                         float* __restrict__ C, uint32_t M, uint32_t N, uint32_t K, uint32_t logK,
-                         uint32_t m_per_block, float fscale)
+                         float* __restrict__ C, uint32_t M, uint32_t N, uint32_t K_full,
+                         uint32_t logK_full, uint32_t m_per_block, float fscale)
 {
+    const uint32_t K = K_full / HALVES, logK = logK_full - (HALVES == 2 ? 1u : 0u);
     constexpr int NB = BN / 16;
     constexpr int LOG_NB = NB == 4 ? 2 : (NB == 2 ? 1 : 0);
     extern __shared__ __attribute__((aligned(16))) unsigned char ylds[];
@@ -40,22 +46,41 @@ fused_ht_gemm_f32_kernel(const float* __restrict__ W, const float* __restrict__ 
     const uint32_t swz_mask = (chunks_per_col >= 16u ? 16u : chunks_per_col) - 1u;
     const uint32_t col_bytes = K * 4u;
 
+    // staging layout: row r (64 bytes), 16-byte chunk c stored at position c ^ ((r >> 1) & 3)
+    // (conflict-free for both the writer's and the reader's lane order)
+    unsigned char* stage = ylds + (size_t)BN * K * 4u + wave * kStageBytes;
+    const uint32_t wr_off = (lane >> 2) * 64u + (((lane & 3u) ^ ((lane >> 3) & 3u)) << 4);
+    const uint32_t rd_off = lo * 64u + ((hi ^ ((lo >> 1) & 3u)) << 4);
+
+    const uint32_t m_begin = blockIdx.y * m_per_block;
+    const uint32_t m_end = min(M, m_begin + m_per_block);
+    const uint32_t ksteps = K >> 4;
+    f32x4 acc[NB][4];
+
+#pragma unroll 1
+    for (int half = 0; half < HALVES; ++half) {
+    if (half) __syncthreads();  // every wavefront is done with the first half's tile
     {
         TileOperands<BF16> ops;
         make_tile_operands<BF16, 4>(logK, ops);
         constexpr int NT = 1 << XB;
         const uint32_t block_tiles = (BN * K) >> 9;
-        const uint64_t total = (uint64_t)N * K;
-        const uint64_t tile_base = ((uint64_t)n0 * K) >> 9;
+        const uint64_t total = (uint64_t)N * K_full;
         for (uint32_t t0 = wave * NT; t0 < block_tiles; t0 += kWaves * NT) {
             float in[NT][8];
 #pragma unroll
             for (int c = 0; c < NT; ++c)
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
-                    const uint64_t off = (tile_base + t0 + c) * 512u + 256u * t + 4u * lane;
+                    // element e of the block's transformed tile: column e >> logK, k = e % K
+                    const uint32_t e = (t0 + c) * 512u + 256u * t + 4u * lane;
+                    const uint64_t off = (uint64_t)(n0 + (e >> logK)) * K_full + (e & (K - 1u));
                     f32x4 q = {0.f, 0.f, 0.f, 0.f};
                     if (off + 4u <= total) q = *reinterpret_cast<const f32x4*>(Xt + off);
+                    if (HALVES == 2 && off + K + 4u <= total) {
+                        const f32x4 u = *reinterpret_cast<const f32x4*>(Xt + off + K);
+                        q = half ? q - u : q + u;
+                    }
 #pragma unroll
                     for (int r = 0; r < 4; ++r) in[c][4 * t + r] = q[r];
                 }
@@ -76,22 +101,13 @@ fused_ht_gemm_f32_kernel(const float* __restrict__ W, const float* __restrict__ 
     }
     __syncthreads();
 
-    // staging layout: row r (64 bytes), 16-byte chunk c stored at position c ^ ((r >> 1) & 3)
-    // (conflict-free for both the writer's and the reader's lane order)
-    unsigned char* stage = ylds + (size_t)BN * K * 4u + wave * kStageBytes;
-    const uint32_t wr_off = (lane >> 2) * 64u + (((lane & 3u) ^ ((lane >> 3) & 3u)) << 4);
-    const uint32_t rd_off = lo * 64u + ((hi ^ ((lo >> 1) & 3u)) << 4);
-
-    const uint32_t m_begin = blockIdx.y * m_per_block;
-    const uint32_t m_end = min(M, m_begin + m_per_block);
-    const uint32_t ksteps = K >> 4;
-
     for (uint32_t mb = m_begin + wave * 64u; mb < m_end; mb += kWaves * 64u) {
-        f32x4 acc[NB][4];
+        if (half == 0) {
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
+            for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-            for (int mi = 0; mi < 4; ++mi) acc[nb][mi] = f32x4{0.f, 0.f, 0.f, 0.f};
+                for (int mi = 0; mi < 4; ++mi) acc[nb][mi] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
         // W goes global -> registers with four adjacent lanes on the 64 contiguous bytes a row
         // contributes to a K step (the pattern the L1 coalesces; one lane per row, which is what
         // the MFMA operand wants, runs at a third of the rate), then through a wavefront-private
@@ -102,7 +118,7 @@ fused_ht_gemm_f32_kernel(const float* __restrict__ W, const float* __restrict__ 
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
             const uint32_t m = min(mb + 16u * mi + (lane >> 2), M - 1u);
-            wsrc[mi] = W + (uint64_t)m * K + 4u * (lane & 3u);
+            wsrc[mi] = W + (uint64_t)m * K_full + (uint32_t)half * K + 4u * (lane & 3u);
         }
         // Software pipeline: while step kk is multiplied, the fragments of step kk+1 are already
         // on their way out of LDS and the W pieces of step kk+2 are in flight from memory.
@@ -148,6 +164,7 @@ fused_ht_gemm_f32_kernel(const float* __restrict__ W, const float* __restrict__ 
                                                                            acc[nb][mi], 0, 0, 0);
         }
 
+        if (half + 1 < HALVES) continue;  // the second half adds to the same accumulators
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
             const uint32_t m = mb + 16u * mi + lo;
@@ -163,14 +180,15 @@ fused_ht_gemm_f32_kernel(const float* __restrict__ W, const float* __restrict__ 
                     if ((uint32_t)(NB * r + nb) < ncols) p[NB * r + nb] = acc[nb][mi][r];
         }
     }
+    }  // half
 }
 
-template <int BN, int XB>
+template <int BN, int XB, int HALVES = 1>
 int launch(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, uint32_t K,
            float scale, hipStream_t s)
 {
     const uint32_t logK = ilog2(K);
-    const int shift = tile_stage_shift<4>(logK, false);
+    const int shift = tile_stage_shift<4>(logK - (HALVES == 2 ? 1u : 0u), false);
     const float fscale = (float)((double)scale * (double)(1u << shift));
     const uint32_t n_tiles = (N + BN - 1) / BN;
     const uint32_t row_blocks = (M + 511u) / 512u;
@@ -178,10 +196,11 @@ int launch(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, ui
     uint32_t msplit = (256u + n_tiles - 1u) / n_tiles;
     if (msplit < 1u) msplit = 1u;
     if (msplit > row_blocks) msplit = row_blocks;
-    const uint32_t m_per_block = ((row_blocks + msplit - 1u) / msplit) * 512u;
+    uint32_t m_per_block = ((row_blocks + msplit - 1u) / msplit) * 512u;
+    if (HALVES == 2) m_per_block = 512u;  // one row block per wavefront: accumulators stay put
     msplit = (M + m_per_block - 1u) / m_per_block;
-    const size_t lds = (size_t)BN * K * 4u + (size_t)kWaves * kStageBytes;
-    auto kern = fused_ht_gemm_f32_kernel<BN, XB>;
+    const size_t lds = (size_t)BN * (K / HALVES) * 4u + (size_t)kWaves * kStageBytes;
+    auto kern = fused_ht_gemm_f32_kernel<BN, XB, HALVES>;
     if (lds > 64u * 1024u) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -205,7 +224,8 @@ int fused_gemm_f32(const float* W, const float* Xt, float* C, uint32_t M, uint32
         case 512: return launch<32, 0>(W, Xt, C, M, N, K, scale, s);
         case 1024: return launch<32, 1>(W, Xt, C, M, N, K, scale, s);
         case 2048: return launch<16, 2>(W, Xt, C, M, N, K, scale, s);
-        default: return MI_ERR_SIZE;  // fp32 tile of K = 4096 does not fit in LDS
+        case 4096: return launch<16, 2, 2>(W, Xt, C, M, N, K, scale, s);  // two passes of K = 2048
+        default: return MI_ERR_SIZE;
     }
 }
 

@@ -92,8 +92,7 @@ int mi_fused_ht_gemv(const void* W, const void* X, void* Y, uint32_t M, uint32_t
  *
  *   in_dtype  : MI_F32 (fp32 MFMA) or MI_BF16 / MI_F16 (16-bit MFMA, fp32 accumulate).
  *   out_dtype : MI_F32, or the same 16-bit type as in_dtype.
- *   K : power of two, 32 <= K <= 4096 (MI_F32: K <= 2048, the fp32 tile of K = 4096 does not fit
- *   in LDS).   M, N >= 1 (edge tiles are masked).
+ *   K : power of two, 32 <= K <= 4096.   M, N >= 1 (edge tiles are masked).
  */
 int mi_fused_ht_gemm(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
                      int in_dtype, int out_dtype, float scale, void* stream);

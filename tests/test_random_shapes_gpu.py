@@ -50,7 +50,7 @@ def test_gemm_random_shapes(pkg, oracle):
     rnd = random.Random(103)
     for case in range(30):
         dt = rnd.choice(DTYPES)
-        K = 1 << rnd.randint(5, 11 if dt == torch.float32 else 12)
+        K = 1 << rnd.randint(5, 12)
         M = rnd.randint(1, 600)
         N = rnd.randint(1, 400)
         W, Xt = oracle.inputs_gemm(M, N, K, dt)
