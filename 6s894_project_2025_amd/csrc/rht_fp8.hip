@@ -102,27 +102,24 @@ rht_quant_fp8_kernel(const __bf16* __restrict__ x, const int8_t* __restrict__ si
         for (int c = 0; c < NT; ++c) tile_transform<BF16>(in[c], ops, acc[c]);
         cross_tile_butterflies<NT, XB>(acc);
 
-        // round to bf16 (the pre-quant values); amax per row on the packed magnitudes (bf16 bit
-        // patterns without the sign order like unsigned integers)
+        // round to bf16 (the pre-quant values).  Rounding is monotonic, so the row maximum of the
+        // rounded magnitudes is the rounded maximum of the fp32 magnitudes: one v_max3 per two
+        // values, one rounding per row.
         bf16x8 y[NT];
         float amax[NT];
 #pragma unroll
         for (int c = 0; c < NT; ++c) {
+            float m = 0.0f;
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            for (int t = 0; t < 2; ++t) {
+                f32x4 v = acc[c][t];
+                if (MUL) v = v * mult;
 #pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    y[c][4 * t + r] = (__bf16)(MUL ? acc[c][t][r] * mult : acc[c][t][r]);
-            const u32x4 yb = __builtin_bit_cast(u32x4, y[c]);
-            typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
-            u16x2 m = {0, 0};
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                const u16x2 mag = __builtin_bit_cast(u16x2, yb[w] & 0x7fff7fffu);
-                m = __builtin_elementwise_max(m, mag);
+                for (int r = 0; r < 4; ++r) y[c][4 * t + r] = (__bf16)v[r];
+                m = fmaxf(fmaxf(__builtin_fabsf(v[0]), __builtin_fabsf(v[1])), m);
+                m = fmaxf(fmaxf(__builtin_fabsf(v[2]), __builtin_fabsf(v[3])), m);
             }
-            const uint32_t top = m[0] > m[1] ? m[0] : m[1];
-            amax[c] = __builtin_bit_cast(float, top << 16);
+            amax[c] = m;
         }
         if (XB > 0) {  // one row spans all NT tiles: fold the tiles, then one lane reduction
             float m = amax[0];
@@ -136,11 +133,12 @@ rht_quant_fp8_kernel(const __bf16* __restrict__ x, const int8_t* __restrict__ si
             for (int c = 0; c < NT; ++c) amax[c] = lane_max(amax[c], row_lane_bits);
         }
 
+        u32x2 codes[NT];
 #pragma unroll
         for (int c = 0; c < NT; ++c) {
             const uint64_t off = (step * NT + c) * 512u + 8u * lane;
             if (XB == 0 && off + 8u > total) continue;  // XB > 0: whole rows
-            const float a = fmaxf(amax[c], kAmaxFloor);
+            const float a = fmaxf((float)(__bf16)amax[c], kAmaxFloor);
             const float inv = kFp8Max / a;
             // first lane of each row writes the dequantisation factor
             const bool row_head = XB > 0 ? (c == 0 && lane == 0) : ((off & (uint64_t)(n - 1u)) == 0);
@@ -148,7 +146,6 @@ rht_quant_fp8_kernel(const __bf16* __restrict__ x, const int8_t* __restrict__ si
             // |y| <= amax, so y * inv <= 448 * (1 + 2^-23): always inside the round-to-448 interval
             // and the +-448 clamp of the stated convention never changes a finite value; omitted.
             const u32x4 yb = __builtin_bit_cast(u32x4, y[c]);
-            u32x2 codes;
 #pragma unroll
             for (int w = 0; w < 2; ++w) {
                 float v[4];
@@ -159,10 +156,30 @@ rht_quant_fp8_kernel(const __bf16* __restrict__ x, const int8_t* __restrict__ si
                 }
                 int pk = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
                 pk = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], pk, true);
-                codes[w] = (uint32_t)pk;
+                codes[c][w] = (uint32_t)pk;
             }
-            __builtin_nontemporal_store(codes, reinterpret_cast<u32x2*>(q + off));  // streaming output
+            if (XB == 0) __builtin_nontemporal_store(codes[c], reinterpret_cast<u32x2*>(q + off));
             if (y_out) *reinterpret_cast<bf16x8*>(y_out + off) = y[c];
+        }
+        if constexpr (XB > 0) {
+            // Whole rows: neighbouring lanes trade 8 codes so that the even lane stores 16
+            // consecutive bytes of tile c and the odd lane 16 of tile c+1: half as many store
+            // instructions, each covering two 512-byte runs.  (Streaming stores: the codes are
+            // not read again here.)
+            const bool odd = lane & 1u;
+#pragma unroll
+            for (int c = 0; c < NT; c += 2) {
+                u32x2 give, got;
+#pragma unroll
+                for (int w = 0; w < 2; ++w) {
+                    give[w] = odd ? codes[c][w] : codes[c + 1][w];
+                    got[w] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)give[w], 0xB1, 0xf, 0xf, false);
+                }
+                const u32x4 out = odd ? u32x4{got[0], got[1], codes[c + 1][0], codes[c + 1][1]}
+                                      : u32x4{codes[c][0], codes[c][1], got[0], got[1]};
+                const uint64_t at = (step * NT + c + (odd ? 1u : 0u)) * 512u + 16u * (lane >> 1);
+                __builtin_nontemporal_store(out, reinterpret_cast<u32x4*>(q + at));
+            }
         }
     }
 }
