@@ -221,15 +221,11 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     if (m_begin >= M || n0 >= N) return;  // workgroup-uniform, before any barrier
     const uint32_t m_end = min(M, m_begin + m_per_block);
     const uint32_t nrb = (m_end - m_begin + kRows - 1u) / kRows;
-    // workgroups that share a slice of W start at different row blocks, so that they do not all
-    // ask the L2 for the same lines at the same moment
-    // (a slice whose last block is partial keeps its order, so that the partial block comes last)
-    const uint32_t rb0 = (m_end - m_begin) % kRows ? 0u : cg % nrb;
-    auto row_block = [&](uint32_t rbi) __attribute__((always_inline)) {  // the rbi-th row block this workgroup visits
-        uint32_t rb = rb0 + rbi;  // rbi <= nrb, rb0 < nrb
-        if (rb >= nrb) rb -= nrb;
-        if (rb >= nrb) rb -= nrb;
-        return rb;
+    // Workgroups that share a slice of W walk it in the same order and at the same pace: the first
+    // one to ask for a line brings it into the XCD's L2, the others hit (starting them at
+    // different row blocks, to spread the requests, measured 3 % slower).
+    auto row_block = [&](uint32_t rbi) __attribute__((always_inline)) {  // clamped: rbi <= nrb
+        return rbi < nrb ? rbi : 0u;
     };
 
     // ---- W stream -------------------------------------------------------------------------------
@@ -539,8 +535,8 @@ int fused_gemm16_xreg(const void* W, const void* Xt, void* C, uint32_t M, uint32
     // W and a row block of C are addressed with 32-bit byte offsets
     if ((uint64_t)M * 2048u > 0xffffffffull || (uint64_t)N * 4u * 64u > 0xffffffffull)
         return MI_ERR_SHAPE;
-    if (in_dtype == MI_BF16) return xreg::launch<BF16, 1024>(W, Xt, C, M, N, out_f32, scale, 2u, s);
-    if (in_dtype == MI_F16) return xreg::launch<F16, 1024>(W, Xt, C, M, N, out_f32, scale, 2u, s);
+    if (in_dtype == MI_BF16) return xreg::launch<BF16, 1024>(W, Xt, C, M, N, out_f32, scale, 4u, s);
+    if (in_dtype == MI_F16) return xreg::launch<F16, 1024>(W, Xt, C, M, N, out_f32, scale, 4u, s);
     return MI_ERR_DTYPE;
 }
 
