@@ -1,10 +1,11 @@
 """Benchmark / check harness around the ops, following the reference's protocols.
 
-Two sub-commands (run from the repository root)::
+Sub-commands (run from the repository root)::
 
     python -m 6s894_project_2025_amd.harness fwht  [--check] [--runs-per-size 400] [--sizes ...]
     python -m 6s894_project_2025_amd.harness fused [--dtype bf16|f32] [--runs 8] [--out-prefix P]
     python -m 6s894_project_2025_amd.harness plot P.csv [--out-dir plots]
+    python -m 6s894_project_2025_amd.harness mfma  [--steps 4096]
 
 ``fwht`` follows the protocol of the reference's bench/bench.py: a registry of in-place cases
 (add-one roofline proxies around the transform, :96-103), a correctness pass of every case with
@@ -37,7 +38,7 @@ from typing import Any, Callable
 import torch
 
 from .ops import fused_ht_gemm, hadamard_transform
-from .timing import best_single_call_ms, event_window_ms
+from .timing import best_single_call_ms, event_window_ms, steady_window_ms
 
 ATOL = {torch.float16: 1e-2, torch.bfloat16: 5e-2, torch.float32: 1e-4}
 DTYPES = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}
@@ -198,6 +199,43 @@ def run_fused(dtype: torch.dtype, runs: int = 8, configs=None, out_prefix: str |
     return rows
 
 
+def run_mfma_probe(steps: int = 4096, repeats: int = 20) -> list[dict[str, Any]]:
+    """Sustained matrix-core rate and shader clock of this chip, with random and with constant
+    operands, at 1, 2 and 4 wavefronts per SIMD, with and without LDS fragment reads beside the
+    MFMAs (``mi_debug_mfma_rate``).  This is the ceiling the fused GEMM kernels can be read
+    against: the paper peak assumes 2.4 GHz, the clock under full matrix-core load is lower and
+    depends on the operand data.  ``ghz`` is loop cycles (shader clock counter, slowest wavefront)
+    over the event-timed duration of the whole launch, so it is a slight underestimate."""
+    from . import _lib
+
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    cycles = torch.zeros(512, dtype=torch.int64, device=dev)
+    patterns = {"random": torch.randn(32768, device=dev).to(torch.bfloat16),
+                "constant": torch.full((32768,), 1.0, device=dev, dtype=torch.bfloat16)}
+    rows = []
+    for pname, ops in patterns.items():
+        for shape in (16, 32):
+            for reads in (0, 4):
+                for wps in (1, 2, 4):
+                    def call():
+                        _lib.check(lib.mi_debug_mfma_rate(shape, reads, wps, steps, ops.data_ptr(),
+                                                          cycles.data_ptr(), stream), "mfma probe")
+                    ms, _ = steady_window_ms(call, repeats, 30.0)  # past the clock ramp
+                    flops = 256 * 4 * wps * steps * 131072
+                    clk = cycles[:256].double().mean().item()
+                    row = {"operands": pname, "mfma": f"{shape}x{shape}x{512 // shape}_bf16",
+                           "lds_reads_per_step": reads, "waves_per_simd": wps,
+                           "tflops": flops / ms / 1e9, "ghz": clk / (ms * 1e6),
+                           "cycles_per_step_per_simd": clk / steps / wps}
+                    rows.append(row)
+                    print(f"{pname:8s} {row['mfma']:14s} reads/step {reads} waves/SIMD {wps}: "
+                          f"{row['tflops']:7.1f} TFLOP/s  {row['ghz']:.2f} GHz  "
+                          f"{row['cycles_per_step_per_simd']:.1f} cycles per step per SIMD (128 = issue bound)")
+    return rows
+
+
 def plot_fused(csv_path: str, out_dir: str = "plots") -> list[str]:
     """Figures from the sweep CSV, the counterpart of fused_ht/plot_results.py: speed-up of the fused
     kernel over the unfused baseline against K for every N = M, and achieved TFLOP/s of both."""
@@ -253,6 +291,8 @@ def main(argv=None) -> int:
     p2.add_argument("--dtype", default="bf16", choices=list(DTYPES))
     p2.add_argument("--runs", type=int, default=8)
     p2.add_argument("--out-prefix", default=None)
+    p4 = sub.add_parser("mfma")
+    p4.add_argument("--steps", type=int, default=4096)
     p3 = sub.add_parser("plot")
     p3.add_argument("csv")
     p3.add_argument("--out-dir", default="plots")
@@ -264,6 +304,9 @@ def main(argv=None) -> int:
     if not torch.cuda.is_available():
         sys.stderr.write("harness: no GPU visible\n")
         return 2
+    if args.cmd == "mfma":
+        run_mfma_probe(args.steps)
+        return 0
     if args.cmd == "fwht":
         run_fwht(TestConfig(check=args.check, runs_per_size=args.runs_per_size,
                             json_output_file=args.json_output_file, benchmark_cases=args.cases,

@@ -73,3 +73,15 @@ def test_fused_sweep_small(harness, dtype, tmp_path):
         assert r["fused_ms"] > 0 and r["baseline_ms"] > 0
     assert json.loads((tmp_path / "s.json").read_text())[0]["kdim"] == 256
     assert (tmp_path / "s.csv").read_text().startswith("kdim,ndim,mdim")
+
+
+def test_mfma_probe_reports_a_plausible_ceiling(harness):
+    # the probe is the measured ceiling for the matrix-core-bound kernels: rates between a third of
+    # the 2516.6 TFLOP/s paper peak and the peak itself, a clock between 1 and 2.5 GHz, and never
+    # fewer cycles per step than the 128 the eight MFMAs of a step occupy the pipeline
+    rows = harness.run_mfma_probe(steps=1024, repeats=5)
+    assert len(rows) == 2 * 2 * 2 * 3
+    for r in rows:
+        assert 800.0 < r["tflops"] < 2600.0, r
+        assert 1.0 < r["ghz"] < 2.6, r
+        assert r["cycles_per_step_per_simd"] > 125.0, r
