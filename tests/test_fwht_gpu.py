@@ -243,11 +243,12 @@ def test_reference_sweep_against_matrix_product(pkg, p, dt):
 
 
 # Tensors beyond the 256 MiB Infinity Cache make the launcher pick the other variants (one LDS
-# exchange per row for n >= 8192, one row per wavefront for n <= 4096).  The reference's harness
+# exchange per row for n >= 8192; one step per wavefront and workgroups of one, two or four
+# wavefronts, depending on n and the element size, for n <= 4096).  The reference's harness
 # runs 2^30 elements (bench/bench.py:138); here each tensor is just past 256 MiB, generated on the
 # device, with sampled rows against the fp64 oracle and the involution as a whole-tensor check.
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32, torch.float16], ids=["bf16", "f32", "f16"])
-@pytest.mark.parametrize("n", [4096, 8192, 16384, 32768])
+@pytest.mark.parametrize("n", [256, 1024, 2048, 4096, 8192, 16384, 32768])
 def test_beyond_infinity_cache_variants(pkg, oracle, n, dt):
     esize = 4 if dt == torch.float32 else 2
     rows = (256 << 20) // (n * esize) + 3
