@@ -75,11 +75,11 @@ __global__ void __launch_bounds__(64 << LW)
 fwht_lds_kernel(const void* in, void* out, uint64_t rows, int exp2, float mult)
 {
     extern __shared__ f32x4 xch[];
-    // Consecutive workgroup ids run on different XCDs (id % 8).  Inside every full group of 16
-    // rows, XCD x takes the adjacent rows 2x and 2x+1 (neutral for n = 8192 and 16384, 2.7 %
-    // faster for n = 32768 on tensors beyond the last-level cache).
+    // Consecutive workgroup ids run on different XCDs (id % 8).  On tensors beyond the last-level
+    // cache (the streaming variants), XCD x takes the adjacent rows 2x and 2x+1 inside every full
+    // group of 16 rows: neutral for n = 8192 and 16384, 2.7 % faster for n = 32768.
     uint64_t row = blockIdx.x;
-    if (row < (rows & ~(uint64_t)15u))
+    if (IO::kStreaming && row < (rows & ~(uint64_t)15u))
         row = (row & ~(uint64_t)15u) + ((row & 7u) * 2u + ((row >> 3) & 1u));
     if (row >= rows) return;
     const uint64_t total = rows << (12 + LW);

@@ -35,6 +35,7 @@ namespace mi {
 template <class T16_, bool STREAM = false>
 struct Io16 {
     using Streaming = Io16<T16_, true>;
+    static constexpr bool kStreaming = STREAM;
     using T16 = T16_;
     using E = typename T16::E;
     using Elem = E;
@@ -94,6 +95,7 @@ struct Io16 {
 template <bool STREAM = false>
 struct Io32T {
     using Streaming = Io32T<true>;
+    static constexpr bool kStreaming = STREAM;
     using T16 = BF16;  // matrix-core type used for the three-piece products
     using Elem = float;
     static constexpr int ESIZE = 4;

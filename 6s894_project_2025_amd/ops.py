@@ -119,6 +119,11 @@ def fused_ht_gemm(W: torch.Tensor, Xt: torch.Tensor, scale: float | None = None,
     operand stays on chip.  fp32 (fp32 MFMA) or bf16/fp16 inputs (fp32 accumulate);
     ``out_dtype`` defaults to the input dtype.  ``scale=None`` -> ``K ** -0.5``; ``scale=1.0``
     reproduces the reference kernel.
+
+    Where fusing pays on this chip: 16-bit inputs with K <= 1024 (the transformed operand of 128
+    columns fits a compute unit's registers at K = 1024).  For K >= 2048, and for fp32 inputs,
+    ``hadamard_transform(Xt)`` followed by a library GEMM is the faster route; this op still runs
+    those shapes, for callers that cannot afford the intermediate.
     """
     _require_cuda(W, "W")
     _require_cuda(Xt, "Xt")
