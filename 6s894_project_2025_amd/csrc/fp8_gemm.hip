@@ -17,6 +17,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "lds_layout.hpp"
 
 namespace mi {
 namespace {
@@ -39,10 +40,36 @@ __device__ __forceinline__ void mfma_fp8(f32x4& c, const i32x8& a, const i32x8& 
     asm volatile("s_nop 1\n\tv_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
 
-__device__ __forceinline__ uint32_t tile_off(uint32_t row, uint32_t chunk)
+__host__ __device__ constexpr uint32_t tile_off(uint32_t row, uint32_t chunk)
 {
     return (row * 8u + (chunk ^ (row & 7u))) << 4;
 }
+// Epilogue image of the 256 x 256 bf16 result: [256 rows][512 B], chunk c of row r stored at
+// c ^ (r & 31).
+__host__ __device__ constexpr uint32_t out_tile_off(uint32_t row, uint32_t chunk)
+{
+    return row * 512u + ((chunk ^ (row & 31u)) << 4);
+}
+constexpr bool lds_patterns_conflict_free()
+{
+    // operand fragments: lane (hi, lo) reads row r0 + lo, chunks hi and hi + 4
+    for (uint32_t half = 0; half < 2; ++half)
+        if (!lds::conflict_free_b128(
+                [=](uint32_t lane) { return tile_off(lane & 15u, (lane >> 4) + 4u * half); }))
+            return false;
+    // epilogue: lane (hi, lo) writes row 16 ti + lo, chunk 4 hi + r (+ 16 per wavefront column); the
+    // copy-out reads row 8 i + tid / 32, chunk tid % 32
+    for (uint32_t r = 0; r < 4; ++r)
+        if (!lds::conflict_free_b128(
+                [=](uint32_t lane) { return out_tile_off(lane & 15u, 4u * (lane >> 4) + r); }))
+            return false;
+    for (uint32_t w = 0; w < 4; ++w)
+        if (!lds::conflict_free_b128(
+                [=](uint32_t lane) { return out_tile_off((64u * w + lane) >> 5, (64u * w + lane) & 31u); }))
+            return false;
+    return true;
+}
+static_assert(lds_patterns_conflict_free(), "an LDS access pattern of the FP8 GEMM would serialise");
 
 // LDS row r of the qb tile holds tile row 128*(r>>7) + 8*(r&15) + ((r>>4)&7): fragment block nb of
 // a wavefront (LDS rows 16*nb .. 16*nb+15) then carries columns 8*lo + nb.
@@ -229,7 +256,7 @@ fp8_gemm_rowscale_kernel(const uint8_t* __restrict__ qa, const float* __restrict
 #pragma unroll
             for (int nb = 0; nb < 8; ++nb) o[nb] = (__bf16)(acc[nb][ti][r] * st * sbv[8 * r + nb]);
             const uint32_t ch = col >> 3;
-            *reinterpret_cast<bf16x8v*>(lds + rl * 512u + ((ch ^ (rl & 31u)) << 4)) = o;
+            *reinterpret_cast<bf16x8v*>(lds + out_tile_off(rl, ch)) = o;
         }
     }
     __syncthreads();
@@ -237,7 +264,7 @@ fp8_gemm_rowscale_kernel(const uint8_t* __restrict__ qa, const float* __restrict
 #pragma unroll 4
     for (uint32_t i = 0; i < 32; ++i) {
         const uint32_t rl = 8u * i + (tid >> 5), ch = tid & 31u;
-        const bf16x8v o = *reinterpret_cast<const bf16x8v*>(lds + rl * 512u + ((ch ^ (rl & 31u)) << 4));
+        const bf16x8v o = *reinterpret_cast<const bf16x8v*>(lds + out_tile_off(rl, ch));
         const uint32_t t = t0 + rl, col = n0 + 8u * ch;
         if (t < T && col < N) {
             __bf16* dst = out + (uint64_t)t * N + col;

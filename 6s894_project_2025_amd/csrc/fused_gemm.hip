@@ -28,6 +28,7 @@
 #include <type_traits>
 
 #include "fwht_device.hpp"
+#include "lds_layout.hpp"
 
 namespace mi {
 
@@ -47,13 +48,54 @@ constexpr int kStageBytes = kWaveRows * 64;  // per-wavefront LDS staging: rows 
 // `col_bytes` = bytes per column, LOG_NB = log2(16-column fragments per block): the fragment
 // read of lane `lo` touches column NB*lo + nb, so the swizzle key is n / NB.
 template <int LOG_NB>
-__device__ __forceinline__ uint32_t y_chunk_offset(uint32_t n, uint32_t q, uint32_t col_bytes,
-                                                   uint32_t swz_mask)
+__host__ __device__ constexpr uint32_t y_chunk_offset(uint32_t n, uint32_t q, uint32_t col_bytes,
+                                                      uint32_t swz_mask)
 {
     // built as (16-byte chunk index) << 4 so that the 16-byte alignment is visible to the compiler
     // and every access becomes a single ds_read_b128 / ds_write_b128
     return (n * (col_bytes >> 4) + (q ^ ((n >> LOG_NB) & swz_mask))) << 4;
 }
+
+// Per-wavefront staging of a 64-row x 32-K sub-step of W: row r (64 bytes), 16-byte chunk c stored
+// at position c ^ ((r >> 1) & 3).  Writer lane l holds row l / 4, chunk l % 4 (coalescable global
+// loads); reader lane (hi, lo) takes row lo, chunk hi (MFMA operand order).
+__host__ __device__ constexpr uint32_t stage_write_offset(uint32_t lane)
+{
+    return (lane >> 2) * 64u + (((lane & 3u) ^ ((lane >> 3) & 3u)) << 4);
+}
+__host__ __device__ constexpr uint32_t stage_read_offset(uint32_t lane)
+{
+    return (lane & 15u) * 64u + (((lane >> 4) ^ (((lane & 15u) >> 1) & 3u)) << 4);
+}
+template <int LOG_NB>
+constexpr bool y_patterns_conflict_free()
+{
+    // K >= 64 (at K = 32 a column is four chunks and the four-way key cannot separate eight lanes;
+    // that size is a single step with no loop to protect)
+    for (uint32_t K = 64; K <= 4096; K *= 2) {
+        const uint32_t chunks = K >> 3, mask = (chunks >= 16u ? 16u : chunks) - 1u;
+        // prologue write: lane l of tile t holds elements 512 t + 8 l ..: column e / K, chunk (e % K) / 8
+        for (uint32_t t = 0; t < 4; ++t)
+            if (!lds::conflict_free_b128([=](uint32_t lane) {
+                    const uint32_t e = 512u * t + 8u * lane;
+                    return y_chunk_offset<LOG_NB>(e / K, (e % K) >> 3, K * 2u, mask);
+                }))
+                return false;
+        // fragment read: lane (hi, lo) takes column NB lo + nb, chunk q0 + hi (the pattern repeats
+        // every 16 chunks)
+        for (uint32_t nb = 0; nb < (1u << LOG_NB); ++nb)
+            for (uint32_t q0 = 0; q0 < chunks && q0 < 16u; q0 += 4)
+                if (!lds::conflict_free_b128([=](uint32_t lane) {
+                        return y_chunk_offset<LOG_NB>(((lane & 15u) << LOG_NB) + nb, q0 + (lane >> 4), K * 2u, mask);
+                    }))
+                    return false;
+    }
+    return true;
+}
+static_assert(lds::conflict_free_b128(stage_write_offset) && lds::conflict_free_b128(stage_read_offset),
+              "the W staging pattern would serialise");
+static_assert(y_patterns_conflict_free<0>() && y_patterns_conflict_free<1>() && y_patterns_conflict_free<2>(),
+              "an access pattern of the transformed tile would serialise");
 
 // XB = log2(max(K,512)/512): tiles per column that need cross-tile butterflies.
 // KFIX: K when it is known at compile time (lets the K loop be scheduled without run-time guards),
@@ -176,8 +218,8 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
     // staging layout for a 64-row x 32-K sub-step: row r (64 bytes), 16-byte chunk c stored at
     // position c ^ ((r >> 1) & 3) (measured conflict-free for both access orders).  Writer lane l
     // holds row 16*mi + l/4, chunk l%4; reader lane (hi, lo) takes row 16*mi + lo, chunk hi.
-    const uint32_t wr_off = (lane >> 2) * 64u + (((lane & 3u) ^ ((lane >> 3) & 3u)) << 4);
-    const uint32_t rd_off = lo * 64u + ((hi ^ ((lo >> 1) & 3u)) << 4);
+    const uint32_t wr_off = stage_write_offset(lane);
+    const uint32_t rd_off = stage_read_offset(lane);
 
     while (mb < m_end) {
         f32x4 acc[NB][kMI];

@@ -31,6 +31,7 @@
 #include <type_traits>
 
 #include "fwht_device.hpp"
+#include "lds_layout.hpp"
 
 namespace mi {
 namespace xreg {
@@ -49,6 +50,35 @@ constexpr int kAreaBase = 3 * kStageBytes;
 constexpr int kLdsBytes = kAreaBase + 4 * kAreaBytes;
 
 typedef __attribute__((address_space(3))) void* lptr_t;
+
+// LDS image of a W stage: [64 rows][512 B], the 16-byte chunk q of row r stored at q ^ (r & 15).
+__host__ __device__ constexpr uint32_t stage_offset(uint32_t row, uint32_t q)
+{
+    return row * 512u + ((q ^ (row & 15u)) << 4);
+}
+// A wavefront's area of the prologue: [16 columns][1 KB], chunk q of column j stored at q ^ j.
+__host__ __device__ constexpr uint32_t area_offset(uint32_t j, uint32_t q)
+{
+    return j * 1024u + ((q ^ j) << 4);
+}
+constexpr bool lds_patterns_conflict_free()
+{
+    // fragment read of row block mb, K step ks: lane (hi, lo) takes row 16 mb + lo, chunk 4 ks + hi
+    for (uint32_t mb = 0; mb < 4; ++mb)
+        for (uint32_t ks = 0; ks < 8; ++ks)
+            if (!lds::conflict_free_b128(
+                    [=](uint32_t lane) { return stage_offset(16u * mb + (lane & 15u), 4u * ks + (lane >> 4)); }))
+                return false;
+    // prologue: every lane writes chunk `lane` of column j; lane (hi, lo) reads chunk 4 s + hi of
+    // column lo
+    for (uint32_t j = 0; j < 16; ++j)
+        if (!lds::conflict_free_b128([=](uint32_t lane) { return area_offset(j, lane); })) return false;
+    for (uint32_t s = 0; s < 16; ++s)
+        if (!lds::conflict_free_b128([=](uint32_t lane) { return area_offset(lane & 15u, 4u * s + (lane >> 4)); }))
+            return false;
+    return true;
+}
+static_assert(lds_patterns_conflict_free(), "an LDS access pattern of the fused GEMM would serialise");
 
 // acc (+)= A(16 x 32) * B(32 x 16) with B read straight from the accumulation-register file, where
 // the transformed operand lives for the whole kernel, and the accumulator in ordinary registers.
@@ -288,20 +318,20 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
                     w_issue((p + 1) >> 3, (p + 1) >> 3, (p + 1) & 7);
                 }
                 // area: [16 columns][64 chunks of 16 B], chunk q of column j stored at q ^ j
-                *reinterpret_cast<V8*>(area + j * 1024u + ((lane ^ j) << 4)) = first_half;
+                *reinterpret_cast<V8*>(area + area_offset(j, lane)) = first_half;
             }
             // LDS operations of one wavefront complete in order: no barrier between its own
             // writes and reads
 #pragma unroll
             for (int s = 0; s < KSTEPS / 2; ++s)
-                yf[nb][s] = *reinterpret_cast<const V8*>(area + lo * 1024u + (((4u * s + hi) ^ lo) << 4));
+                yf[nb][s] = *reinterpret_cast<const V8*>(area + area_offset(lo, 4u * s + hi));
 #pragma unroll
             for (int j = 0; j < 16; ++j)
-                *reinterpret_cast<V8*>(area + j * 1024u + ((lane ^ j) << 4)) = hold[j];
+                *reinterpret_cast<V8*>(area + area_offset(j, lane)) = hold[j];
 #pragma unroll
             for (int s = 0; s < KSTEPS / 2; ++s)
                 yf[nb][KSTEPS / 2 + s] =
-                    *reinterpret_cast<const V8*>(area + lo * 1024u + (((4u * s + hi) ^ lo) << 4));
+                    *reinterpret_cast<const V8*>(area + area_offset(lo, 4u * s + hi));
         }
     }
 
@@ -311,8 +341,8 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     __builtin_amdgcn_s_barrier();
 
     auto frag = [&](uint32_t slot, int mb, int ks) __attribute__((always_inline)) -> V8 {
-        return *reinterpret_cast<const V8*>(lds + slot * kStageBytes + (16u * mb + lo) * 512u +
-                                            (((4u * ks + hi) ^ lo) << 4));
+        return *reinterpret_cast<const V8*>(lds + slot * kStageBytes +
+                                            stage_offset(16u * mb + lo, 4u * ks + hi));
     };
     V8 fr[4][4];  // [K step % 4][mb]
 #pragma unroll
@@ -456,12 +486,12 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
 #pragma unroll 1
     for (uint32_t rbi = 0; rbi < nrb; rbi += 2u) {
         run(pend, accA, accB, pend_base, rbi);
-            bool fullA;
+        bool fullA;
         uint64_t baseA;
         finish(accA, rbi, fullA, baseA);
         if (rbi + 1u < nrb) {
             run(fullA, accB, accA, baseA, rbi + 1u);
-                    finish(accB, rbi + 1u, pend, pend_base);
+            finish(accB, rbi + 1u, pend, pend_base);
         } else {
             pend = false;
             if (fullA) {
