@@ -207,12 +207,26 @@ __device__ __forceinline__ void stream_store8(uint32_t lane_off, u32x2 v, void* 
     asm volatile("global_store_dwordx2 %0, %1, %2 nt" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
 }
 
+// Workgroup id -> (column group, M slice); false for an id past the last rectangle.
+__host__ __device__ inline bool tile_of_workgroup(uint32_t id, uint32_t msplit, uint32_t mpx, uint32_t cgx,
+                                                  uint32_t nrect, uint32_t& cg, uint32_t& ms)
+{
+    const uint32_t x = id & 7u, j = id >> 3;  // XCD, index inside the XCD
+    const uint32_t rsz = mpx * cgx;
+    const uint32_t rect = (j / rsz) * 8u + x, in = j % rsz;
+    if (rect >= nrect) return false;
+    const uint32_t rects_m = msplit / mpx;
+    ms = (rect % rects_m) * mpx + in % mpx;
+    cg = (rect / rects_m) * cgx + in / mpx;
+    return true;
+}
+
 template <class T16, int K, bool OUT_F32>
 __global__ void __launch_bounds__(kThreads)
 fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
                           const typename T16::E* __restrict__ Xt, void* __restrict__ C, uint32_t M,
                           uint32_t N, uint32_t m_per_block, uint32_t msplit, uint32_t mpx,
-                          int exp2, float mult)
+                          uint32_t cgx, uint32_t nrect, int exp2, float mult)
 {
     using E = typename T16::E;
     using V8 = typename T16::V8;
@@ -228,24 +242,15 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t lo = lane & 15u, hi = lane >> 4;
 
-    // ---- which tile: consecutive workgroup ids go to different XCDs (id % 8).  `mpx` = M slices
-    // handled inside one XCD: 1 keeps one slice of W per XCD L2 (and makes every XCD read all of
-    // X), larger values trade W locality for fewer redundant X reads per XCD.
+    // ---- which tile: consecutive workgroup ids go to different XCDs (id % 8).  The grid of
+    // (column group, M slice) tiles is cut into rectangles of cgx column groups x mpx M slices, and
+    // a rectangle is handled inside one XCD by workgroups that are dispatched back to back: its
+    // L2 then holds mpx slices of W, each shared by cgx workgroups, and cgx blocks of X, each
+    // shared by mpx.  (mpx = 1 keeps one slice of W per XCD but makes it read eight times as much
+    // of X; 2 - 4 measured best.)  Rectangle r runs on XCD r % 8; ids past the last rectangle have
+    // no work.
     uint32_t cg, ms;
-    {
-        const uint32_t id = blockIdx.x;
-        const uint32_t ngroups = gridDim.x / msplit;
-        if (msplit == 8u && (ngroups % mpx) == 0u && mpx <= 8u) {
-            const uint32_t x = id & 7u, j = id >> 3;  // XCD, index inside the XCD
-            const uint32_t sets = 8u / mpx;           // distinct slice sets
-            const uint32_t ss = x % sets, part = x / sets;
-            ms = ss * mpx + j % mpx;
-            cg = part * (ngroups / mpx) + j / mpx;
-        } else {
-            ms = id % msplit;
-            cg = id / msplit;
-        }
-    }
+    if (!tile_of_workgroup(blockIdx.x, msplit, mpx, cgx, nrect, cg, ms)) return;  // uniform, before any barrier
     const uint32_t n0 = cg * kCols;
     const uint32_t m_begin = ms * m_per_block;
     if (m_begin >= M || n0 >= N) return;  // workgroup-uniform, before any barrier
@@ -514,20 +519,65 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     // it, so none is in flight when the workgroup's LDS is released.
 }
 
-// msplit / m_per_block: about one workgroup per compute unit, every slice a multiple of 64 rows.
+// How the (column group, M slice) grid is cut.  One workgroup fills a compute unit (all of its
+// registers and LDS), so the launch runs in rounds of 256 workgroups; a workgroup costs one prologue
+// (measured ~6.5 us) plus ~2.9 us per 64-row block.  The number of M slices is the one that
+// minimises rounds x (prologue + row blocks per slice) in those units (9 : 4): enough slices to
+// fill the chip, no more than that (every slice repeats the transform of its columns), and no
+// nearly empty last round.
 struct Plan {
     uint32_t ngroups, msplit, m_per_block;
+    uint32_t mpx, cgx, nrect, grid;  // XCD rectangles
 };
-inline Plan plan(uint32_t M, uint32_t N)
+inline Plan plan(uint32_t M, uint32_t N, uint32_t mpx_max)
 {
-    Plan p;
+    Plan p{};
     p.ngroups = (N + kCols - 1u) / kCols;
     const uint32_t row_blocks = (M + kRows - 1u) / kRows;
-    uint32_t msplit = (256u + p.ngroups - 1u) / p.ngroups;
-    if (msplit > row_blocks) msplit = row_blocks;
-    if (msplit < 1u) msplit = 1u;
-    p.m_per_block = ((row_blocks + msplit - 1u) / msplit) * kRows;
+    uint64_t best = ~0ull;
+    uint32_t best_s = 1;
+    for (uint32_t sp = 1; sp <= row_blocks && sp <= 256u; ++sp) {
+        const uint32_t rb = (row_blocks + sp - 1u) / sp;
+        const uint32_t slices = (row_blocks + rb - 1u) / rb;  // what sp really yields
+        const uint64_t rounds = ((uint64_t)p.ngroups * slices + 255u) / 256u;
+        const uint64_t cost = rounds * (9u + 4u * (uint64_t)rb);
+        if (cost < best) {
+            best = cost;
+            best_s = slices;
+        }
+    }
+    const uint32_t rb = (row_blocks + best_s - 1u) / best_s;
+    p.m_per_block = rb * kRows;
     p.msplit = (M + p.m_per_block - 1u) / p.m_per_block;
+    // Rectangles: mpx | msplit, cgx | ngroups, at most 32 workgroups (one round of an XCD).
+    // Rectangle r runs on XCD r % 8, so the busiest XCD gets ceil(nrect / 8) rectangles.  Wanted,
+    // in this order: as few rounds on the busiest XCD as possible, a load within 15 % of an even
+    // spread over the eight XCDs, the largest rectangle, M extent 4 before 2, 8, 1.  (1 x 1 is
+    // the plain order, so there is always a candidate.)
+    const uint32_t total = p.ngroups * p.msplit;
+    const uint32_t even = (total + 7u) / 8u;
+    const uint32_t pref[4] = {4u, 2u, 8u, 1u};
+    uint64_t best_key = ~0ull;
+    for (uint32_t k = 0; k < 4; ++k) {
+        const uint32_t m = pref[k];
+        if (m > mpx_max || p.msplit % m != 0u) continue;
+        for (uint32_t c = 1; c * m <= 32u; ++c) {
+            if (p.ngroups % c != 0u) continue;
+            const uint32_t nrect = (p.msplit / m) * (p.ngroups / c);
+            const uint32_t busiest = ((nrect + 7u) / 8u) * m * c;
+            const uint64_t rounds = (busiest + 31u) / 32u;
+            const uint64_t uneven = (uint64_t)busiest * 100u > (uint64_t)even * 115u ? 1u : 0u;
+            const uint64_t key = (rounds << 40) | (uneven << 36) | ((uint64_t)(32u - m * c) << 24) |
+                                 ((uint64_t)k << 20) | busiest;
+            if (key < best_key) {
+                best_key = key;
+                p.mpx = m;
+                p.cgx = c;
+                p.nrect = nrect;
+            }
+        }
+    }
+    p.grid = ((p.nrect + 7u) / 8u) * 8u * p.mpx * p.cgx;
     return p;
 }
 
@@ -536,15 +586,15 @@ int launch_as(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, fl
               uint32_t mpx, hipStream_t s)
 {
     const OutputScale os = split_output_scale((double)scale, tile_stage_shift<2>(10, kNarrowRange<T16>));
-    const Plan p = plan(M, N);
+    const Plan p = plan(M, N, mpx);
     auto kern = fused_ht_gemm_xreg_kernel<T16, K, OUT_F32>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess)
         return MI_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3(p.ngroups * p.msplit), dim3(kThreads), kLdsBytes, s,
+    hipLaunchKernelGGL(kern, dim3(p.grid), dim3(kThreads), kLdsBytes, s,
                        static_cast<const typename T16::E*>(W),
-                       static_cast<const typename T16::E*>(Xt), C, M, N, p.m_per_block, p.msplit, mpx,
-                       os.exp2, os.mult);
+                       static_cast<const typename T16::E*>(Xt), C, M, N, p.m_per_block, p.msplit, p.mpx,
+                       p.cgx, p.nrect, os.exp2, os.mult);
     return launch_status();
 }
 
@@ -565,9 +615,29 @@ int fused_gemm16_xreg(const void* W, const void* Xt, void* C, uint32_t M, uint32
     // W and a row block of C are addressed with 32-bit byte offsets
     if ((uint64_t)M * 2048u > 0xffffffffull || (uint64_t)N * 4u * 64u > 0xffffffffull)
         return MI_ERR_SHAPE;
-    if (in_dtype == MI_BF16) return xreg::launch<BF16, 1024>(W, Xt, C, M, N, out_f32, scale, 4u, s);
-    if (in_dtype == MI_F16) return xreg::launch<F16, 1024>(W, Xt, C, M, N, out_f32, scale, 4u, s);
+    if (in_dtype == MI_BF16) return xreg::launch<BF16, 1024>(W, Xt, C, M, N, out_f32, scale, 8u, s);
+    if (in_dtype == MI_F16) return xreg::launch<F16, 1024>(W, Xt, C, M, N, out_f32, scale, 8u, s);
     return MI_ERR_DTYPE;
 }
 
 }  // namespace mi
+
+extern "C" int mi_debug_fused_gemm_tiling(uint32_t M, uint32_t N, uint32_t* header, uint32_t* tiles,
+                                          uint32_t capacity)
+{
+    using namespace mi;
+    if (!header) return MI_ERR_NULL;
+    if (M == 0 || N == 0) return MI_ERR_SHAPE;
+    const xreg::Plan p = xreg::plan(M, N, 8u);
+    const uint32_t h[8] = {p.ngroups, p.msplit, p.m_per_block, p.mpx, p.cgx, p.nrect, p.grid, 0u};
+    for (int i = 0; i < 8; ++i) header[i] = h[i];
+    if (!tiles) return MI_OK;
+    if (capacity < p.grid) return MI_ERR_SIZE;
+    for (uint32_t id = 0; id < p.grid; ++id) {
+        uint32_t cg = 0xffffffffu, ms = 0xffffffffu;
+        if (!xreg::tile_of_workgroup(id, p.msplit, p.mpx, p.cgx, p.nrect, cg, ms)) cg = ms = 0xffffffffu;
+        tiles[2u * id] = cg;
+        tiles[2u * id + 1u] = ms;
+    }
+    return MI_OK;
+}

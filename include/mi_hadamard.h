@@ -161,11 +161,27 @@ int mi_debug_device_fwht(const void* in, void* out, uint64_t rows, uint32_t n, i
  * to measure the clock and the matrix-core rate the chip sustains for a given operand pattern.
  * No counterpart in the reference.
  *   operands : device, 16-byte aligned, at least 64 KiB (any bit pattern; bf16 operands)
- *   cycles   : device, 512 x uint64 (the second half is scratch for the probe's own use)
+ *   cycles   : device, 512 x uint64: [0, 256) cycles per workgroup, [256, 512) a checksum of each
+ *              workgroup's accumulators (an output whose only purpose is to keep the arithmetic alive)
  *   waves_per_simd in {1, 2, 4};  steps a positive multiple of 4.
  */
 int mi_debug_mfma_rate(int shape, int lds_reads, uint32_t waves_per_simd, uint32_t steps,
                        const void* operands, uint64_t* cycles, void* stream);
+
+/*
+ * Host-only: how mi_fused_ht_gemm cuts a K = 1024, 16-bit problem into workgroups (no GPU call).
+ * The (column group, M slice) grid, the XCD rectangles and the map from workgroup id to tile are
+ * what decides L2 reuse and the number of launch rounds; this hook lets a test check on the CPU
+ * that every tile is handled by exactly one workgroup.  No counterpart in the reference.
+ *   header[8] : ngroups (128-column groups), msplit (M slices), m_per_block (rows per slice),
+ *               mpx, cgx (rectangle extents in M slices and column groups), nrect, grid
+ *               (workgroups launched), 0
+ *   tiles     : NULL, or 2 * capacity uint32: for workgroup id i, tiles[2i] = column group and
+ *               tiles[2i+1] = M slice, or 0xffffffff twice for an id without work
+ * Returns MI_ERR_SIZE when capacity < grid (header is filled in either way).
+ */
+int mi_debug_fused_gemm_tiling(uint32_t M, uint32_t N, uint32_t* header, uint32_t* tiles,
+                               uint32_t capacity);
 
 #ifdef __cplusplus
 }

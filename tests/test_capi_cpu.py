@@ -98,3 +98,60 @@ def test_product_code_never_touches_the_oracle():
                 assert "oracle" not in text.lower(), f"{f} mentions the oracle"
     hdr = open(HEADER).read().lower()
     assert "oracle" not in hdr
+
+
+def _tiling(lib, M, N):
+    import ctypes
+
+    header = (ctypes.c_uint32 * 8)()
+    assert lib.mi_debug_fused_gemm_tiling(M, N, header, None, 0) == 0
+    ngroups, msplit, m_per_block, mpx, cgx, nrect, grid, _ = list(header)
+    tiles = (ctypes.c_uint32 * (2 * grid))()
+    assert lib.mi_debug_fused_gemm_tiling(M, N, header, tiles, grid) == 0
+    return dict(ngroups=ngroups, msplit=msplit, m_per_block=m_per_block, mpx=mpx, cgx=cgx,
+                nrect=nrect, grid=grid), [(tiles[2 * i], tiles[2 * i + 1]) for i in range(grid)]
+
+
+def test_fused_gemm_tiling_covers_every_tile_exactly_once(libmod):
+    # host logic of the K = 1024 fused GEMM launch: no GPU call involved
+    lib = libmod.load()
+    shapes = [(4096, 4096), (1, 1), (64, 128), (65, 129), (577, 1333), (5000, 3000), (12288, 12288),
+              (2048, 8192), (8192, 2048), (4096, 16384), (16384, 4096), (700, 4095), (130, 2000),
+              (4096, 130), (100000, 128), (64, 100000), (9999, 7777), (8192, 8192), (3968, 31 * 128)]
+    for M, N in shapes:
+        p, tiles = _tiling(lib, M, N)
+        assert p["ngroups"] == -(-N // 128)
+        assert p["m_per_block"] % 64 == 0 and p["msplit"] == -(-M // p["m_per_block"])
+        assert (p["msplit"] - 1) * p["m_per_block"] < M          # no empty slice
+        real = [t for t in tiles if t != (0xFFFFFFFF, 0xFFFFFFFF)]
+        want = {(cg, ms) for cg in range(p["ngroups"]) for ms in range(p["msplit"])}
+        assert len(real) == len(want) and set(real) == want, (M, N, p)
+        if True:
+            assert p["msplit"] % p["mpx"] == 0 and p["ngroups"] % p["cgx"] == 0
+            assert 1 <= p["mpx"] * p["cgx"] <= 32
+            # no XCD carries more rounds of 32 workgroups than an even spread would need
+            per_xcd = [sum(1 for i, t in enumerate(tiles) if i % 8 == x and t[0] != 0xFFFFFFFF) for x in range(8)]
+            assert -(-max(per_xcd) // 32) == -(-(-(-len(real) // 8)) // 32), (M, N, p, per_xcd)
+            # a rectangle lives on one XCD (workgroup id % 8) and its workgroups are dispatched
+            # back to back there
+            where = {}
+            for i, (cg, ms) in enumerate(tiles):
+                if cg != 0xFFFFFFFF:
+                    where.setdefault((cg // p["cgx"], ms // p["mpx"]), []).append(i)
+            for ids in where.values():
+                assert len({i % 8 for i in ids}) == 1
+                local = sorted(i // 8 for i in ids)
+                assert local == list(range(local[0], local[0] + len(ids)))
+
+
+def test_fused_gemm_tiling_avoids_a_nearly_empty_last_round(libmod):
+    lib = libmod.load()
+    # benchmark shape: one workgroup per compute unit, 4 x 8 rectangles, one per XCD
+    p, _ = _tiling(lib, 4096, 4096)
+    assert (p["ngroups"], p["msplit"], p["m_per_block"], p["mpx"], p["cgx"], p["grid"]) == (32, 8, 512, 4, 8, 256)
+    # 96 column groups: three slices would give 288 workgroups = one full round + 32 stragglers
+    p, _ = _tiling(lib, 12288, 12288)
+    assert (p["ngroups"] * p["msplit"]) % 256 == 0
+    # 24 column groups: 11 slices would be 264 workgroups; 10 fit one round
+    p, _ = _tiling(lib, 5000, 3000)
+    assert p["ngroups"] * p["msplit"] <= 256
