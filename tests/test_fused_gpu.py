@@ -144,6 +144,29 @@ def test_gemm_k1024_every_output_written_once(pkg, oracle):
         assert err <= (8e-3 if od == torch.bfloat16 else 2e-3), (od, err)
 
 
+# Shapes whose launch plan differs from the benchmark's: rectangles that do not fill all eight XCDs
+# evenly (workgroup ids without work), M slices that are not a power of two, more than one round of
+# workgroups, a ragged last slice and last column group.  Every element against the unfused
+# product computed on the device from the library's own transform.
+@pytest.mark.parametrize("M,N", [(5000, 3000), (6144, 6144), (2048, 8192), (12288, 1536), (1000, 9000)])
+def test_gemm_k1024_launch_plans(pkg, oracle, M, N):
+    K = 1024
+    g = torch.Generator(device="cuda").manual_seed(M + N)
+    Wd = torch.randn(M, K, generator=g, device="cuda").to(torch.bfloat16)
+    Xd = torch.randn(N, K, generator=g, device="cuda").to(torch.bfloat16)
+    Y = pkg.hadamard_transform(Xd)
+    ref = Wd.float() @ Y.float().t()
+    scale = ref.abs().max().item()
+    C = pkg.fused_ht_gemm(Wd, Xd)
+    torch.cuda.synchronize()
+    assert torch.isfinite(C.float()).all()
+    assert (C.float() - ref).abs().max().item() / scale <= 8e-3
+    # a few rows against the fp64 oracle as well
+    idx = torch.tensor([0, 63, 64, M // 2, M - 1])
+    want = oracle.fused_ht_gemm_f64_blas(Wd[idx].cpu().double().numpy(), Xd.cpu().double().numpy(), 1.0 / 32.0)
+    assert _rel(oracle, C[idx], want) <= 2e-2
+
+
 def test_gemm_small_bruteforce(pkg, oracle):
     # triple-loop oracle (no BLAS), fp32
     M, N, K = 16, 20, 64
