@@ -199,19 +199,35 @@ def run_fused(dtype: torch.dtype, runs: int = 8, configs=None, out_prefix: str |
     return rows
 
 
-def run_mfma_probe(steps: int = 4096, repeats: int = 20) -> list[dict[str, Any]]:
-    """Sustained matrix-core rate and shader clock of this chip, with random and with constant
-    operands, at 1, 2 and 4 wavefronts per SIMD, with and without LDS fragment reads beside the
-    MFMAs (``mi_debug_mfma_rate``).  This is the ceiling the fused GEMM kernels can be read
-    against: the paper peak assumes 2.4 GHz, the clock under full matrix-core load is lower and
-    depends on the operand data.  ``ghz`` is loop cycles (shader clock counter, slowest wavefront)
-    over the event-timed duration of the whole launch, so it is a slight underestimate."""
+def mfma_probe(shape: int, lds_reads: int, waves_per_simd: int, operands: torch.Tensor,
+               steps: int = 4096, repeats: int = 20, warm_ms: float = 30.0) -> dict[str, Any]:
+    """One configuration of ``mi_debug_mfma_rate``: nothing but back-to-back bf16 MFMAs on every
+    SIMD (plus ``lds_reads`` fragment reads per step), timed past the clock ramp.  ``ghz`` is loop
+    cycles (shader clock counter, slowest wavefront) over the event-timed duration of the whole
+    launch, so it is a slight underestimate."""
     from . import _lib
 
     lib = _lib.load()
-    dev = torch.device("cuda:0")
     stream = torch.cuda.current_stream().cuda_stream
-    cycles = torch.zeros(512, dtype=torch.int64, device=dev)
+    cycles = torch.zeros(512, dtype=torch.int64, device=operands.device)
+
+    def call():
+        _lib.check(lib.mi_debug_mfma_rate(shape, lds_reads, waves_per_simd, steps, operands.data_ptr(),
+                                          cycles.data_ptr(), stream), "mfma probe")
+    ms, _ = steady_window_ms(call, repeats, warm_ms)
+    flops = 256 * 4 * waves_per_simd * steps * 131072
+    clk = cycles[:256].double().mean().item()
+    return {"mfma": f"{shape}x{shape}x{512 // shape}_bf16", "lds_reads_per_step": lds_reads,
+            "waves_per_simd": waves_per_simd, "tflops": flops / ms / 1e9, "ghz": clk / (ms * 1e6),
+            "cycles_per_step_per_simd": clk / steps / waves_per_simd, "us_per_launch": ms * 1e3}
+
+
+def run_mfma_probe(steps: int = 4096, repeats: int = 20) -> list[dict[str, Any]]:
+    """Sustained matrix-core rate and shader clock of this chip, with random and with constant
+    operands, at 1, 2 and 4 wavefronts per SIMD, with and without LDS fragment reads beside the
+    MFMAs.  This is the ceiling the fused GEMM kernels can be read against: the paper peak assumes
+    2.4 GHz, the clock under full matrix-core load is lower and depends on the operand data."""
+    dev = torch.device("cuda:0")
     patterns = {"random": torch.randn(32768, device=dev).to(torch.bfloat16),
                 "constant": torch.full((32768,), 1.0, device=dev, dtype=torch.bfloat16)}
     rows = []
@@ -219,16 +235,7 @@ def run_mfma_probe(steps: int = 4096, repeats: int = 20) -> list[dict[str, Any]]
         for shape in (16, 32):
             for reads in (0, 4):
                 for wps in (1, 2, 4):
-                    def call():
-                        _lib.check(lib.mi_debug_mfma_rate(shape, reads, wps, steps, ops.data_ptr(),
-                                                          cycles.data_ptr(), stream), "mfma probe")
-                    ms, _ = steady_window_ms(call, repeats, 30.0)  # past the clock ramp
-                    flops = 256 * 4 * wps * steps * 131072
-                    clk = cycles[:256].double().mean().item()
-                    row = {"operands": pname, "mfma": f"{shape}x{shape}x{512 // shape}_bf16",
-                           "lds_reads_per_step": reads, "waves_per_simd": wps,
-                           "tflops": flops / ms / 1e9, "ghz": clk / (ms * 1e6),
-                           "cycles_per_step_per_simd": clk / steps / wps}
+                    row = {"operands": pname, **mfma_probe(shape, reads, wps, ops, steps, repeats)}
                     rows.append(row)
                     print(f"{pname:8s} {row['mfma']:14s} reads/step {reads} waves/SIMD {wps}: "
                           f"{row['tflops']:7.1f} TFLOP/s  {row['ghz']:.2f} GHz  "

@@ -131,6 +131,12 @@ def main() -> int:
         # the reference's "Baseline (Unfused)" (fusion_pipelined.cu:640-656): transform kernel, H(X)
         # through HBM, then the GEMM (here the vendor library's)
         un_ms, _ = steady_ms(lambda: torch.matmul(W, hada.hadamard_transform(Xt).t()), gsteps)
+        # what this box sustains with nothing but MFMAs (random bf16 operands, one wavefront per
+        # SIMD with four LDS fragment reads per step, the regime of the fused kernel), and the
+        # launch-to-launch time of a kernel that does next to nothing
+        harness = importlib.import_module("6s894_project_2025_amd.harness")
+        probe = harness.mfma_probe(16, 4, 1, Xt.reshape(-1)[:32768], 4096, 20, 30.0)
+        floor = harness.mfma_probe(16, 0, 1, Xt.reshape(-1)[:32768], 4, 200, 0.0)
         result.update({
             "metric": BASELINE_METRIC,
             "value": round(tf, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": gsteps, "warmup": warmup,
@@ -148,6 +154,13 @@ def main() -> int:
             "library_gemm_without_transform_tflops": round(flops / mm_ms / 1e9, 1),
             "unfused_transform_then_library_gemm_ms": round(un_ms, 6),
             "fused_over_unfused_speedup": round(un_ms / ms, 3),
+            "matrix_core_probe": {
+                "sustained_tflops": round(probe["tflops"], 1), "shader_ghz": round(probe["ghz"], 3),
+                "frac_of_peak": round(probe["tflops"] / PEAK_TFLOPS["bf16"], 4),
+                "note": "back-to-back v_mfma_f32_16x16x32_bf16 on every SIMD from registers, random bf16 "
+                        "operands (mi_debug_mfma_rate): the rate this box sustains under full matrix-core "
+                        "load; value / sustained_tflops = " + str(round(tf / probe["tflops"], 3))},
+            "launch_floor_us": round(floor["us_per_launch"], 2),
         })
         del W, Xt, C
 
