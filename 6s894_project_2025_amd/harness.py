@@ -5,6 +5,7 @@ Sub-commands (run from the repository root)::
     python -m 6s894_project_2025_amd.harness fwht  [--check] [--runs-per-size 400] [--sizes ...]
     python -m 6s894_project_2025_amd.harness fused [--dtype bf16|f32] [--runs 8] [--out-prefix P]
     python -m 6s894_project_2025_amd.harness plot P.csv [--out-dir plots]
+    python -m 6s894_project_2025_amd.harness gemv  [--iters 100] [--out-prefix P]
     python -m 6s894_project_2025_amd.harness mfma  [--steps 4096]
 
 ``fwht`` follows the protocol of the reference's bench/bench.py: a registry of in-place cases
@@ -22,6 +23,10 @@ unfused baseline next to the fused kernel the way fused_ht/fusion_pipelined.cu:6
 "transform kernel, then GEMM" (here: ``hadamard_transform`` + ``torch.matmul``, i.e. the vendor
 GEMM) versus ``fused_ht_gemm``; min over runs after 2 warm-ups (:631-683), max-abs difference
 between the two reported like :694-703.
+
+``gemv`` is the benchmark half of fused_ht/fwht_gemv_fusion.cu's main() (:643-653): its seven
+(M, N, B) shapes, fused HT+GEMV against transform-then-GEMM, with its FLOP count and its
+memory-traffic model (:576-588).
 """
 from __future__ import annotations
 
@@ -37,7 +42,7 @@ from typing import Any, Callable
 
 import torch
 
-from .ops import fused_ht_gemm, hadamard_transform
+from .ops import fused_ht_gemm, fused_ht_gemv, hadamard_transform
 from .timing import best_single_call_ms, event_window_ms, steady_window_ms
 
 ATOL = {torch.float16: 1e-2, torch.bfloat16: 5e-2, torch.float32: 1e-4}
@@ -199,6 +204,54 @@ def run_fused(dtype: torch.dtype, runs: int = 8, configs=None, out_prefix: str |
     return rows
 
 
+# (M, N, B) of fused_ht/fwht_gemv_fusion.cu:643-653
+GEMV_CONFIGS = [(256, 256, 512), (512, 512, 1024), (1024, 1024, 2048), (1024, 1024, 256),
+                (2048, 2048, 512), (64, 128, 256), (128, 256, 512)]
+
+
+def gemv_metrics(M: int, N: int, B: int) -> dict[str, float]:
+    """The reference's accounting for one fused HT+GEMV shape (fused_ht/fwht_gemv_fusion.cu:576-588):
+    N log2 N B butterfly operations plus 2 M N B for the product; the unfused path writes H(X) and
+    reads it back, the fused path does not."""
+    unfused = 4 * (M * N + 3 * N * B + M * B)
+    fused = 4 * (M * N + N * B + M * B)
+    return {"flops": N * (N.bit_length() - 1) * B + 2.0 * M * N * B, "bytes_unfused": unfused,
+            "bytes_fused": fused, "saved_fraction": (unfused - fused) / unfused}
+
+
+def run_gemv(configs=None, warmup: int = 10, iters: int = 100, out_prefix: str | None = None):
+    """Fused HT+GEMV against the unfused path on the reference's shapes and protocol
+    (fused_ht/fwht_gemv_fusion.cu:323-411,521-553: 10 warm-up and 100 timed back-to-back runs, fp32,
+    un-normalised transform, uniform [0,1) inputs).  The unfused path is the library's own
+    transform down the columns (on an untimed transposed copy of X) followed by the vendor GEMM."""
+    rows = []
+    g = torch.Generator().manual_seed(42)
+    for (M, N, B) in configs or GEMV_CONFIGS:
+        W = torch.rand(M, N, generator=g).cuda()
+        X = torch.rand(N, B, generator=g).cuda()
+        Xcols = X.t().contiguous()
+        fused = lambda: fused_ht_gemv(W, X, 1.0)
+        unfused = lambda: torch.matmul(W, hadamard_transform(Xcols, 1.0).t())
+        t_f, _ = event_window_ms(fused, iters, warmup)
+        t_u, _ = event_window_ms(unfused, iters, warmup)
+        yu = unfused()
+        diff = (fused() - yu).abs().max().item()
+        m = gemv_metrics(M, N, B)
+        print(f"M={M:5d} N={N:5d} B={B:5d}  unfused {t_u * 1e3:8.1f} us ({m['flops'] / t_u / 1e6:9.1f} GFLOPS)  "
+              f"fused {t_f * 1e3:8.1f} us ({m['flops'] / t_f / 1e6:9.1f} GFLOPS)  speedup {t_u / t_f:5.2f}x  "
+              f"memory saved {100 * m['saved_fraction']:.1f} %  max|diff| {diff:.3e} (scale {yu.abs().max().item():.3e})")
+        rows.append({"M": M, "N": N, "B": B, "unfused_ms": t_u, "fused_ms": t_f, "speedup": t_u / t_f,
+                     "fused_gflops": m["flops"] / t_f / 1e6, "unfused_gflops": m["flops"] / t_u / 1e6,
+                     "memory_saved_fraction": m["saved_fraction"], "max_error": diff,
+                     "max_abs_reference": yu.abs().max().item()})
+        del W, X, Xcols
+    if out_prefix:
+        with open(out_prefix + ".json", "w") as f:
+            json.dump(rows, f, indent=2)
+        print(f"Wrote {out_prefix}.json")
+    return rows
+
+
 def mfma_probe(shape: int, lds_reads: int, waves_per_simd: int, operands: torch.Tensor,
                steps: int = 4096, repeats: int = 20, warm_ms: float = 30.0) -> dict[str, Any]:
     """One configuration of ``mi_debug_mfma_rate``: nothing but back-to-back bf16 MFMAs on every
@@ -298,6 +351,9 @@ def main(argv=None) -> int:
     p2.add_argument("--dtype", default="bf16", choices=list(DTYPES))
     p2.add_argument("--runs", type=int, default=8)
     p2.add_argument("--out-prefix", default=None)
+    p5 = sub.add_parser("gemv")
+    p5.add_argument("--iters", type=int, default=100)
+    p5.add_argument("--out-prefix", default=None)
     p4 = sub.add_parser("mfma")
     p4.add_argument("--steps", type=int, default=4096)
     p3 = sub.add_parser("plot")
@@ -313,6 +369,9 @@ def main(argv=None) -> int:
         return 2
     if args.cmd == "mfma":
         run_mfma_probe(args.steps)
+        return 0
+    if args.cmd == "gemv":
+        run_gemv(iters=args.iters, out_prefix=args.out_prefix)
         return 0
     if args.cmd == "fwht":
         run_fwht(TestConfig(check=args.check, runs_per_size=args.runs_per_size,

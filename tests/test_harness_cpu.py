@@ -31,6 +31,17 @@ def test_sweep_metrics_known_values(harness):
     assert g2 == pytest.approx(2 * gflops) and b2 == pytest.approx(gbps)
 
 
+def test_gemv_shapes_and_metrics(harness):
+    # the seven shapes of fused_ht/fwht_gemv_fusion.cu:643-653 and its accounting (:576-588)
+    assert harness.GEMV_CONFIGS == [(256, 256, 512), (512, 512, 1024), (1024, 1024, 2048),
+                                    (1024, 1024, 256), (2048, 2048, 512), (64, 128, 256), (128, 256, 512)]
+    m = harness.gemv_metrics(256, 256, 512)
+    assert m["flops"] == 256 * 8 * 512 + 2 * 256 * 256 * 512
+    assert m["bytes_fused"] == 4 * (256 * 256 + 256 * 512 + 256 * 512)
+    assert m["bytes_unfused"] - m["bytes_fused"] == 4 * 2 * 256 * 512   # H(X) written and read back
+    assert abs(m["saved_fraction"] - 2 * 256 * 512 / (256 * 256 + 3 * 256 * 512 + 256 * 512)) < 1e-12
+
+
 def test_case_registry_and_tolerances(harness):
     assert list(harness.CASES) == ["AddOne1", "AddOne2", "Ours", "AddOne3"]
     assert harness.ATOL[torch.float16] == 1e-2 and harness.ATOL[torch.bfloat16] == 5e-2

@@ -75,6 +75,16 @@ def test_fused_sweep_small(harness, dtype, tmp_path):
     assert (tmp_path / "s.csv").read_text().startswith("kdim,ndim,mdim")
 
 
+def test_gemv_table_small(harness, tmp_path):
+    rows = harness.run_gemv(configs=[(64, 128, 256), (256, 256, 512)], warmup=2, iters=5,
+                            out_prefix=str(tmp_path / "gemv"))
+    assert len(rows) == 2 and (tmp_path / "gemv.json").exists()
+    for r in rows:
+        # the reference's own bar between its fused and unfused results (fwht_gemv_fusion.cu:293)
+        assert r["max_error"] <= 1e-3 * max(1.0, r["max_abs_reference"])
+        assert r["fused_ms"] > 0 and r["unfused_ms"] > 0
+
+
 def test_mfma_probe_reports_a_plausible_ceiling(harness):
     # the probe is the measured ceiling for the matrix-core-bound kernels: rates between a third of
     # the 2516.6 TFLOP/s paper peak and the peak itself, a clock between 1 and 2.5 GHz, and never
