@@ -297,8 +297,11 @@ def run_mfma_probe(steps: int = 4096, repeats: int = 20) -> list[dict[str, Any]]
 
 
 def plot_fused(csv_path: str, out_dir: str = "plots") -> list[str]:
-    """Figures from the sweep CSV, the counterpart of fused_ht/plot_results.py: speed-up of the fused
-    kernel over the unfused baseline against K for every N = M, and achieved TFLOP/s of both."""
+    """Figures and a table from the sweep CSV, the counterpart of the five outputs of
+    fused_ht/plot_results.py (speed-up by dimension :23-68, rate / time comparison :72-125, speed-up
+    map :129-258, bandwidth :262-304, summary table :308-365): speed-up and TFLOP/s against K for
+    every N = M, times of both paths per shape, the speed-up grid over (K, N = M), bandwidth under
+    the reference's byte model, and the summary as a Markdown table."""
     import os
 
     import matplotlib
@@ -309,18 +312,31 @@ def plot_fused(csv_path: str, out_dir: str = "plots") -> list[str]:
         rows = [{k: (v if k == "dtype" else float(v)) for k, v in r.items()} for r in csv.DictReader(f)]
     os.makedirs(out_dir, exist_ok=True)
     sizes = sorted({int(r["ndim"]) for r in rows})
+    kdims = sorted({int(r["kdim"]) for r in rows})
+    by_shape = {(int(r["kdim"]), int(r["ndim"])): r for r in rows}
     written = []
+
+    def finish(fig, name):
+        path = os.path.join(out_dir, name)
+        fig.tight_layout()
+        fig.savefig(path, dpi=120)
+        plt.close(fig)
+        written.append(path)
+
+    # lines against K, one per N = M
     for key, ylabel, name in (("speedup", "fused / unfused speed-up", "speedup_vs_k.png"),
-                              ("fused_gflops", "TFLOP/s", "tflops_vs_k.png")):
+                              ("fused_gflops", "TFLOP/s", "tflops_vs_k.png"),
+                              ("fused_bandwidth_gbps", "GB/s of operands and result (fused)",
+                               "bandwidth_vs_k.png")):
         fig, ax = plt.subplots(figsize=(7, 4.5))
         for n in sizes:
             sub = sorted((r for r in rows if int(r["ndim"]) == n), key=lambda r: r["kdim"])
             ks = [r["kdim"] for r in sub]
-            if key == "speedup":
-                ax.plot(ks, [r[key] for r in sub], "o-", label=f"N=M={n}")
-            else:
+            if key == "fused_gflops":
                 ax.plot(ks, [r["fused_gflops"] / 1e3 for r in sub], "o-", label=f"fused N=M={n}")
                 ax.plot(ks, [r["baseline_gflops"] / 1e3 for r in sub], "s--", label=f"unfused N=M={n}")
+            else:
+                ax.plot(ks, [r[key] for r in sub], "o-", label=f"N=M={n}")
         if key == "speedup":
             ax.axhline(1.0, color="gray", linewidth=0.8)
         ax.set_xscale("log", base=2)
@@ -328,11 +344,50 @@ def plot_fused(csv_path: str, out_dir: str = "plots") -> list[str]:
         ax.set_ylabel(ylabel)
         ax.grid(True, alpha=0.3)
         ax.legend(fontsize=8)
-        path = os.path.join(out_dir, name)
-        fig.tight_layout()
-        fig.savefig(path, dpi=120)
-        plt.close(fig)
-        written.append(path)
+        finish(fig, name)
+
+    # both paths' time per shape, side by side
+    fig, ax = plt.subplots(figsize=(max(7, 0.6 * len(rows)), 4.5))
+    order = sorted(by_shape)
+    pos = range(len(order))
+    ax.bar([p - 0.2 for p in pos], [by_shape[s]["baseline_ms"] * 1e3 for s in order], 0.4, label="unfused")
+    ax.bar([p + 0.2 for p in pos], [by_shape[s]["fused_ms"] * 1e3 for s in order], 0.4, label="fused")
+    ax.set_xticks(list(pos))
+    ax.set_xticklabels([f"K={k}\nN=M={n}" for k, n in order], fontsize=7)
+    ax.set_ylabel("microseconds per call")
+    ax.set_yscale("log")
+    ax.legend()
+    finish(fig, "time_per_shape.png")
+
+    # speed-up over the (K, N = M) grid
+    fig, ax = plt.subplots(figsize=(1.2 * len(kdims) + 2, 0.9 * len(sizes) + 2))
+    grid = [[by_shape.get((k, n), {"speedup": float("nan")})["speedup"] for k in kdims] for n in sizes]
+    im = ax.imshow(grid, cmap="RdYlGn", vmin=0.25, vmax=2.0, aspect="auto")
+    ax.set_xticks(range(len(kdims)))
+    ax.set_xticklabels(kdims)
+    ax.set_yticks(range(len(sizes)))
+    ax.set_yticklabels(sizes)
+    ax.set_xlabel("K")
+    ax.set_ylabel("N = M")
+    for i in range(len(sizes)):
+        for j in range(len(kdims)):
+            ax.text(j, i, f"{grid[i][j]:.2f}", ha="center", va="center", fontsize=9)
+    fig.colorbar(im, ax=ax, label="fused / unfused speed-up")
+    finish(fig, "speedup_grid.png")
+
+    # the summary as text
+    path = os.path.join(out_dir, "summary.md")
+    with open(path, "w") as f:
+        f.write("| K | N = M | dtype | unfused us | fused us | speed-up | fused TFLOP/s | max abs diff |\n")
+        f.write("|---|---|---|---|---|---|---|---|\n")
+        for (k, n) in order:
+            r = by_shape[(k, n)]
+            f.write(f"| {k} | {n} | {r['dtype']} | {r['baseline_ms'] * 1e3:.1f} | {r['fused_ms'] * 1e3:.1f} | "
+                    f"{r['speedup']:.2f} | {r['fused_gflops'] / 1e3:.1f} | {r['max_error']:.3g} |\n")
+        wins = [r["speedup"] for r in rows if r["speedup"] >= 1.0]
+        f.write(f"\nfused faster on {len(wins)} of {len(rows)} shapes; best {max(r['speedup'] for r in rows):.2f}x, "
+                f"worst {min(r['speedup'] for r in rows):.2f}x\n")
+    written.append(path)
     return written
 
 

@@ -75,7 +75,11 @@ def test_plot_from_sweep_csv(harness, tmp_path):
         w.writeheader()
         w.writerows(rows)
     out = harness.plot_fused(str(path), str(tmp_path / "plots"))
-    assert len(out) == 2
+    names = sorted(p.split("/")[-1] for p in out)
+    assert names == sorted(["bandwidth_vs_k.png", "speedup_grid.png", "speedup_vs_k.png", "summary.md",
+                            "time_per_shape.png", "tflops_vs_k.png"])
     for p in out:
-        assert (tmp_path / "plots" / p.split("/")[-1]).stat().st_size > 1000
+        assert (tmp_path / "plots" / p.split("/")[-1]).stat().st_size > (1000 if p.endswith(".png") else 300)
+    text = (tmp_path / "plots" / "summary.md").read_text()
+    assert "| 1024 | 4096 | bfloat16 | 50.0 | 40.0 | 1.25 | 500.0 |" in text and "fused faster on 6 of 6 shapes" in text
     assert harness.main(["plot", str(path), "--out-dir", str(tmp_path / "p2")]) == 0
