@@ -24,7 +24,7 @@ SIGNATURES = {
     "mi_debug_convert": (_i, [_i, _vp, _vp, _u64, _vp]),
     "mi_debug_device_fwht": (_i, [_vp, _vp, _u64, _u32, _i, _f, _vp]),
     "mi_debug_mfma_rate": (_i, [_i, _i, _u32, _u32, _vp, _vp, _vp]),
-    "mi_debug_fused_gemm_tiling": (_i, [_u32, _u32, _vp, _vp, _u32]),
+    "mi_debug_fused_gemm_tiling": (_i, [_u32, _u32, _u32, _vp, _vp, _u32]),
 }
 
 _lib = None

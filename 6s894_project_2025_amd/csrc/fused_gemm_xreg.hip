@@ -1,14 +1,15 @@
 // Fused Hadamard -> GEMM with the transformed operand held in registers, gfx950, 16-bit inputs:
-//     C[M,N] = W[M,K] * (scale * H_K * X[K,N]),  X given as Xt[N,K],  K = 1024.
+//     C[M,N] = W[M,K] * (scale * H_K * X[K,N]),  X given as Xt[N,K],  K = 512 or 1024.
 //
 // One workgroup = four wavefronts, one per SIMD, each with the whole 512-register budget.
-//   prologue : wavefront w transforms 32 columns of X on the matrix cores (coalesced 16-byte
-//              loads, the two-stage tile transform of fwht_device.hpp with the last butterfly
-//              folded into the second stage), passes them once through a wavefront-private LDS
-//              area to get from "a lane owns 8 consecutive k of one column" to MFMA operand order
-//              "lane (hi, lo) owns 8 consecutive k of column lo", and keeps all K x 32 values in
-//              the 256 accumulation registers for the rest of the kernel.  The workgroup
-//              therefore owns 128 columns, twice what fits in LDS.
+//   prologue : wavefront w transforms 32768 / K columns of X (32 at K = 1024, 64 at K = 512) on the
+//              matrix cores (coalesced 16-byte loads, the two-stage tile transform of
+//              fwht_device.hpp; at K = 1024 the last butterfly is folded into the second stage),
+//              passes them once through a wavefront-private LDS area to get from "a lane owns 8
+//              consecutive k of one column" to MFMA operand order "lane (hi, lo) owns 8
+//              consecutive k of column lo", and keeps all 32768 values in the 256 accumulation
+//              registers for the rest of the kernel.  The workgroup therefore owns 128 (256)
+//              columns, twice what fits in LDS.
 //   main loop: the workgroup walks its M range in 64-row blocks.  W is the only operand that
 //              moves: global -> LDS directly (no register hop), each wavefront fetching a quarter
 //              of a 64-row x 256-K stage as whole 512-byte row segments into a ring of four
@@ -37,7 +38,6 @@ namespace mi {
 namespace xreg {
 
 constexpr int kThreads = 256;
-constexpr int kCols = 128;                        // columns of X per workgroup
 constexpr int kRows = 64;                         // rows of W per row block
 constexpr int kStageK = 256;                      // K extent of one W stage
 constexpr int kStageBytes = kRows * kStageK * 2;  // 32 KB
@@ -50,6 +50,20 @@ constexpr int kAreaBase = 3 * kStageBytes;
 constexpr int kLdsBytes = kAreaBase + 4 * kAreaBytes;
 
 typedef __attribute__((address_space(3))) void* lptr_t;
+
+// What follows from K: the transformed operand of a wavefront always fills its 256 accumulation
+// registers (64 fragments of 16 columns x 32 k).
+template <int K>
+struct Geom {
+    static_assert(K == 512 || K == 1024, "register budget: 16 NBF columns x K = 32768 values per wavefront");
+    static constexpr int NBF = 2048 / K;            // 16-column fragments per wavefront
+    static constexpr int CPW = 16 * NBF;            // columns per wavefront
+    static constexpr int COLS = 4 * CPW;            // columns per workgroup
+    static constexpr int KSTEPS = K / 32;           // MFMA K steps per row block
+    static constexpr int SPB = K / kStageK;         // W stages per row block
+    static constexpr int AHEAD = SPB >= 3 ? 3 : 2;  // stages the W stream runs ahead of the MFMAs
+    static constexpr int NM = 4 * NBF;              // MFMAs per K step
+};
 
 // LDS image of a W stage: [64 rows][512 B], the 16-byte chunk q of row r stored at q ^ (r & 15).
 __host__ __device__ constexpr uint32_t stage_offset(uint32_t row, uint32_t q)
@@ -112,14 +126,32 @@ struct XMfma<F16> {
     }
 };
 
-// Waits out the matrix-core pipeline before `acc` is read by anything but an MFMA.  The
-// accumulators pass through the statement, so that the compiler cannot move a read of them (a
-// register copy, say) above the wait.
+// Waits out the matrix-core pipeline before `acc` is read by anything but an MFMA.  Two statements:
+// the delay itself, which names no register (naming them lets the compiler set the operands up
+// with register copies *in front of* the statement, i.e. reads of the accumulators right behind
+// the last MFMA: observed with sixteen accumulators), and an empty statement that the
+// accumulators pass through, so that no read of them (a register copy, say) can move above the
+// delay.
+__device__ __forceinline__ void mfma_delay()
+{
+    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
 __device__ __forceinline__ void drain_mfma(f32x4 (&acc)[4][2])
 {
-    asm volatile("s_nop 15\n\ts_nop 7"
+    mfma_delay();
+    asm volatile(""
                  : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[1][0]), "+v"(acc[1][1]),
                    "+v"(acc[2][0]), "+v"(acc[2][1]), "+v"(acc[3][0]), "+v"(acc[3][1]));
+}
+__device__ __forceinline__ void drain_mfma(f32x4 (&acc)[4][4])
+{
+    mfma_delay();
+    asm volatile(""
+                 : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]), "+v"(acc[0][3]),
+                   "+v"(acc[1][0]), "+v"(acc[1][1]), "+v"(acc[1][2]), "+v"(acc[1][3]),
+                   "+v"(acc[2][0]), "+v"(acc[2][1]), "+v"(acc[2][2]), "+v"(acc[2][3]),
+                   "+v"(acc[3][0]), "+v"(acc[3][1]), "+v"(acc[3][2]), "+v"(acc[3][3]));
 }
 
 // A column = two 512-element tiles.  Stage 1 as in tile_transform; stage 2 contracts the two
@@ -206,6 +238,12 @@ __device__ __forceinline__ void stream_store8(uint32_t lane_off, u32x2 v, void* 
 {
     asm volatile("global_store_dwordx2 %0, %1, %2 nt" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
 }
+// (A store of more than 8 bytes still reads its data registers during the next cycles; the compiler
+// keeps ordinary code away from them for that long, but does not know what this statement is.)
+__device__ __forceinline__ void stream_store16(uint32_t lane_off, u32x4 v, void* base)
+{
+    asm volatile("global_store_dwordx4 %0, %1, %2 nt\n\ts_nop 1" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
+}
 
 // Workgroup id -> (column group, M slice); false for an id past the last rectangle.
 __host__ __device__ inline bool tile_of_workgroup(uint32_t id, uint32_t msplit, uint32_t mpx, uint32_t cgx,
@@ -231,10 +269,11 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     using E = typename T16::E;
     using V8 = typename T16::V8;
     typedef E V2 __attribute__((ext_vector_type(2)));
-    static_assert(K == 1024, "register budget: 32 columns x K / 128 = 256 registers per lane");
-    constexpr int KSTEPS = K / 32;
-    constexpr int SPB = K / kStageK;  // stages per row block
-    static_assert(SPB == kSlots, "the stage buffer of a stage is its K quarter");
+    typedef E V4 __attribute__((ext_vector_type(4)));
+    using G = Geom<K>;
+    constexpr int NBF = G::NBF, KSTEPS = G::KSTEPS, SPB = G::SPB, AHEAD = G::AHEAD, NM = G::NM;
+    constexpr uint32_t kCols = G::COLS, CPW = G::CPW;
+    static_assert(kSlots == 4 && AHEAD <= SPB && AHEAD + 1 <= kSlots, "stage g lives in buffer g % 4");
     constexpr uint32_t ROW_BYTES = K * 2u;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -264,7 +303,7 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     };
 
     // ---- W stream -------------------------------------------------------------------------------
-    // Stage g = (row block g / 4, K quarter g % 4) lives in stage buffer g % 4.  Wavefront w moves
+    // Stage g = (row block g / SPB, K range 256 (g % SPB) ...) lives in stage buffer g % 4.  Wavefront w moves
     // rows 16w .. 16w+15 of the block in eight pieces; piece i = rows 2i, 2i+1: lane l fetches row
     // 2i + l/32 and lands at byte 16 l of the piece's 1 KB of LDS (the transfer's fixed lane order).
     // LDS stage image: [64 rows][512 B] with 16-byte chunk q of row r stored at q ^ (r & 15), so
@@ -287,62 +326,97 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     };
     set_voff(0);
 
-    // ---- prologue: Y fragments of this wavefront's 32 columns ------------------------------------
-    // Column of fragment nb, fragment column j (= MFMA B column = lane lo): n0 + 32w + 2j + nb, so
-    // that a lane ends up with pairs of adjacent output columns.
-    V8 yf[2][KSTEPS];
+    // ---- prologue: Y fragments of this wavefront's columns ---------------------------------------
+    // Column of fragment nb, fragment column j (= MFMA B column = lane lo): n0 + CPW w + NBF j + nb,
+    // so that a lane ends up with NBF adjacent output columns.  One round = the 16 columns of one
+    // fragment index; the tiles of the next round are requested as this round's are consumed, and
+    // the first AHEAD stages of W behind the last X tile (vector memory operations complete in
+    // order, so anything issued earlier would hold the tiles back), two pieces per column of the
+    // last round, while its tiles arrive.
+    V8 yf[NBF][KSTEPS];
     {
-        PairOperands<T16> po;
-        make_pair_operands<T16>(po, exp2);
         unsigned char* area = lds + kAreaBase + wave * kAreaBytes;
-        // the 32 tiles of a round are all in flight at once (128 registers); the tiles of the
-        // second round are requested as the first round's are consumed
-        V8 in[16][2];
-        auto load_col = [&](int nb, int j) {
-            const uint32_t col = min(n0 + 32u * wave + 2u * j + nb, N - 1u);
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-                in[j][t] = *reinterpret_cast<const V8*>(Xt + ((uint64_t)col * K + 512u * t + 8u * lane));
-        };
-#pragma unroll
-        for (int j = 0; j < 16; ++j) load_col(0, j);
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
-            V8 hold[16];  // second halves (k >= 512) wait here while the first go through LDS
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                V8 first_half;
-                column_transform<T16>(in[j][0], in[j][1], po, first_half, hold[j]);
-                if (nb == 0) load_col(1, j);
-                // The first three W stages are requested behind the last X tile (vector memory
-                // operations complete in order, so anything issued earlier would hold the tiles
-                // back), two pieces per column of the second round, while its tiles arrive.
-                if (nb == 1 && j >= 2 && j < 14) {
-                    const int p = 2 * (j - 2);
-                    w_issue(p >> 3, p >> 3, p & 7);
-                    w_issue((p + 1) >> 3, (p + 1) >> 3, (p + 1) & 7);
-                }
-                // area: [16 columns][64 chunks of 16 B], chunk q of column j stored at q ^ j
-                *reinterpret_cast<V8*>(area + area_offset(j, lane)) = first_half;
+        auto prefetch_w = [&](int nb, int j) __attribute__((always_inline)) {
+            if (nb == NBF - 1 && j >= 2 && j < 2 + 4 * AHEAD) {
+                const int p = 2 * (j - 2);
+                w_issue(p >> 3, p >> 3, p & 7);
+                w_issue((p + 1) >> 3, (p + 1) >> 3, (p + 1) & 7);
             }
-            // LDS operations of one wavefront complete in order: no barrier between its own
-            // writes and reads
+        };
+        if constexpr (K == 1024) {
+            PairOperands<T16> po;
+            make_pair_operands<T16>(po, exp2);
+            V8 in[16][2];
+            auto load_col = [&](int nb, int j) {
+                const uint32_t col = min(n0 + CPW * wave + (uint32_t)(NBF * j + nb), N - 1u);
 #pragma unroll
-            for (int s = 0; s < KSTEPS / 2; ++s)
-                yf[nb][s] = *reinterpret_cast<const V8*>(area + area_offset(lo, 4u * s + hi));
+                for (int t = 0; t < 2; ++t)
+                    in[j][t] = *reinterpret_cast<const V8*>(Xt + ((uint64_t)col * K + 512u * t + 8u * lane));
+            };
 #pragma unroll
-            for (int j = 0; j < 16; ++j)
-                *reinterpret_cast<V8*>(area + area_offset(j, lane)) = hold[j];
+            for (int j = 0; j < 16; ++j) load_col(0, j);
 #pragma unroll
-            for (int s = 0; s < KSTEPS / 2; ++s)
-                yf[nb][KSTEPS / 2 + s] =
-                    *reinterpret_cast<const V8*>(area + area_offset(lo, 4u * s + hi));
+            for (int nb = 0; nb < NBF; ++nb) {
+                V8 hold[16];  // second halves (k >= 512) wait here while the first go through LDS
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    V8 first_half;
+                    column_transform<T16>(in[j][0], in[j][1], po, first_half, hold[j]);
+                    if (nb + 1 < NBF) load_col(nb + 1, j);
+                    prefetch_w(nb, j);
+                    // area: [16 columns][64 chunks of 16 B], chunk q of column j stored at q ^ j
+                    *reinterpret_cast<V8*>(area + area_offset(j, lane)) = first_half;
+                }
+                // LDS operations of one wavefront complete in order: no barrier between its own
+                // writes and reads
+#pragma unroll
+                for (int s = 0; s < KSTEPS / 2; ++s)
+                    yf[nb][s] = *reinterpret_cast<const V8*>(area + area_offset(lo, 4u * s + hi));
+#pragma unroll
+                for (int j = 0; j < 16; ++j)
+                    *reinterpret_cast<V8*>(area + area_offset(j, lane)) = hold[j];
+#pragma unroll
+                for (int s = 0; s < KSTEPS / 2; ++s)
+                    yf[nb][KSTEPS / 2 + s] =
+                        *reinterpret_cast<const V8*>(area + area_offset(lo, 4u * s + hi));
+            }
+        } else {  // K = 512: a column is one tile
+            TileOperands<T16> ops;
+            make_tile_operands<T16, 2>(9, ops, exp2);
+            V8 in[16];
+            auto load_col = [&](int nb, int j) {
+                const uint32_t col = min(n0 + CPW * wave + (uint32_t)(NBF * j + nb), N - 1u);
+                in[j] = *reinterpret_cast<const V8*>(Xt + ((uint64_t)col * K + 8u * lane));
+            };
+#pragma unroll
+            for (int j = 0; j < 16; ++j) load_col(0, j);
+#pragma unroll
+            for (int nb = 0; nb < NBF; ++nb) {
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    f32x4 t2[2];
+                    tile_transform<T16>(in[j], ops, t2);
+                    V8 o;
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) o[4 * t + r] = (E)t2[t][r];
+                    if (nb + 1 < NBF) load_col(nb + 1, j);
+                    prefetch_w(nb, j);
+                    *reinterpret_cast<V8*>(area + area_offset(j, lane)) = o;
+                }
+#pragma unroll
+                for (int s = 0; s < KSTEPS; ++s)
+                    yf[nb][s] = *reinterpret_cast<const V8*>(area + area_offset(lo, 4u * s + hi));
+            }
         }
     }
 
     // Every wavefront has finished with its area (stage buffer 3 may be filled from now on), and
-    // its pieces of stage 0 have landed (the 16 pieces of stages 1 and 2 may still be in flight).
-    asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
+    // its pieces of stage 0 have landed (those of the AHEAD - 1 stages behind it may still be in
+    // flight).
+    wait_vm(8 * (AHEAD - 1));
+    wait_lds();
     __builtin_amdgcn_s_barrier();
 
     auto frag = [&](uint32_t slot, int mb, int ks) __attribute__((always_inline)) -> V8 {
@@ -357,30 +431,41 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     }
 
     // ---- output addressing ------------------------------------------------------------------------
-    // lane (hi, lo) of a row block owns rows 16 mb + 4 hi + r and the column pair 2 lo, 2 lo + 1 of
-    // its wavefront's 32 columns
+    // lane (hi, lo) of a row block owns rows 16 mb + 4 hi + r and the NBF adjacent columns
+    // NBF lo .. NBF lo + NBF - 1 of its wavefront's columns
     constexpr uint32_t esize = OUT_F32 ? 4u : 2u;
-    const uint32_t col = n0 + 32u * wave + 2u * lo;
+    const uint32_t col = n0 + CPW * wave + (uint32_t)NBF * lo;
     const uint32_t lane_off = (4u * hi * N + col) * esize;  // inside the row block, < 2^32
     unsigned char* const Cb = static_cast<unsigned char*>(C);
-    // `mult` is the part of the scale that is not a power of two: 1 for the usual scales, and only
-    // then do row blocks take the interleaved store path
-    const bool cols_full = n0 + kCols <= N && (N & 1u) == 0 && mult == 1.0f;
+    // `mult` is the part of the scale that is not a power of two (1 for K = 1024 and the usual
+    // n^-1/2, sqrt(2)-ish for K = 512); it is applied to the fp32 result at the store.  Row blocks
+    // of full column groups take the vector store path.
+    const bool cols_full = n0 + kCols <= N && (N % (uint32_t)NBF) == 0;
 
     // one store of the interleaved epilogue: rows 16 mb + 4 hi + r of a full row block
-    auto store_pair = [&](const f32x4 (&acc)[4][2], uint64_t block_base, int mb, int r)
+    auto store_pair = [&](const f32x4 (&acc)[4][NBF], uint64_t block_base, int mb, int r)
         __attribute__((always_inline)) {
-        const float v0 = acc[mb][0][r], v1 = acc[mb][1][r];
         // streaming stores: C is not read again, and keeping it out of the L2 leaves the cache to
         // the operands
         unsigned char* row_ptr = Cb + (block_base + (uint64_t)((16u * mb + r) * N) * esize);  // scalar
-        if (OUT_F32)
-            stream_store8(lane_off, u32x2{__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1)}, row_ptr);
-        else
-            stream_store4(lane_off, __builtin_bit_cast(uint32_t, V2{(E)v0, (E)v1}), row_ptr);
+        if constexpr (NBF == 2) {
+            const float v0 = acc[mb][0][r] * mult, v1 = acc[mb][1][r] * mult;
+            if (OUT_F32)
+                stream_store8(lane_off, u32x2{__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1)}, row_ptr);
+            else
+                stream_store4(lane_off, __builtin_bit_cast(uint32_t, V2{(E)v0, (E)v1}), row_ptr);
+        } else {
+            const float v0 = acc[mb][0][r] * mult, v1 = acc[mb][1][r] * mult, v2 = acc[mb][2][r] * mult,
+                        v3 = acc[mb][3][r] * mult;
+            if (OUT_F32)
+                stream_store16(lane_off, u32x4{__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1),
+                                               __builtin_bit_cast(uint32_t, v2), __builtin_bit_cast(uint32_t, v3)}, row_ptr);
+            else
+                stream_store8(lane_off, __builtin_bit_cast(u32x2, V4{(E)v0, (E)v1, (E)v2, (E)v3}), row_ptr);
+        }
     };
     // the same for a row block at the edge of the matrix (masked, element by element)
-    auto store_edge = [&](const f32x4 (&acc)[4][2], uint32_t row_base) __attribute__((always_inline)) {
+    auto store_edge = [&](const f32x4 (&acc)[4][NBF], uint32_t row_base) __attribute__((always_inline)) {
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
@@ -388,7 +473,7 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
                 const uint32_t row = row_base + 16u * mb + 4u * hi + r;
                 if (row >= m_end) continue;
 #pragma unroll
-                for (int nb = 0; nb < 2; ++nb) {
+                for (int nb = 0; nb < NBF; ++nb) {
                     if (col + nb >= N) continue;
                     const float v = acc[mb][nb][r] * mult;
                     const uint64_t at = (uint64_t)row * N + col + nb;
@@ -400,24 +485,36 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
             }
     };
 
-    // ---- one row block: 32 K steps into `acc`, while `prev` (the previous row block's result, when
-    // the tag says there is one) is stored two pieces per K step of the first stage ----------------
-    auto row_block_body = [&](auto prev_tag, f32x4 (&acc)[4][2], const f32x4 (&prev)[4][2],
-                              uint64_t prev_base, uint32_t rbi) __attribute__((always_inline)) {
+    // ---- one row block: KSTEPS K steps into `acc`, while `prev` (the previous row block's result,
+    // when the tag says there is one) is stored one piece behind each MFMA of the K steps that follow
+    // the first stage's barrier.  `second_tag`: the block is the second of its pair, whose stages
+    // continue the ring where the first block's stopped (buffer (SPB + kq) % 4). -------------------
+    auto row_block_body = [&](auto prev_tag, auto second_tag, f32x4 (&acc)[4][NBF],
+                              const f32x4 (&prev)[4][NBF], uint64_t prev_base, uint32_t rbi)
+        __attribute__((always_inline)) {
         constexpr bool prev_full = decltype(prev_tag)::value;
-        // the last row block requests only its own fourth stage: nothing follows it
+        constexpr int slot_base = decltype(second_tag)::value ? (SPB & 3) : 0;
+        // the last row block requests only its own remaining stages: nothing follows it
         const bool last = rbi + 1u == nrb;
 #pragma unroll
         for (int kq = 0; kq < SPB; ++kq) {
-            // pieces of stage g+3 issued during K step ks of this stage
+            // pieces of stage g+AHEAD issued during K step ks of this stage (everything below folds to
+            // constants once the loops are unrolled)
             constexpr int kPieceAt[7] = {0, 2, 4, 5, 6, 7, 8};
+            const int cur_slot = (slot_base + kq) & 3;
+            const int next_slot = (slot_base + kq + 1) & 3;
+            const int fill_slot = (slot_base + kq + AHEAD) & 3;
+            const int fill_kq = (kq + AHEAD) % SPB;
+            const bool fill_own_block = kq + AHEAD < SPB;
 #pragma unroll
             for (int ks = 0; ks < kStepsPerStage; ++ks) {
-                if (kq == 1 && ks == 0 && !last) set_voff(rbi + 1u);  // stages g+3: the next block's
+                // from the first stage whose transfers belong to the next row block on, the lane
+                // offsets are the next block's
+                if (kq == SPB - AHEAD && ks == 0 && !last) set_voff(rbi + 1u);
                 const int kk = kq * kStepsPerStage + ks;
 #pragma unroll
-                for (int m = 0; m < 8; ++m) {
-                    const int mb = m >> 1, nb = m & 1;
+                for (int m = 0; m < NM; ++m) {
+                    const int mb = m / NBF, nb = m % NBF;
                     if (kk == 0)
                         XMfma<T16>::first(acc[mb][nb], fr[ks & 3][mb], yf[nb][0]);
                     else
@@ -426,18 +523,18 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
                     if (m < 4) {
                         // fragments two K steps ahead; the last two steps of a stage read the
                         // first two of the next stage, behind the barrier
-                        fr[(ks + 2) & 3][m] = ks < 6 ? frag(kq, m, ks + 2) : frag((kq + 1) & 3, m, ks - 6);
+                        fr[(ks + 2) & 3][m] = ks < 6 ? frag(cur_slot, m, ks + 2) : frag(next_slot, m, ks - 6);
                     } else if (m < 6) {
-                        if (ks < 6 && (kq == 0 || !last)) {
+                        if (ks < 6 && (fill_own_block || !last)) {
                             const int i = kPieceAt[ks] + (m - 4);
-                            if (i < kPieceAt[ks + 1]) w_issue((kq + 3) & 3, (kq + 3) & 3, i);
+                            if (i < kPieceAt[ks + 1]) w_issue(fill_kq, fill_slot, i);
                         }
                     }
-                    // the previous block's sixteen stores, one behind each MFMA of the two K steps
-                    // that follow the first stage's barrier: they then have a whole stage to
+                    // the previous block's sixteen stores, one behind each MFMA of the K steps
+                    // that follow the first stage's barrier: they then have most of a stage to
                     // complete before the next barrier counts outstanding memory operations
-                    if (prev_full && kq == 0 && ks >= 6) {
-                        const int e = 8 * (ks - 6) + m;
+                    if (prev_full && kk >= 6 && kk < 6 + 16 / NM) {
+                        const int e = NM * (kk - 6) + m;
                         store_pair(prev, prev_base, e >> 2, e & 3);
                     }
                     __builtin_amdgcn_sched_barrier(0);
@@ -452,14 +549,15 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
                 if (ks == 5) {
                     // Own pieces of stage g+1 have landed.  Loads complete in order among
                     // themselves, but not relative to stores, so the count allowed to remain
-                    // outstanding is the number of *loads* requested after those pieces (8 of
-                    // stage g+2, 8 of stage g+3; fewer at the end of the last row block): pending
+                    // outstanding is the number of *loads* requested after those pieces (8 per
+                    // stage g+2 .. g+AHEAD; fewer at the end of the last row block): pending
                     // stores can only make this wait longer, never shorter.
-                    constexpr int kAfterLast[4] = {16, 8, 0, -1};
+                    const int later = SPB - kq - 2 < AHEAD - 1 ? SPB - kq - 2 : AHEAD - 1;
+                    const int after_last = kq == SPB - 1 ? -1 : 8 * (later > 0 ? later : 0);
                     if (last)
-                        wait_vm(kAfterLast[kq]);
+                        wait_vm(after_last);
                     else
-                        wait_vm(16);
+                        wait_vm(8 * (AHEAD - 1));
                     wait_lds();
                     __builtin_amdgcn_s_barrier();
                 }
@@ -467,53 +565,79 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
         }
     };
 
-    f32x4 accA[4][2], accB[4][2];
-    bool pend = false;        // accB holds a finished full row block that is not stored yet
-    uint64_t pend_base = 0;
-    auto run = [&](bool prev_full, f32x4 (&acc)[4][2], const f32x4 (&prev)[4][2], uint64_t prev_base,
-                   uint32_t rbi) __attribute__((always_inline)) {
-        if (prev_full)
-            row_block_body(std::true_type{}, acc, prev, prev_base, rbi);
-        else
-            row_block_body(std::false_type{}, acc, prev, prev_base, rbi);
-    };
-    auto finish = [&](f32x4 (&acc)[4][2], uint32_t rbi, bool& full, uint64_t& base)
-        __attribute__((always_inline)) {
-        // a full block is stored during the next block; an edge block right away
-        const uint32_t row_base = m_begin + row_block(rbi) * kRows;
-        full = cols_full && row_base + kRows <= m_end;
-        base = (uint64_t)row_base * N * esize;
-        if (!full) {
-            drain_mfma(acc);
-            store_edge(acc, row_base);
-        }
-    };
-#pragma unroll 1
-    for (uint32_t rbi = 0; rbi < nrb; rbi += 2u) {
-        run(pend, accA, accB, pend_base, rbi);
-        bool fullA;
-        uint64_t baseA;
-        finish(accA, rbi, fullA, baseA);
-        if (rbi + 1u < nrb) {
-            run(fullA, accB, accA, baseA, rbi + 1u);
-            finish(accB, rbi + 1u, pend, pend_base);
-        } else {
-            pend = false;
-            if (fullA) {
-                drain_mfma(accA);
-#pragma unroll
-                for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) store_pair(accA, baseA, mb, r);
-            }
-        }
-    }
-    if (pend) {
-        drain_mfma(accB);
+    auto store_block = [&](f32x4 (&acc)[4][NBF], uint64_t base) __attribute__((always_inline)) {
+        drain_mfma(acc);
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) store_pair(accB, pend_base, mb, r);
+            for (int r = 0; r < 4; ++r) store_pair(acc, base, mb, r);
+    };
+    auto block_place = [&](uint32_t rbi, bool& full, uint64_t& base, uint32_t& row_base)
+        __attribute__((always_inline)) {
+        row_base = m_begin + row_block(rbi) * kRows;
+        full = cols_full && row_base + kRows <= m_end;
+        base = (uint64_t)row_base * N * esize;
+    };
+    if constexpr (NBF <= 2) {
+        // Two accumulator sets take turns: a finished full block is stored during the next one.
+        f32x4 accA[4][NBF], accB[4][NBF];
+        bool pend = false;        // accB holds a finished full row block that is not stored yet
+        uint64_t pend_base = 0;
+        auto run = [&](bool prev_full, auto second_tag, f32x4 (&acc)[4][NBF], const f32x4 (&prev)[4][NBF],
+                       uint64_t prev_base, uint32_t rbi) __attribute__((always_inline)) {
+            if (prev_full)
+                row_block_body(std::true_type{}, second_tag, acc, prev, prev_base, rbi);
+            else
+                row_block_body(std::false_type{}, second_tag, acc, prev, prev_base, rbi);
+        };
+        auto finish = [&](f32x4 (&acc)[4][NBF], uint32_t rbi, bool& full, uint64_t& base)
+            __attribute__((always_inline)) {
+            // a full block is stored during the next block; an edge block right away
+            uint32_t row_base;
+            block_place(rbi, full, base, row_base);
+            if (!full) {
+                drain_mfma(acc);
+                store_edge(acc, row_base);
+            }
+        };
+#pragma unroll 1
+        for (uint32_t rbi = 0; rbi < nrb; rbi += 2u) {
+            run(pend, std::false_type{}, accA, accB, pend_base, rbi);
+            bool fullA;
+            uint64_t baseA;
+            finish(accA, rbi, fullA, baseA);
+            if (rbi + 1u < nrb) {
+                run(fullA, std::true_type{}, accB, accA, baseA, rbi + 1u);
+                finish(accB, rbi + 1u, pend, pend_base);
+            } else {
+                pend = false;
+                if (fullA) store_block(accA, baseA);
+            }
+        }
+        if (pend) store_block(accB, pend_base);
+    } else {
+        // Four column fragments: one accumulator set is all the register file has room for (a
+        // second one spilled), so a block is stored as soon as it is finished; with sixteen MFMAs
+        // per K step the sixteen stores and the drain cost a few per cent of a block.
+        f32x4 acc[4][NBF];
+        auto one = [&](auto second_tag, uint32_t rbi) __attribute__((always_inline)) {
+            row_block_body(std::false_type{}, second_tag, acc, acc, 0, rbi);
+            bool full;
+            uint64_t base;
+            uint32_t row_base;
+            block_place(rbi, full, base, row_base);
+            if (full) {
+                store_block(acc, base);
+            } else {
+                drain_mfma(acc);
+                store_edge(acc, row_base);
+            }
+        };
+#pragma unroll 1
+        for (uint32_t rbi = 0; rbi < nrb; rbi += 2u) {
+            one(std::false_type{}, rbi);
+            if (rbi + 1u < nrb) one(std::true_type{}, rbi + 1u);
+        }
     }
     // Every transfer into LDS was waited for at the barrier of the stage before the one that read
     // it, so none is in flight when the workgroup's LDS is released.
@@ -521,7 +645,8 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
 
 // How the (column group, M slice) grid is cut.  One workgroup fills a compute unit (all of its
 // registers and LDS), so the launch runs in rounds of 256 workgroups; a workgroup costs one prologue
-// (measured ~6.5 us) plus ~2.9 us per 64-row block.  The number of M slices is the one that
+// (measured ~6.5 us) plus ~2.9 us per 64-row block (the same for both K: a row block is 64 rows x
+// 32768 / K columns x K).  The number of M slices is the one that
 // minimises rounds x (prologue + row blocks per slice) in those units (9 : 4): enough slices to
 // fill the chip, no more than that (every slice repeats the transform of its columns), and no
 // nearly empty last round.
@@ -529,10 +654,10 @@ struct Plan {
     uint32_t ngroups, msplit, m_per_block;
     uint32_t mpx, cgx, nrect, grid;  // XCD rectangles
 };
-inline Plan plan(uint32_t M, uint32_t N, uint32_t mpx_max)
+inline Plan plan(uint32_t M, uint32_t N, uint32_t cols, uint32_t mpx_max)
 {
     Plan p{};
-    p.ngroups = (N + kCols - 1u) / kCols;
+    p.ngroups = (N + cols - 1u) / cols;
     const uint32_t row_blocks = (M + kRows - 1u) / kRows;
     uint64_t best = ~0ull;
     uint32_t best_s = 1;
@@ -585,8 +710,9 @@ template <class T16, int K, bool OUT_F32>
 int launch_as(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, float scale,
               uint32_t mpx, hipStream_t s)
 {
-    const OutputScale os = split_output_scale((double)scale, tile_stage_shift<2>(10, kNarrowRange<T16>));
-    const Plan p = plan(M, N, mpx);
+    const OutputScale os =
+        split_output_scale((double)scale, tile_stage_shift<2>(ilog2((uint32_t)K), kNarrowRange<T16>));
+    const Plan p = plan(M, N, Geom<K>::COLS, mpx);
     auto kern = fused_ht_gemm_xreg_kernel<T16, K, OUT_F32>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess)
@@ -608,27 +734,36 @@ int launch(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, int o
 
 }  // namespace xreg
 
-// Called by the dispatcher of mi_fused_ht_gemm for K = 1024 (arguments already validated there).
-int fused_gemm16_xreg(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, int in_dtype,
-                      int out_f32, float scale, hipStream_t s)
+// Called by the dispatcher of mi_fused_ht_gemm for K = 512 and K = 1024 (arguments already validated
+// there).
+int fused_gemm16_xreg(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
+                      int in_dtype, int out_f32, float scale, hipStream_t s)
 {
     // W and a row block of C are addressed with 32-bit byte offsets
-    if ((uint64_t)M * 2048u > 0xffffffffull || (uint64_t)N * 4u * 64u > 0xffffffffull)
+    if ((uint64_t)M * K * 2u > 0xffffffffull || (uint64_t)N * 4u * 64u > 0xffffffffull)
         return MI_ERR_SHAPE;
-    if (in_dtype == MI_BF16) return xreg::launch<BF16, 1024>(W, Xt, C, M, N, out_f32, scale, 8u, s);
-    if (in_dtype == MI_F16) return xreg::launch<F16, 1024>(W, Xt, C, M, N, out_f32, scale, 8u, s);
+    if (K == 1024u) {
+        if (in_dtype == MI_BF16) return xreg::launch<BF16, 1024>(W, Xt, C, M, N, out_f32, scale, 8u, s);
+        if (in_dtype == MI_F16) return xreg::launch<F16, 1024>(W, Xt, C, M, N, out_f32, scale, 8u, s);
+    } else if (K == 512u) {
+        if (in_dtype == MI_BF16) return xreg::launch<BF16, 512>(W, Xt, C, M, N, out_f32, scale, 8u, s);
+        if (in_dtype == MI_F16) return xreg::launch<F16, 512>(W, Xt, C, M, N, out_f32, scale, 8u, s);
+    } else {
+        return MI_ERR_SIZE;
+    }
     return MI_ERR_DTYPE;
 }
 
 }  // namespace mi
 
-extern "C" int mi_debug_fused_gemm_tiling(uint32_t M, uint32_t N, uint32_t* header, uint32_t* tiles,
-                                          uint32_t capacity)
+extern "C" int mi_debug_fused_gemm_tiling(uint32_t M, uint32_t N, uint32_t K, uint32_t* header,
+                                          uint32_t* tiles, uint32_t capacity)
 {
     using namespace mi;
     if (!header) return MI_ERR_NULL;
     if (M == 0 || N == 0) return MI_ERR_SHAPE;
-    const xreg::Plan p = xreg::plan(M, N, 8u);
+    if (K != 512u && K != 1024u) return MI_ERR_SIZE;
+    const xreg::Plan p = xreg::plan(M, N, K == 512u ? xreg::Geom<512>::COLS : xreg::Geom<1024>::COLS, 8u);
     const uint32_t h[8] = {p.ngroups, p.msplit, p.m_per_block, p.mpx, p.cgx, p.nrect, p.grid, 0u};
     for (int i = 0; i < 8; ++i) header[i] = h[i];
     if (!tiles) return MI_OK;

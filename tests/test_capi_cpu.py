@@ -100,14 +100,14 @@ def test_product_code_never_touches_the_oracle():
     assert "oracle" not in hdr
 
 
-def _tiling(lib, M, N):
+def _tiling(lib, M, N, K=1024):
     import ctypes
 
     header = (ctypes.c_uint32 * 8)()
-    assert lib.mi_debug_fused_gemm_tiling(M, N, header, None, 0) == 0
+    assert lib.mi_debug_fused_gemm_tiling(M, N, K, header, None, 0) == 0
     ngroups, msplit, m_per_block, mpx, cgx, nrect, grid, _ = list(header)
     tiles = (ctypes.c_uint32 * (2 * grid))()
-    assert lib.mi_debug_fused_gemm_tiling(M, N, header, tiles, grid) == 0
+    assert lib.mi_debug_fused_gemm_tiling(M, N, K, header, tiles, grid) == 0
     return dict(ngroups=ngroups, msplit=msplit, m_per_block=m_per_block, mpx=mpx, cgx=cgx,
                 nrect=nrect, grid=grid), [(tiles[2 * i], tiles[2 * i + 1]) for i in range(grid)]
 
@@ -118,20 +118,20 @@ def test_fused_gemm_tiling_covers_every_tile_exactly_once(libmod):
     shapes = [(4096, 4096), (1, 1), (64, 128), (65, 129), (577, 1333), (5000, 3000), (12288, 12288),
               (2048, 8192), (8192, 2048), (4096, 16384), (16384, 4096), (700, 4095), (130, 2000),
               (4096, 130), (100000, 128), (64, 100000), (9999, 7777), (8192, 8192), (3968, 31 * 128)]
-    for M, N in shapes:
-        p, tiles = _tiling(lib, M, N)
-        assert p["ngroups"] == -(-N // 128)
+    for M, N, K in [(m, n, 1024) for m, n in shapes] + [(m, n, 512) for m, n in shapes[:12]]:
+        p, tiles = _tiling(lib, M, N, K)
+        assert p["ngroups"] == -(-N // (131072 // K))
         assert p["m_per_block"] % 64 == 0 and p["msplit"] == -(-M // p["m_per_block"])
         assert (p["msplit"] - 1) * p["m_per_block"] < M          # no empty slice
         real = [t for t in tiles if t != (0xFFFFFFFF, 0xFFFFFFFF)]
         want = {(cg, ms) for cg in range(p["ngroups"]) for ms in range(p["msplit"])}
-        assert len(real) == len(want) and set(real) == want, (M, N, p)
+        assert len(real) == len(want) and set(real) == want, (M, N, K, p)
         if True:
             assert p["msplit"] % p["mpx"] == 0 and p["ngroups"] % p["cgx"] == 0
             assert 1 <= p["mpx"] * p["cgx"] <= 32
             # no XCD carries more rounds of 32 workgroups than an even spread would need
             per_xcd = [sum(1 for i, t in enumerate(tiles) if i % 8 == x and t[0] != 0xFFFFFFFF) for x in range(8)]
-            assert -(-max(per_xcd) // 32) == -(-(-(-len(real) // 8)) // 32), (M, N, p, per_xcd)
+            assert -(-max(per_xcd) // 32) == -(-(-(-len(real) // 8)) // 32), (M, N, K, p, per_xcd)
             # a rectangle lives on one XCD (workgroup id % 8) and its workgroups are dispatched
             # back to back there
             where = {}
@@ -155,3 +155,6 @@ def test_fused_gemm_tiling_avoids_a_nearly_empty_last_round(libmod):
     # 24 column groups: 11 slices would be 264 workgroups; 10 fit one round
     p, _ = _tiling(lib, 5000, 3000)
     assert p["ngroups"] * p["msplit"] <= 256
+    # other K: rejected before anything else
+    import ctypes
+    assert lib.mi_debug_fused_gemm_tiling(64, 64, 2048, (ctypes.c_uint32 * 8)(), None, 0) != 0

@@ -104,41 +104,43 @@ def test_gemm_against_oracle(pkg, oracle, M, N, K, dt, tol):
         assert _rel(oracle, C16, want) <= tol
 
 
-# K = 1024 runs the register-resident kernel: 128-column groups, 64-row blocks, results stored
-# while the next row block is multiplied.  Shapes around every tile boundary, a single row block,
-# odd N (no paired stores), a scale that is not a power of two (separate store path), both 16-bit
-# types and both output types.
-@pytest.mark.parametrize("M,N", [(1, 1), (63, 127), (64, 128), (65, 129), (128, 256), (577, 1333),
-                                 (130, 2000), (4096, 130), (700, 4095)])
-def test_gemm_k1024_tile_boundaries(pkg, oracle, M, N):
-    K = 1024
+# K = 512 and 1024 run the register-resident kernel: groups of 65536 / K columns, 64-row blocks,
+# results stored while the next row block is multiplied (K = 1024) or right after it (K = 512).
+# Shapes around every tile boundary, a single row block, N not a multiple of the columns a lane
+# stores together (no vector stores), a scale that is not a power of two (separate store path),
+# both 16-bit types and both output types.
+@pytest.mark.parametrize("K", [1024, 512])
+@pytest.mark.parametrize("M,N", [(1, 1), (63, 127), (64, 128), (65, 129), (128, 256), (129, 257),
+                                 (577, 1333), (130, 2000), (4096, 130), (700, 4095), (200, 514)])
+def test_gemm_k1024_tile_boundaries(pkg, oracle, M, N, K):
     for dt in (torch.bfloat16, torch.float16):
         W, Xt = oracle.inputs_gemm(M, N, K, dt)
         for scale, od in ((None, torch.float32), (None, dt), (0.37 / 32.0, torch.float32),
                           (1.0, torch.float32), (1.0 / 64.0, dt)):
             if dt == torch.float16 and scale == 1.0:
                 continue  # unnormalised fp16 overflows the storage range by construction
-            s = 1.0 / 32.0 if scale is None else scale
+            s = 1.0 / math.sqrt(K) if scale is None else scale
             C = pkg.fused_ht_gemm(W.cuda(), Xt.cuda(), scale, out_dtype=od)
             torch.cuda.synchronize()
             want = oracle.fused_ht_gemm_f64_blas(W.double().numpy(), Xt.double().numpy(), s)
             assert C.shape == (M, N) and C.dtype == od
-            assert _rel(oracle, C, want) <= 2e-2, (M, N, dt, scale, od)
+            assert _rel(oracle, C, want) <= 2e-2, (M, N, K, dt, scale, od)
 
 
-def test_gemm_k1024_every_output_written_once(pkg, oracle):
+@pytest.mark.parametrize("K", [1024, 512])
+def test_gemm_k1024_every_output_written_once(pkg, oracle, K):
     # size-independent check on the full benchmark shape, both output types: C against the
     # unfused product computed on the device from the library's own transform, every element
     M = N = 4096
-    K = 1024
+    s2 = 1.0 / 32.0 if K == 1024 else 1.0 / 16.0        # a power of two: the vector-store path
     W, Xt = oracle.inputs_gemm(M, N, K, torch.bfloat16)
     Wd, Xd = W.cuda(), Xt.cuda()
-    Y = pkg.hadamard_transform(Xd)                      # bf16, same rounding as the fused operand
+    Y = pkg.hadamard_transform(Xd, s2)                  # bf16, same rounding as the fused operand
     ref = Wd.float() @ Y.float().t()
     scale = ref.abs().max().item()
     for od in (torch.bfloat16, torch.float32):
         for _ in range(3):                               # back-to-back launches reuse LDS and registers
-            C = pkg.fused_ht_gemm(Wd, Xd, out_dtype=od)
+            C = pkg.fused_ht_gemm(Wd, Xd, s2, out_dtype=od)
         torch.cuda.synchronize()
         err = (C.float() - ref).abs().max().item() / scale
         assert err <= (8e-3 if od == torch.bfloat16 else 2e-3), (od, err)
@@ -148,22 +150,23 @@ def test_gemm_k1024_every_output_written_once(pkg, oracle):
 # evenly (workgroup ids without work), M slices that are not a power of two, more than one round of
 # workgroups, a ragged last slice and last column group.  Every element against the unfused
 # product computed on the device from the library's own transform.
+@pytest.mark.parametrize("K", [1024, 512])
 @pytest.mark.parametrize("M,N", [(5000, 3000), (6144, 6144), (2048, 8192), (12288, 1536), (1000, 9000)])
-def test_gemm_k1024_launch_plans(pkg, oracle, M, N):
-    K = 1024
+def test_gemm_k1024_launch_plans(pkg, oracle, M, N, K):
     g = torch.Generator(device="cuda").manual_seed(M + N)
+    s2 = 1.0 / 32.0 if K == 1024 else 1.0 / 16.0        # a power of two: the vector-store path
     Wd = torch.randn(M, K, generator=g, device="cuda").to(torch.bfloat16)
     Xd = torch.randn(N, K, generator=g, device="cuda").to(torch.bfloat16)
-    Y = pkg.hadamard_transform(Xd)
+    Y = pkg.hadamard_transform(Xd, s2)
     ref = Wd.float() @ Y.float().t()
     scale = ref.abs().max().item()
-    C = pkg.fused_ht_gemm(Wd, Xd)
+    C = pkg.fused_ht_gemm(Wd, Xd, s2)
     torch.cuda.synchronize()
     assert torch.isfinite(C.float()).all()
     assert (C.float() - ref).abs().max().item() / scale <= 8e-3
     # a few rows against the fp64 oracle as well
     idx = torch.tensor([0, 63, 64, M // 2, M - 1])
-    want = oracle.fused_ht_gemm_f64_blas(Wd[idx].cpu().double().numpy(), Xd.cpu().double().numpy(), 1.0 / 32.0)
+    want = oracle.fused_ht_gemm_f64_blas(Wd[idx].cpu().double().numpy(), Xd.cpu().double().numpy(), s2)
     assert _rel(oracle, C[idx], want) <= 2e-2
 
 
