@@ -219,6 +219,24 @@ def main() -> int:
         print(json.dumps(result))
         return 0
 
+    # ---- the same kernel at other sizes: larger N and M amortise the prologue, K = 512 halves the LDS
+    # traffic per flop (bf16, fused / vendor GEMM without transform / transform + vendor GEMM) ---------
+    if not only:
+        for (Kx, Mx, Nx) in ((1024, 8192, 8192), (512, 4096, 4096), (512, 8192, 8192)):
+            Wx = torch.randn(Mx, Kx, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(dev)
+            Xx = torch.randn(Nx, Kx, generator=torch.Generator().manual_seed(0)).to(torch.bfloat16).to(dev)
+            fx = 2 * Mx * Nx * Kx
+            f_ms, _ = steady_ms(lambda: hada.fused_ht_gemm(Wx, Xx), 30, 30.0)
+            v_ms, _ = steady_ms(lambda: torch.matmul(Wx, Xx.t()), 30, 30.0)
+            u_ms, _ = steady_ms(lambda: torch.matmul(Wx, hada.hadamard_transform(Xx).t()), 30, 30.0)
+            others[f"fused_ht_gemm_bf16_K{Kx}_M{Mx}_N{Nx}"] = {
+                "us": round(f_ms * 1e3, 2), "algorithmic_flops": fx,
+                "roofline": roofline("mfma", fx / f_ms / 1e9, PEAK_TFLOPS["bf16"], "TFLOP/s", None),
+                "library_gemm_without_transform_us": round(v_ms * 1e3, 2),
+                "unfused_transform_then_library_gemm_us": round(u_ms * 1e3, 2),
+                "fused_over_unfused_speedup": round(u_ms / f_ms, 3)}
+            del Wx, Xx
+
     # ---- fp32 fused GEMM -------------------------------------------------------------------------------
     if want("gemm_f32"):
         W = torch.randn(M, K, generator=torch.Generator().manual_seed(1)).to(dev)
