@@ -32,7 +32,7 @@
 
 namespace mi {
 
-// K = 512 and 1024 with the transformed operand in registers: fused_gemm_xreg.hip
+// K = 512, 1024 and 2048 with the transformed operand in registers: fused_gemm_xreg.hip
 int fused_gemm16_xreg(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
                       int in_dtype, int out_f32, float scale, hipStream_t s);
 
@@ -456,8 +456,8 @@ int dispatch_gemm16(const void* W, const void* Xt, void* C, uint32_t M, uint32_t
         case 128:
         case 256: return launch_gemm16<T16, 64, 0, 0>(W, Xt, C, M, N, K, out_f32, scale, s);
         case 512:
-        case 1024: return fused_gemm16_xreg(W, Xt, C, M, N, K, T16::kCode, out_f32, scale, s);
-        case 2048: return launch_gemm16<T16, 32, 2, 0>(W, Xt, C, M, N, K, out_f32, scale, s);
+        case 1024:
+        case 2048: return fused_gemm16_xreg(W, Xt, C, M, N, K, T16::kCode, out_f32, scale, s);
         case 4096: return launch_gemm16<T16, 16, 3, 0>(W, Xt, C, M, N, K, out_f32, scale, s);
         default: return MI_ERR_SIZE;
     }

@@ -1,15 +1,15 @@
 // Fused Hadamard -> GEMM with the transformed operand held in registers, gfx950, 16-bit inputs:
-//     C[M,N] = W[M,K] * (scale * H_K * X[K,N]),  X given as Xt[N,K],  K = 512 or 1024.
+//     C[M,N] = W[M,K] * (scale * H_K * X[K,N]),  X given as Xt[N,K],  K = 512, 1024 or 2048.
 //
 // One workgroup = four wavefronts, one per SIMD, each with the whole 512-register budget.
-//   prologue : wavefront w transforms 32768 / K columns of X (32 at K = 1024, 64 at K = 512) on the
+//   prologue : wavefront w transforms 32768 / K columns of X (64, 32 or 16) on the
 //              matrix cores (coalesced 16-byte loads, the two-stage tile transform of
 //              fwht_device.hpp; at K = 1024 the last butterfly is folded into the second stage),
 //              passes them once through a wavefront-private LDS area to get from "a lane owns 8
 //              consecutive k of one column" to MFMA operand order "lane (hi, lo) owns 8
 //              consecutive k of column lo", and keeps all 32768 values in the 256 accumulation
-//              registers for the rest of the kernel.  The workgroup therefore owns 128 (256)
-//              columns, twice what fits in LDS.
+//              registers for the rest of the kernel.  The workgroup therefore owns 256, 128 or
+//              64 columns, twice what fits in LDS.
 //   main loop: the workgroup walks its M range in 64-row blocks.  W is the only operand that
 //              moves: global -> LDS directly (no register hop), each wavefront fetching a quarter
 //              of a 64-row x 256-K stage as whole 512-byte row segments into a ring of four
@@ -55,7 +55,8 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 // registers (64 fragments of 16 columns x 32 k).
 template <int K>
 struct Geom {
-    static_assert(K == 512 || K == 1024, "register budget: 16 NBF columns x K = 32768 values per wavefront");
+    static_assert(K == 512 || K == 1024 || K == 2048,
+                  "register budget: 16 NBF columns x K = 32768 values per wavefront");
     static constexpr int NBF = 2048 / K;            // 16-column fragments per wavefront
     static constexpr int CPW = 16 * NBF;            // columns per wavefront
     static constexpr int COLS = 4 * CPW;            // columns per workgroup
@@ -75,8 +76,26 @@ __host__ __device__ constexpr uint32_t area_offset(uint32_t j, uint32_t q)
 {
     return j * 1024u + ((q ^ j) << 4);
 }
+// The same area at K = 2048, four columns at a time: [4 columns][256 chunks], chunk q of column c
+// stored at q ^ 2c.
+__host__ __device__ constexpr uint32_t area4_offset(uint32_t c, uint32_t q)
+{
+    return c * 4096u + ((q ^ (2u * c)) << 4);
+}
 constexpr bool lds_patterns_conflict_free()
 {
+    // K = 2048: every lane writes chunk 64 t + lane of column c; in round p only the lanes with
+    // lo / 4 == p read, chunk 4 s + hi of column lo % 4
+    for (uint32_t c = 0; c < 4; ++c)
+        for (uint32_t t = 0; t < 4; ++t)
+            if (!lds::conflict_free_b128([=](uint32_t lane) { return area4_offset(c, 64u * t + lane); }))
+                return false;
+    for (uint32_t p = 0; p < 4; ++p)
+        for (uint32_t s = 0; s < 64; ++s)
+            if (!lds::conflict_free_b128_masked(
+                    [=](uint32_t lane) { return area4_offset(lane & 3u, 4u * s + (lane >> 4)); },
+                    [=](uint32_t lane) { return ((lane & 15u) >> 2) == p; }))
+                return false;
     // fragment read of row block mb, K step ks: lane (hi, lo) takes row 16 mb + lo, chunk 4 ks + hi
     for (uint32_t mb = 0; mb < 4; ++mb)
         for (uint32_t ks = 0; ks < 8; ++ks)
@@ -136,6 +155,11 @@ __device__ __forceinline__ void mfma_delay()
 {
     asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
+}
+__device__ __forceinline__ void drain_mfma(f32x4 (&acc)[4][1])
+{
+    mfma_delay();
+    asm volatile("" : "+v"(acc[0][0]), "+v"(acc[1][0]), "+v"(acc[2][0]), "+v"(acc[3][0]));
 }
 __device__ __forceinline__ void drain_mfma(f32x4 (&acc)[4][2])
 {
@@ -208,6 +232,30 @@ __device__ __forceinline__ void column_transform(typename T16::V8 t0, typename T
     }
 }
 
+// The same without the final rounding: s[h] / d[h] hold elements 4h .. 4h+3 of the lane's eight for
+// the first / second half (K = 2048 adds one more butterfly, between two such pairs, in fp32).
+template <class T16>
+__device__ __forceinline__ void column_pair_f32(typename T16::V8 t0, typename T16::V8 t1,
+                                                const PairOperands<T16>& po, f32x4 (&s)[2],
+                                                f32x4 (&d)[2])
+{
+    using E = typename T16::E;
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const f32x4 d0 = T16::mfma32(t0, po.g1[h], zero);
+        const f32x4 d1 = T16::mfma32(t1, po.g1[h], zero);
+        typename T16::V8 a2;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            a2[r] = (E)d0[r];
+            a2[4 + r] = (E)d1[r];
+        }
+        s[h] = T16::mfma32(a2, po.g2s, zero);
+        d[h] = T16::mfma32(a2, po.g2d, zero);
+    }
+}
+
 __device__ __forceinline__ void wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 // at most N vector memory operations of this wavefront still outstanding (they complete in order)
 // (`n` folds to a constant once the loops around the call are unrolled)
@@ -230,6 +278,10 @@ __device__ __forceinline__ void global_to_lds16(uint32_t lane_off, const void* b
                  :: "v"(lane_off), "s"(base), "s"(lds_base) : "memory");
 }
 // streaming (non-temporal) stores, scalar base + 32-bit lane offset
+__device__ __forceinline__ void stream_store2(uint32_t lane_off, uint32_t v, void* base)
+{
+    asm volatile("global_store_short %0, %1, %2 nt" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
+}
 __device__ __forceinline__ void stream_store4(uint32_t lane_off, uint32_t v, void* base)
 {
     asm volatile("global_store_dword %0, %1, %2 nt" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
@@ -380,6 +432,57 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
                     yf[nb][KSTEPS / 2 + s] =
                         *reinterpret_cast<const V8*>(area + area_offset(lo, 4u * s + hi));
             }
+        } else if constexpr (K == 2048) {
+            // A column is four tiles: two pairs through the pair transform, one fp32 butterfly
+            // between them (H_2048 = [[H, H], [H, -H]] over the halves).  Sixteen columns do not
+            // fit the area at once: four rounds of four columns; in round p only the lanes whose
+            // fragment column lo belongs to the round (lo / 4 == p) read their column back.
+            PairOperands<T16> po;
+            make_pair_operands<T16>(po, exp2);
+            V8 in[4][4];
+            auto load_col = [&](int p4, int c) {
+                const uint32_t col = min(n0 + CPW * wave + (uint32_t)(4 * p4 + c), N - 1u);
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    in[c][t] = *reinterpret_cast<const V8*>(Xt + ((uint64_t)col * K + 512u * t + 8u * lane));
+            };
+#pragma unroll
+            for (int c = 0; c < 4; ++c) load_col(0, c);
+#pragma unroll
+            for (int p4 = 0; p4 < 4; ++p4) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    f32x4 sa[2], da[2], sb[2], db[2];
+                    column_pair_f32<T16>(in[c][0], in[c][1], po, sa, da);
+                    column_pair_f32<T16>(in[c][2], in[c][3], po, sb, db);
+                    if (p4 + 1 < 4) load_col(p4 + 1, c);
+                    if (p4 == 3) {  // the first AHEAD stages of W: 8 AHEAD pieces over four columns
+#pragma unroll
+                        for (int u = 0; u < 2 * AHEAD; ++u) {
+                            const int pc = 2 * AHEAD * c + u;
+                            w_issue(pc >> 3, pc >> 3, pc & 7);
+                        }
+                    }
+                    V8 o[4];  // k quarters: A_lo + B_lo, A_hi + B_hi, A_lo - B_lo, A_hi - B_hi
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            o[0][4 * h + r] = (E)(sa[h][r] + sb[h][r]);
+                            o[1][4 * h + r] = (E)(da[h][r] + db[h][r]);
+                            o[2][4 * h + r] = (E)(sa[h][r] - sb[h][r]);
+                            o[3][4 * h + r] = (E)(da[h][r] - db[h][r]);
+                        }
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        *reinterpret_cast<V8*>(area + area4_offset(c, 64u * t + lane)) = o[t];
+                }
+                if ((int)(lo >> 2) == p4) {
+#pragma unroll
+                    for (int s = 0; s < KSTEPS; ++s)
+                        yf[0][s] = *reinterpret_cast<const V8*>(area + area4_offset(lo & 3u, 4u * s + hi));
+                }
+            }
         } else {  // K = 512: a column is one tile
             TileOperands<T16> ops;
             make_tile_operands<T16, 2>(9, ops, exp2);
@@ -448,7 +551,13 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
         // streaming stores: C is not read again, and keeping it out of the L2 leaves the cache to
         // the operands
         unsigned char* row_ptr = Cb + (block_base + (uint64_t)((16u * mb + r) * N) * esize);  // scalar
-        if constexpr (NBF == 2) {
+        if constexpr (NBF == 1) {
+            const float v0 = acc[mb][0][r] * mult;
+            if (OUT_F32)
+                stream_store4(lane_off, __builtin_bit_cast(uint32_t, v0), row_ptr);
+            else
+                stream_store2(lane_off, (uint32_t)__builtin_bit_cast(uint16_t, (E)v0), row_ptr);
+        } else if constexpr (NBF == 2) {
             const float v0 = acc[mb][0][r] * mult, v1 = acc[mb][1][r] * mult;
             if (OUT_F32)
                 stream_store8(lane_off, u32x2{__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1)}, row_ptr);
@@ -524,11 +633,13 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
                         // fragments two K steps ahead; the last two steps of a stage read the
                         // first two of the next stage, behind the barrier
                         fr[(ks + 2) & 3][m] = ks < 6 ? frag(cur_slot, m, ks + 2) : frag(next_slot, m, ks - 6);
-                    } else if (m < 6) {
-                        if (ks < 6 && (fill_own_block || !last)) {
-                            const int i = kPieceAt[ks] + (m - 4);
-                            if (i < kPieceAt[ks + 1]) w_issue(fill_kq, fill_slot, i);
-                        }
+                    }
+                    // up to two transfer pieces: behind MFMAs 4 and 5 where a K step has that
+                    // many, else next to the fragment reads of MFMAs 1 and 3
+                    const int piece = NM >= 6 ? m - 4 : (m == 1 ? 0 : (m == 3 ? 1 : -1));
+                    if (piece >= 0 && piece < 2 && ks < 6 && (fill_own_block || !last)) {
+                        const int i = kPieceAt[ks] + piece;
+                        if (i < kPieceAt[ks + 1]) w_issue(fill_kq, fill_slot, i);
                     }
                     // the previous block's sixteen stores, one behind each MFMA of the K steps
                     // that follow the first stage's barrier: they then have most of a stage to
@@ -734,8 +845,8 @@ int launch(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, int o
 
 }  // namespace xreg
 
-// Called by the dispatcher of mi_fused_ht_gemm for K = 512 and K = 1024 (arguments already validated
-// there).
+// Called by the dispatcher of mi_fused_ht_gemm for K = 512, 1024 and 2048 (arguments already
+// validated there).
 int fused_gemm16_xreg(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
                       int in_dtype, int out_f32, float scale, hipStream_t s)
 {
@@ -748,6 +859,9 @@ int fused_gemm16_xreg(const void* W, const void* Xt, void* C, uint32_t M, uint32
     } else if (K == 512u) {
         if (in_dtype == MI_BF16) return xreg::launch<BF16, 512>(W, Xt, C, M, N, out_f32, scale, 8u, s);
         if (in_dtype == MI_F16) return xreg::launch<F16, 512>(W, Xt, C, M, N, out_f32, scale, 8u, s);
+    } else if (K == 2048u) {
+        if (in_dtype == MI_BF16) return xreg::launch<BF16, 2048>(W, Xt, C, M, N, out_f32, scale, 8u, s);
+        if (in_dtype == MI_F16) return xreg::launch<F16, 2048>(W, Xt, C, M, N, out_f32, scale, 8u, s);
     } else {
         return MI_ERR_SIZE;
     }
@@ -762,8 +876,8 @@ extern "C" int mi_debug_fused_gemm_tiling(uint32_t M, uint32_t N, uint32_t K, ui
     using namespace mi;
     if (!header) return MI_ERR_NULL;
     if (M == 0 || N == 0) return MI_ERR_SHAPE;
-    if (K != 512u && K != 1024u) return MI_ERR_SIZE;
-    const xreg::Plan p = xreg::plan(M, N, K == 512u ? xreg::Geom<512>::COLS : xreg::Geom<1024>::COLS, 8u);
+    if (K != 512u && K != 1024u && K != 2048u) return MI_ERR_SIZE;
+    const xreg::Plan p = xreg::plan(M, N, 131072u / K, 8u);
     const uint32_t h[8] = {p.ngroups, p.msplit, p.m_per_block, p.mpx, p.cgx, p.nrect, p.grid, 0u};
     for (int i = 0; i < 8; ++i) header[i] = h[i];
     if (!tiles) return MI_OK;

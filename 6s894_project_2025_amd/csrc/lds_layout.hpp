@@ -31,5 +31,24 @@ constexpr bool conflict_free_b128(AddrOfLane addr)
     return true;
 }
 
+// The same when only some lanes take part (`active(lane)`): the others are masked off and touch
+// nothing.
+template <class AddrOfLane, class Active>
+constexpr bool conflict_free_b128_masked(AddrOfLane addr, Active active)
+{
+    for (uint32_t pass = 0; pass < 8; ++pass) {
+        uint32_t seen = 0;
+        for (uint32_t l = 0; l < 8; ++l) {
+            if (!active(8u * pass + l)) continue;
+            const uint32_t a = addr(8u * pass + l);
+            if (a % 16u != 0) return false;
+            const uint32_t column = (a / 16u) % 8u;
+            if (seen & (1u << column)) return false;
+            seen |= 1u << column;
+        }
+    }
+    return true;
+}
+
 }  // namespace lds
 }  // namespace mi

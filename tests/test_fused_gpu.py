@@ -104,12 +104,12 @@ def test_gemm_against_oracle(pkg, oracle, M, N, K, dt, tol):
         assert _rel(oracle, C16, want) <= tol
 
 
-# K = 512 and 1024 run the register-resident kernel: groups of 65536 / K columns, 64-row blocks,
-# results stored while the next row block is multiplied (K = 1024) or right after it (K = 512).
+# K = 512, 1024 and 2048 run the register-resident kernel: groups of 131072 / K columns, 64-row
+# blocks, results stored while the next row block is multiplied or (K = 512) right after it.
 # Shapes around every tile boundary, a single row block, N not a multiple of the columns a lane
 # stores together (no vector stores), a scale that is not a power of two (separate store path),
 # both 16-bit types and both output types.
-@pytest.mark.parametrize("K", [1024, 512])
+@pytest.mark.parametrize("K", [1024, 512, 2048])
 @pytest.mark.parametrize("M,N", [(1, 1), (63, 127), (64, 128), (65, 129), (128, 256), (129, 257),
                                  (577, 1333), (130, 2000), (4096, 130), (700, 4095), (200, 514)])
 def test_gemm_k1024_tile_boundaries(pkg, oracle, M, N, K):
@@ -124,15 +124,18 @@ def test_gemm_k1024_tile_boundaries(pkg, oracle, M, N, K):
             torch.cuda.synchronize()
             want = oracle.fused_ht_gemm_f64_blas(W.double().numpy(), Xt.double().numpy(), s)
             assert C.shape == (M, N) and C.dtype == od
-            assert _rel(oracle, C, want) <= 2e-2, (M, N, K, dt, scale, od)
+            # error against the larger of max|C| and the typical magnitude of an output (s K for
+            # unit-variance inputs): a 1 x 1 result can be small by chance
+            err = np.abs(C.cpu().double().numpy() - want).max() / max(np.abs(want).max(), s * K)
+            assert err <= 2e-2, (M, N, K, dt, scale, od)
 
 
-@pytest.mark.parametrize("K", [1024, 512])
+@pytest.mark.parametrize("K", [1024, 512, 2048])
 def test_gemm_k1024_every_output_written_once(pkg, oracle, K):
     # size-independent check on the full benchmark shape, both output types: C against the
     # unfused product computed on the device from the library's own transform, every element
     M = N = 4096
-    s2 = 1.0 / 32.0 if K == 1024 else 1.0 / 16.0        # a power of two: the vector-store path
+    s2 = {512: 1.0 / 16.0, 1024: 1.0 / 32.0, 2048: 1.0 / 32.0}[K]   # a power of two
     W, Xt = oracle.inputs_gemm(M, N, K, torch.bfloat16)
     Wd, Xd = W.cuda(), Xt.cuda()
     Y = pkg.hadamard_transform(Xd, s2)                  # bf16, same rounding as the fused operand
@@ -150,11 +153,11 @@ def test_gemm_k1024_every_output_written_once(pkg, oracle, K):
 # evenly (workgroup ids without work), M slices that are not a power of two, more than one round of
 # workgroups, a ragged last slice and last column group.  Every element against the unfused
 # product computed on the device from the library's own transform.
-@pytest.mark.parametrize("K", [1024, 512])
+@pytest.mark.parametrize("K", [1024, 512, 2048])
 @pytest.mark.parametrize("M,N", [(5000, 3000), (6144, 6144), (2048, 8192), (12288, 1536), (1000, 9000)])
 def test_gemm_k1024_launch_plans(pkg, oracle, M, N, K):
     g = torch.Generator(device="cuda").manual_seed(M + N)
-    s2 = 1.0 / 32.0 if K == 1024 else 1.0 / 16.0        # a power of two: the vector-store path
+    s2 = {512: 1.0 / 16.0, 1024: 1.0 / 32.0, 2048: 1.0 / 32.0}[K]   # a power of two
     Wd = torch.randn(M, K, generator=g, device="cuda").to(torch.bfloat16)
     Xd = torch.randn(N, K, generator=g, device="cuda").to(torch.bfloat16)
     Y = pkg.hadamard_transform(Xd, s2)
