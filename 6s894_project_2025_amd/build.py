@@ -35,6 +35,7 @@ PER_FILE_FLAGS = {
     "rht_fp8.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     # the prologue's MFMA results feed VALU conversions; the main loop's MFMAs are inline assembly
     "fused_gemm_xreg.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "fused_gemm_xreg_f32.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
 }
 
 

@@ -10,6 +10,11 @@
 #include "fwht_device.hpp"
 
 namespace mi {
+
+// K = 1024 with the transformed operand in registers: fused_gemm_xreg_f32.hip
+int fused_gemm_f32_xreg(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, uint32_t K,
+                        float scale, hipStream_t s);
+
 namespace {
 
 constexpr int kThreads = 512;
@@ -222,7 +227,7 @@ int fused_gemm_f32(const float* W, const float* Xt, float* C, uint32_t M, uint32
         case 128:
         case 256:
         case 512: return launch<32, 0>(W, Xt, C, M, N, K, scale, s);
-        case 1024: return launch<32, 1>(W, Xt, C, M, N, K, scale, s);
+        case 1024: return fused_gemm_f32_xreg(W, Xt, C, M, N, K, scale, s);
         case 2048: return launch<16, 2>(W, Xt, C, M, N, K, scale, s);
         case 4096: return launch<16, 2, 2>(W, Xt, C, M, N, K, scale, s);  // two passes of K = 2048
         default: return MI_ERR_SIZE;

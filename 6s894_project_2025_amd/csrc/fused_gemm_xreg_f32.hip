@@ -1,0 +1,302 @@
+// Fused Hadamard -> GEMM in fp32 (the reference's precision) with the transformed operand held in
+// registers, gfx950:
+//     C[M,N] = W[M,K] * (scale * H_K * X[K,N]),  X given as Xt[N,K],  K = 1024, fp32 in and out.
+//
+// Same structure as the 16-bit kernel of fused_gemm_xreg.hip (one wavefront per SIMD, W streamed
+// global -> LDS directly through a ring of four 32 KB stages, fragments broadcast to the four
+// wavefronts through LDS, results stored behind the next block's MFMAs); what differs:
+//   * a wavefront's 256 accumulation registers hold 16 columns x 1024 k as fp32 (64 columns per
+//     workgroup, where the transformed tile in LDS allowed 32);
+//   * the prologue is the exact fp32 transform on the bf16 matrix cores (tile_transform_f32:
+//     three-piece operands), two tiles per column and one fp32 butterfly between them, passed
+//     through the LDS area four columns at a time;
+//   * the contraction is v_mfma_f32_16x16x4_f32: a 16-byte fragment per lane carries four
+//     consecutive k for four MFMAs (lane (hi, lo) of fragment kk holds k = 16 kk + 4 hi + s), a
+//     stage of 64 rows x 512 bytes is 128 k, and sixteen MFMAs of 32 cycles stand behind every four
+//     fragment reads: the loop is bound by the fp32 matrix-core rate and by nothing else.
+//
+// Behaviour replaced: fused_ht_gemm_pipelined (fp32), fused_ht/fusion_pipelined.cu:306-563.
+#include <type_traits>
+
+#include "xreg_common.hpp"
+
+namespace mi {
+namespace xreg {
+
+// acc (+)= A(16 x 4) * B(4 x 16), B straight from the accumulation-register file (see XMfma in
+// fused_gemm_xreg.hip for why this is an opaque statement and what that implies for readers of c)
+__device__ __forceinline__ void xmfma_f32_first(f32x4& c, float a, float b)
+{
+    asm volatile("v_mfma_f32_16x16x4_f32 %0, %1, %2, 0" : "=v"(c) : "v"(a), "a"(b));
+}
+__device__ __forceinline__ void xmfma_f32_next(f32x4& c, float a, float b)
+{
+    asm volatile("v_mfma_f32_16x16x4_f32 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+}
+
+template <int K>
+__global__ void __launch_bounds__(kThreads)
+fused_ht_gemm_xreg_f32_kernel(const float* __restrict__ W, const float* __restrict__ Xt,
+                              float* __restrict__ C, uint32_t M, uint32_t N, uint32_t m_per_block,
+                              uint32_t msplit, uint32_t mpx, uint32_t cgx, uint32_t nrect, float fscale)
+{
+    static_assert(K == 1024, "16 columns x K fp32 values = 256 registers per lane");
+    constexpr int KSTEPS = K / 16;        // 16-byte fragments (4 k per lane, 16 k per step) per column
+    constexpr int SPB = K / 128;          // W stages (64 rows x 128 k) per row block
+    constexpr int AHEAD = 3;              // stages the W stream runs ahead of the MFMAs
+    constexpr int NM = 16;                // MFMAs per K step: 4 row fragments x 4 k
+    constexpr uint32_t kCols = 64, CPW = 16;
+    static_assert(kSlots == 4 && AHEAD <= SPB && (SPB & 3) == 0, "stage g lives in buffer g % 4");
+    constexpr uint32_t ROW_BYTES = K * 4u;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t lo = lane & 15u, hi = lane >> 4;
+
+    uint32_t cg, ms;
+    if (!tile_of_workgroup(blockIdx.x, msplit, mpx, cgx, nrect, cg, ms)) return;  // uniform, before any barrier
+    const uint32_t n0 = cg * kCols;
+    const uint32_t m_begin = ms * m_per_block;
+    if (m_begin >= M || n0 >= N) return;  // workgroup-uniform, before any barrier
+    const uint32_t m_end = min(M, m_begin + m_per_block);
+    const uint32_t nrb = (m_end - m_begin + kRows - 1u) / kRows;
+    auto row_block = [&](uint32_t rbi) __attribute__((always_inline)) {  // clamped: rbi <= nrb
+        return rbi < nrb ? rbi : 0u;
+    };
+
+    // ---- W stream: as in the 16-bit kernel, with 4-byte elements (a stage row is 128 k) ------------
+    const unsigned char* Wb = reinterpret_cast<const unsigned char*>(W);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;
+    const uint32_t lrow = lane >> 5, lq = lane & 31u;
+    uint32_t voff[8];
+    auto set_voff = [&](uint32_t rbi) __attribute__((always_inline)) {
+        const uint32_t r0 = m_begin + row_block(rbi) * kRows + 16u * wave + lrow;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            voff[i] = min(r0 + 2u * i, M - 1u) * ROW_BYTES + ((lq ^ (2u * i + lrow)) << 4);
+    };
+    auto w_issue = [&](uint32_t kq, uint32_t slot, int i) __attribute__((always_inline)) {
+        global_to_lds16(voff[i], Wb + kq * 512u, lds_base + slot * kStageBytes + (16u * wave + 2u * i) * 512u);
+    };
+    set_voff(0);
+
+    // ---- prologue: fragment column lo of this wavefront = column n0 + 16 w + lo -------------------
+    // (scalars, not 4-vectors: an MFMA names one register, and the compiler keeps a vector's
+    // elements in the accumulation-register file only as a whole; with vectors it copied every
+    // element into one scratch register right before use, while the previous MFMA was still
+    // reading that register)
+    float yf[KSTEPS][4];
+    {
+        unsigned char* area = lds + kAreaBase + wave * kAreaBytes;
+        TileOperands<BF16> ops;
+        make_tile_operands<BF16, 4>(10, ops);
+        float in[4][2][8];
+        auto load_col = [&](int p4, int c) {
+            const uint32_t col = min(n0 + CPW * wave + (uint32_t)(4 * p4 + c), N - 1u);
+#pragma unroll
+            for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const f32x4 q = *reinterpret_cast<const f32x4*>(
+                        Xt + ((uint64_t)col * K + 512u * tile + 256u * t + 4u * lane));
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) in[c][tile][4 * t + r] = q[r];
+                }
+        };
+#pragma unroll
+        for (int c = 0; c < 4; ++c) load_col(0, c);
+#pragma unroll
+        for (int p4 = 0; p4 < 4; ++p4) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                f32x4 a0[2], a1[2];
+                tile_transform_f32(in[c][0], ops, a0);
+                tile_transform_f32(in[c][1], ops, a1);
+                if (p4 + 1 < 4) load_col(p4 + 1, c);
+                if (p4 == 3) {  // the first AHEAD stages of W, behind the last X tile
+#pragma unroll
+                    for (int u = 0; u < 2 * AHEAD; ++u) {
+                        const int pc = 2 * AHEAD * c + u;
+                        w_issue(pc >> 3, pc >> 3, pc & 7);
+                    }
+                }
+                // element 512 half + 256 t + 4 lane + r of the column = chunk 128 half + 64 t + lane
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    *reinterpret_cast<f32x4*>(area + area4_offset(c, 64u * t + lane)) = (a0[t] + a1[t]) * fscale;
+                    *reinterpret_cast<f32x4*>(area + area4_offset(c, 128u + 64u * t + lane)) =
+                        (a0[t] - a1[t]) * fscale;
+                }
+            }
+            if ((int)(lo >> 2) == p4) {
+#pragma unroll
+                for (int s = 0; s < KSTEPS; ++s) {
+                    const f32x4 q = *reinterpret_cast<const f32x4*>(area + area4_offset(lo & 3u, 4u * s + hi));
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) yf[s][e] = q[e];
+                }
+            }
+        }
+    }
+
+    wait_vm(8 * (AHEAD - 1));
+    wait_lds();
+    __builtin_amdgcn_s_barrier();
+
+    auto frag = [&](uint32_t slot, int mb, int ks) __attribute__((always_inline)) -> f32x4 {
+        return *reinterpret_cast<const f32x4*>(lds + slot * kStageBytes +
+                                               stage_offset(16u * mb + lo, 4u * ks + hi));
+    };
+    f32x4 fr[4][4];  // [K step % 4][mb]
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) {
+        fr[0][mb] = frag(0, mb, 0);
+        fr[1][mb] = frag(0, mb, 1);
+    }
+
+    // lane (hi, lo) of a row block owns rows 16 mb + 4 hi + r of column n0 + 16 w + lo
+    const uint32_t col = n0 + CPW * wave + lo;
+    const uint32_t lane_off = (4u * hi * N + col) * 4u;  // inside the row block, < 2^32
+    unsigned char* const Cb = reinterpret_cast<unsigned char*>(C);
+    const bool cols_full = n0 + kCols <= N;
+    auto store_one = [&](const f32x4 (&acc)[4][1], uint64_t block_base, int mb, int r)
+        __attribute__((always_inline)) {
+        unsigned char* row_ptr = Cb + (block_base + (uint64_t)((16u * mb + r) * N) * 4u);  // scalar
+        const float v = acc[mb][0][r];  // (a bit cast applied to the element expression itself reads element 0)
+        stream_store4(lane_off, __float_as_uint(v), row_ptr);
+    };
+    auto store_edge = [&](const f32x4 (&acc)[4][1], uint32_t row_base) __attribute__((always_inline)) {
+        if (col >= N) return;
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t row = row_base + 16u * mb + 4u * hi + r;
+                if (row < m_end) C[(uint64_t)row * N + col] = acc[mb][0][r];
+            }
+    };
+
+    auto row_block_body = [&](auto prev_tag, f32x4 (&acc)[4][1], const f32x4 (&prev)[4][1],
+                              uint64_t prev_base, uint32_t rbi) __attribute__((always_inline)) {
+        constexpr bool prev_full = decltype(prev_tag)::value;
+        const bool last = rbi + 1u == nrb;
+#pragma unroll
+        for (int kq = 0; kq < SPB; ++kq) {
+            constexpr int kPieceAt[7] = {0, 2, 4, 5, 6, 7, 8};
+            // (everything below folds to constants once the loops are unrolled; SPB is a multiple
+            // of 4, so stage kq of every row block lives in buffer kq % 4)
+            const int cur_slot = kq & 3, next_slot = (kq + 1) & 3, fill_slot = (kq + AHEAD) & 3;
+            const int fill_kq = (kq + AHEAD) % SPB;
+            const bool fill_own_block = kq + AHEAD < SPB;
+#pragma unroll
+            for (int ks = 0; ks < kStepsPerStage; ++ks) {
+                if (kq == SPB - AHEAD && ks == 0 && !last) set_voff(rbi + 1u);
+                const int kk = kq * kStepsPerStage + ks;
+#pragma unroll
+                for (int m = 0; m < NM; ++m) {
+                    const int s = m >> 2, mb = m & 3;  // consecutive MFMAs go to different accumulators
+                    if (kk == 0 && s == 0)
+                        xmfma_f32_first(acc[mb][0], fr[ks & 3][mb][s], yf[0][s]);
+                    else
+                        xmfma_f32_next(acc[mb][0], fr[ks & 3][mb][s], yf[kk][s]);
+                    // one memory instruction in the shadow of an MFMA: fragments two K steps ahead
+                    // (m = 12 .. 15: their registers were last read by the MFMAs of two steps ago),
+                    // up to two transfer pieces, the previous block's sixteen stores
+                    if (m >= 12)
+                        fr[(ks + 2) & 3][m - 12] =
+                            ks < 6 ? frag(cur_slot, m - 12, ks + 2) : frag(next_slot, m - 12, ks - 6);
+                    else if (m >= 4 && m < 6) {
+                        if (ks < 6 && (fill_own_block || !last)) {
+                            const int i = kPieceAt[ks] + (m - 4);
+                            if (i < kPieceAt[ks + 1]) w_issue(fill_kq, fill_slot, i);
+                        }
+                    }
+                    if (prev_full && kk == 6) store_one(prev, prev_base, m >> 2, m & 3);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                // keep the previous step's fragment registers allocated while the matrix core may
+                // still be reading them (see the 16-bit kernel)
+                asm volatile("" ::"v"(fr[(ks + 3) & 3][0]), "v"(fr[(ks + 3) & 3][1]),
+                             "v"(fr[(ks + 3) & 3][2]), "v"(fr[(ks + 3) & 3][3]));
+                if (ks == 5) {
+                    const int later = SPB - kq - 2 < AHEAD - 1 ? SPB - kq - 2 : AHEAD - 1;
+                    const int after_last = kq == SPB - 1 ? -1 : 8 * (later > 0 ? later : 0);
+                    if (last)
+                        wait_vm(after_last);
+                    else
+                        wait_vm(8 * (AHEAD - 1));
+                    wait_lds();
+                    __builtin_amdgcn_s_barrier();
+                }
+            }
+        }
+    };
+
+    auto store_block = [&](f32x4 (&acc)[4][1], uint64_t base) __attribute__((always_inline)) {
+        drain_mfma(acc);
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) store_one(acc, base, mb, r);
+    };
+    f32x4 accA[4][1], accB[4][1];
+    bool pend = false;        // accB holds a finished full row block that is not stored yet
+    uint64_t pend_base = 0;
+    auto run = [&](bool prev_full, f32x4 (&acc)[4][1], const f32x4 (&prev)[4][1], uint64_t prev_base,
+                   uint32_t rbi) __attribute__((always_inline)) {
+        if (prev_full)
+            row_block_body(std::true_type{}, acc, prev, prev_base, rbi);
+        else
+            row_block_body(std::false_type{}, acc, prev, prev_base, rbi);
+    };
+    auto finish = [&](f32x4 (&acc)[4][1], uint32_t rbi, bool& full, uint64_t& base)
+        __attribute__((always_inline)) {
+        const uint32_t row_base = m_begin + row_block(rbi) * kRows;
+        full = cols_full && row_base + kRows <= m_end;
+        base = (uint64_t)row_base * N * 4u;
+        if (!full) {
+            drain_mfma(acc);
+            store_edge(acc, row_base);
+        }
+    };
+#pragma unroll 1
+    for (uint32_t rbi = 0; rbi < nrb; rbi += 2u) {
+        run(pend, accA, accB, pend_base, rbi);
+        bool fullA;
+        uint64_t baseA;
+        finish(accA, rbi, fullA, baseA);
+        if (rbi + 1u < nrb) {
+            run(fullA, accB, accA, baseA, rbi + 1u);
+            finish(accB, rbi + 1u, pend, pend_base);
+        } else {
+            pend = false;
+            if (fullA) store_block(accA, baseA);
+        }
+    }
+    if (pend) store_block(accB, pend_base);
+}
+
+}  // namespace xreg
+
+// Called by the fp32 dispatcher of mi_fused_ht_gemm for K = 1024 (arguments already validated).
+int fused_gemm_f32_xreg(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, uint32_t K,
+                        float scale, hipStream_t s)
+{
+    using namespace xreg;
+    if (K != 1024u) return MI_ERR_SIZE;
+    // W and a row block of C are addressed with 32-bit byte offsets
+    if ((uint64_t)M * K * 4u > 0xffffffffull || (uint64_t)N * 4u * 64u > 0xffffffffull) return MI_ERR_SHAPE;
+    const int shift = tile_stage_shift<4>(10, false);
+    const float fscale = (float)((double)scale * (double)(1u << shift));
+    const Plan p = plan(M, N, 64u, 8u);
+    auto kern = fused_ht_gemm_xreg_f32_kernel<1024>;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kLdsBytes) != hipSuccess)
+        return MI_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(p.grid), dim3(kThreads), kLdsBytes, s, W, Xt, C, M, N, p.m_per_block,
+                       p.msplit, p.mpx, p.cgx, p.nrect, fscale);
+    return launch_status();
+}
+
+}  // namespace mi

@@ -1,0 +1,224 @@
+// Pieces shared by the register-resident fused GEMM kernels (fused_gemm_xreg.hip for 16-bit inputs,
+// fused_gemm_xreg_f32.hip for fp32): the LDS geometry of the W stream and of the prologue's layout
+// change, the opaque memory statements, the workgroup tiling and its launch plan.
+#pragma once
+#include "fwht_device.hpp"
+#include "lds_layout.hpp"
+
+namespace mi {
+namespace xreg {
+
+constexpr int kThreads = 256;
+constexpr int kRows = 64;                         // rows of W per row block
+constexpr int kStageK = 256;                      // K extent of one W stage
+constexpr int kStageBytes = kRows * kStageK * 2;  // 32 KB
+constexpr int kSlots = 4;                         // ring of stage buffers
+constexpr int kStepsPerStage = kStageK / 32;      // 8 MFMA K steps
+constexpr int kAreaBytes = 16 * 512 * 2;          // per wavefront: 16 columns x 512 k
+// stage buffers 0..3 at [0, 128K); the wavefront areas of the prologue at [96K, 160K), i.e.
+// on top of stage buffer 3, which is first filled after the prologue
+constexpr int kAreaBase = 3 * kStageBytes;
+constexpr int kLdsBytes = kAreaBase + 4 * kAreaBytes;
+
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+// LDS image of a W stage: [64 rows][512 B], the 16-byte chunk q of row r stored at q ^ (r & 15).
+__host__ __device__ constexpr uint32_t stage_offset(uint32_t row, uint32_t q)
+{
+    return row * 512u + ((q ^ (row & 15u)) << 4);
+}
+// A wavefront's area of the prologue: [16 columns][1 KB], chunk q of column j stored at q ^ j.
+__host__ __device__ constexpr uint32_t area_offset(uint32_t j, uint32_t q)
+{
+    return j * 1024u + ((q ^ j) << 4);
+}
+// The same area at K = 2048, four columns at a time: [4 columns][256 chunks], chunk q of column c
+// stored at q ^ 2c.
+__host__ __device__ constexpr uint32_t area4_offset(uint32_t c, uint32_t q)
+{
+    return c * 4096u + ((q ^ (2u * c)) << 4);
+}
+constexpr bool lds_patterns_conflict_free()
+{
+    // K = 2048: every lane writes chunk 64 t + lane of column c; in round p only the lanes with
+    // lo / 4 == p read, chunk 4 s + hi of column lo % 4
+    for (uint32_t c = 0; c < 4; ++c)
+        for (uint32_t t = 0; t < 4; ++t)
+            if (!lds::conflict_free_b128([=](uint32_t lane) { return area4_offset(c, 64u * t + lane); }))
+                return false;
+    for (uint32_t p = 0; p < 4; ++p)
+        for (uint32_t s = 0; s < 64; ++s)
+            if (!lds::conflict_free_b128_masked(
+                    [=](uint32_t lane) { return area4_offset(lane & 3u, 4u * s + (lane >> 4)); },
+                    [=](uint32_t lane) { return ((lane & 15u) >> 2) == p; }))
+                return false;
+    // fragment read of row block mb, K step ks: lane (hi, lo) takes row 16 mb + lo, chunk 4 ks + hi
+    for (uint32_t mb = 0; mb < 4; ++mb)
+        for (uint32_t ks = 0; ks < 8; ++ks)
+            if (!lds::conflict_free_b128(
+                    [=](uint32_t lane) { return stage_offset(16u * mb + (lane & 15u), 4u * ks + (lane >> 4)); }))
+                return false;
+    // prologue: every lane writes chunk `lane` of column j; lane (hi, lo) reads chunk 4 s + hi of
+    // column lo
+    for (uint32_t j = 0; j < 16; ++j)
+        if (!lds::conflict_free_b128([=](uint32_t lane) { return area_offset(j, lane); })) return false;
+    for (uint32_t s = 0; s < 16; ++s)
+        if (!lds::conflict_free_b128([=](uint32_t lane) { return area_offset(lane & 15u, 4u * s + (lane >> 4)); }))
+            return false;
+    return true;
+}
+static_assert(lds_patterns_conflict_free(), "an LDS access pattern of the fused GEMM would serialise");
+
+// Waits out the matrix-core pipeline before `acc` is read by anything but an MFMA.  Two statements:
+// the delay itself, which names no register (naming them lets the compiler set the operands up
+// with register copies *in front of* the statement, i.e. reads of the accumulators right behind
+// the last MFMA: observed with sixteen accumulators), and an empty statement that the
+// accumulators pass through, so that no read of them (a register copy, say) can move above the
+// delay.
+__device__ __forceinline__ void mfma_delay()
+{
+    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+__device__ __forceinline__ void drain_mfma(f32x4 (&acc)[4][1])
+{
+    mfma_delay();
+    asm volatile("" : "+v"(acc[0][0]), "+v"(acc[1][0]), "+v"(acc[2][0]), "+v"(acc[3][0]));
+}
+__device__ __forceinline__ void drain_mfma(f32x4 (&acc)[4][2])
+{
+    mfma_delay();
+    asm volatile(""
+                 : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[1][0]), "+v"(acc[1][1]),
+                   "+v"(acc[2][0]), "+v"(acc[2][1]), "+v"(acc[3][0]), "+v"(acc[3][1]));
+}
+__device__ __forceinline__ void drain_mfma(f32x4 (&acc)[4][4])
+{
+    mfma_delay();
+    asm volatile(""
+                 : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]), "+v"(acc[0][3]),
+                   "+v"(acc[1][0]), "+v"(acc[1][1]), "+v"(acc[1][2]), "+v"(acc[1][3]),
+                   "+v"(acc[2][0]), "+v"(acc[2][1]), "+v"(acc[2][2]), "+v"(acc[2][3]),
+                   "+v"(acc[3][0]), "+v"(acc[3][1]), "+v"(acc[3][2]), "+v"(acc[3][3]));
+}
+
+__device__ __forceinline__ void wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+// at most N vector memory operations of this wavefront still outstanding (they complete in order)
+// (`n` folds to a constant once the loops around the call are unrolled)
+__device__ __forceinline__ void wait_vm(int n)
+{
+    switch (n) {
+        case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+        case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+        case 16: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
+        default: break;  // nothing to wait for
+    }
+}
+
+// 16 bytes per lane from global memory straight into LDS: lane l's bytes land at lds_base + 16 l.
+// Scalar base + 32-bit lane offset form, so that no vector arithmetic is spent on addresses.
+// (M0 carries the LDS base of the transfer; nothing else in this kernel uses it.)
+__device__ __forceinline__ void global_to_lds16(uint32_t lane_off, const void* base, uint32_t lds_base)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(lane_off), "s"(base), "s"(lds_base) : "memory");
+}
+// streaming (non-temporal) stores, scalar base + 32-bit lane offset
+__device__ __forceinline__ void stream_store2(uint32_t lane_off, uint32_t v, void* base)
+{
+    asm volatile("global_store_short %0, %1, %2 nt" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
+}
+__device__ __forceinline__ void stream_store4(uint32_t lane_off, uint32_t v, void* base)
+{
+    asm volatile("global_store_dword %0, %1, %2 nt" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
+}
+__device__ __forceinline__ void stream_store8(uint32_t lane_off, u32x2 v, void* base)
+{
+    asm volatile("global_store_dwordx2 %0, %1, %2 nt" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
+}
+// (A store of more than 8 bytes still reads its data registers during the next cycles; the compiler
+// keeps ordinary code away from them for that long, but does not know what this statement is.)
+__device__ __forceinline__ void stream_store16(uint32_t lane_off, u32x4 v, void* base)
+{
+    asm volatile("global_store_dwordx4 %0, %1, %2 nt\n\ts_nop 1" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
+}
+
+// Workgroup id -> (column group, M slice); false for an id past the last rectangle.
+__host__ __device__ inline bool tile_of_workgroup(uint32_t id, uint32_t msplit, uint32_t mpx, uint32_t cgx,
+                                                  uint32_t nrect, uint32_t& cg, uint32_t& ms)
+{
+    const uint32_t x = id & 7u, j = id >> 3;  // XCD, index inside the XCD
+    const uint32_t rsz = mpx * cgx;
+    const uint32_t rect = (j / rsz) * 8u + x, in = j % rsz;
+    if (rect >= nrect) return false;
+    const uint32_t rects_m = msplit / mpx;
+    ms = (rect % rects_m) * mpx + in % mpx;
+    cg = (rect / rects_m) * cgx + in / mpx;
+    return true;
+}
+
+// How the (column group, M slice) grid is cut.  One workgroup fills a compute unit (all of its
+// registers and LDS), so the launch runs in rounds of 256 workgroups; a workgroup costs one prologue
+// (measured ~6.5 us) plus ~2.9 us per 64-row block (the same for both K: a row block is 64 rows x
+// 32768 / K columns x K).  The number of M slices is the one that
+// minimises rounds x (prologue + row blocks per slice) in those units (9 : 4): enough slices to
+// fill the chip, no more than that (every slice repeats the transform of its columns), and no
+// nearly empty last round.
+struct Plan {
+    uint32_t ngroups, msplit, m_per_block;
+    uint32_t mpx, cgx, nrect, grid;  // XCD rectangles
+};
+inline Plan plan(uint32_t M, uint32_t N, uint32_t cols, uint32_t mpx_max)
+{
+    Plan p{};
+    p.ngroups = (N + cols - 1u) / cols;
+    const uint32_t row_blocks = (M + kRows - 1u) / kRows;
+    uint64_t best = ~0ull;
+    uint32_t best_s = 1;
+    for (uint32_t sp = 1; sp <= row_blocks && sp <= 256u; ++sp) {
+        const uint32_t rb = (row_blocks + sp - 1u) / sp;
+        const uint32_t slices = (row_blocks + rb - 1u) / rb;  // what sp really yields
+        const uint64_t rounds = ((uint64_t)p.ngroups * slices + 255u) / 256u;
+        const uint64_t cost = rounds * (9u + 4u * (uint64_t)rb);
+        if (cost < best) {
+            best = cost;
+            best_s = slices;
+        }
+    }
+    const uint32_t rb = (row_blocks + best_s - 1u) / best_s;
+    p.m_per_block = rb * kRows;
+    p.msplit = (M + p.m_per_block - 1u) / p.m_per_block;
+    // Rectangles: mpx | msplit, cgx | ngroups, at most 32 workgroups (one round of an XCD).
+    // Rectangle r runs on XCD r % 8, so the busiest XCD gets ceil(nrect / 8) rectangles.  Wanted,
+    // in this order: as few rounds on the busiest XCD as possible, a load within 15 % of an even
+    // spread over the eight XCDs, the largest rectangle, M extent 4 before 2, 8, 1.  (1 x 1 is
+    // the plain order, so there is always a candidate.)
+    const uint32_t total = p.ngroups * p.msplit;
+    const uint32_t even = (total + 7u) / 8u;
+    const uint32_t pref[4] = {4u, 2u, 8u, 1u};
+    uint64_t best_key = ~0ull;
+    for (uint32_t k = 0; k < 4; ++k) {
+        const uint32_t m = pref[k];
+        if (m > mpx_max || p.msplit % m != 0u) continue;
+        for (uint32_t c = 1; c * m <= 32u; ++c) {
+            if (p.ngroups % c != 0u) continue;
+            const uint32_t nrect = (p.msplit / m) * (p.ngroups / c);
+            const uint32_t busiest = ((nrect + 7u) / 8u) * m * c;
+            const uint64_t rounds = (busiest + 31u) / 32u;
+            const uint64_t uneven = (uint64_t)busiest * 100u > (uint64_t)even * 115u ? 1u : 0u;
+            const uint64_t key = (rounds << 40) | (uneven << 36) | ((uint64_t)(32u - m * c) << 24) |
+                                 ((uint64_t)k << 20) | busiest;
+            if (key < best_key) {
+                best_key = key;
+                p.mpx = m;
+                p.cgx = c;
+                p.nrect = nrect;
+            }
+        }
+    }
+    p.grid = ((p.nrect + 7u) / 8u) * 8u * p.mpx * p.cgx;
+    return p;
+}
+
+}  // namespace xreg
+}  // namespace mi

@@ -173,6 +173,48 @@ def test_gemm_k1024_launch_plans(pkg, oracle, M, N, K):
     assert _rel(oracle, C[idx], want) <= 2e-2
 
 
+# fp32 at K = 1024 runs the register-resident fp32 kernel: groups of 64 columns, 64-row blocks, one
+# 4-byte store per lane and row.  Shapes around every tile boundary (edge store path, one row
+# block, odd and even numbers of row blocks), several scales, against the fp64 oracle at 1e-5.
+@pytest.mark.parametrize("M,N", [(1, 1), (63, 63), (64, 64), (65, 65), (128, 64), (129, 127), (192, 130),
+                                 (577, 333), (130, 1000), (2048, 70), (700, 1023)])
+def test_gemm_f32_k1024_tile_boundaries(pkg, oracle, M, N):
+    K = 1024
+    W, Xt = oracle.inputs_gemm(M, N, K, torch.float32)
+    for scale in (None, 0.37 / 32.0, 1.0):
+        s = 1.0 / math.sqrt(K) if scale is None else scale
+        for _ in range(2):                                   # back-to-back launches reuse LDS and registers
+            C = pkg.fused_ht_gemm(W.cuda(), Xt.cuda(), scale)
+        torch.cuda.synchronize()
+        want = oracle.fused_ht_gemm_f64_blas(W.double().numpy(), Xt.double().numpy(), s)
+        assert C.shape == (M, N) and C.dtype == torch.float32
+        err = np.abs(C.cpu().double().numpy() - want).max() / max(np.abs(want).max(), s * K)
+        assert err <= 1e-5, (M, N, scale, err)
+
+
+# fp32, K = 1024, launch plans other than the benchmark's (ragged slices, more than one round of
+# workgroups, rectangles that leave workgroup ids without work): every element against the product
+# of W with the library's own fp32 transform, accumulated in fp64 on the device.
+@pytest.mark.parametrize("M,N", [(4096, 4096), (5000, 3000), (2048, 8192), (12288, 1536), (1000, 9000)])
+def test_gemm_f32_k1024_launch_plans(pkg, oracle, M, N):
+    K = 1024
+    g = torch.Generator(device="cuda").manual_seed(M + N)
+    Wd = torch.randn(M, K, generator=g, device="cuda")
+    Xd = torch.randn(N, K, generator=g, device="cuda")
+    Y = pkg.hadamard_transform(Xd, 1.0 / 32.0)
+    C = pkg.fused_ht_gemm(Wd, Xd, 1.0 / 32.0)
+    torch.cuda.synchronize()
+    assert torch.isfinite(C).all()
+    worst = 0.0
+    for r0 in range(0, M, 1024):                             # fp64 product in slices (memory)
+        ref = Wd[r0:r0 + 1024].double() @ Y.double().t()
+        worst = max(worst, (C[r0:r0 + 1024].double() - ref).abs().max().item())
+    assert worst / 32.0 <= 1e-5, worst
+    idx = torch.tensor([0, 63, 64, M // 2, M - 1])
+    want = oracle.fused_ht_gemm_f64_blas(Wd[idx].cpu().double().numpy(), Xd.cpu().double().numpy(), 1.0 / 32.0)
+    assert _rel(oracle, C[idx], want) <= 1e-5
+
+
 def test_gemm_small_bruteforce(pkg, oracle):
     # triple-loop oracle (no BLAS), fp32
     M, N, K = 16, 20, 64
