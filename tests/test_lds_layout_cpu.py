@@ -52,6 +52,6 @@ def test_checker_rejects_unswizzled_rows_and_misaligned_pieces():
 
 
 def test_kernels_apply_the_checker_to_their_own_layouts():
-    for name in ("fused_gemm_xreg.hip", "fused_gemm.hip", "fp8_gemm.hip"):
+    for name in ("xreg_common.hpp", "fused_gemm.hip", "fp8_gemm.hip"):
         text = open(os.path.join(CSRC, name)).read()
         assert "lds::conflict_free_b128" in text and "static_assert" in text, name
