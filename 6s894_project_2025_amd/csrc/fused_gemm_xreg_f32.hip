@@ -34,19 +34,60 @@ __device__ __forceinline__ void xmfma_f32_next(f32x4& c, float a, float b)
     asm volatile("v_mfma_f32_16x16x4_f32 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
 }
 
+// Geometry by K: a wavefront's 256 accumulation registers hold 16 NBF columns x K values.
+template <int K>
+struct GeomF32 {
+    static_assert(K == 256 || K == 512 || K == 1024, "16 NBF columns x K fp32 values = 256 registers per lane");
+    static constexpr int NBF = 1024 / K;      // 16-column fragments per wavefront
+    static constexpr int CPW = 16 * NBF;      // columns per wavefront
+    static constexpr int COLS = 4 * CPW;      // columns per workgroup
+    static constexpr int KSTEPS = K / 16;     // 16-byte fragments (4 k per lane, 16 k per step) per column
+    static constexpr int SPB = K / 128;       // W stages (64 rows x 128 k) per row block
+    static constexpr int AHEAD = SPB >= 3 ? 3 : SPB;  // stages the W stream runs ahead of the MFMAs
+    static constexpr int NM = 16 * NBF;       // MFMAs per K step: 4 row fragments x 4 k x NBF
+    static constexpr int RCOLS = 4 * NBF;     // columns that pass through the LDS area together
+};
+
+// The prologue's LDS area of a wavefront (16 KB): [4 NBF columns][K / 4 chunks], chunk q of column
+// c stored at q ^ 2 (c / NBF).  Every lane writes one chunk of a column (consecutive lanes,
+// consecutive chunks); in round p only the lanes with lo / 4 == p read, chunk 4 s + hi of the
+// columns NBF (lo % 4) + f.
+template <int K>
+__host__ __device__ constexpr uint32_t area_f32_offset(uint32_t c, uint32_t q)
+{
+    return c * (uint32_t)K * 4u + ((q ^ (2u * (c / (uint32_t)GeomF32<K>::NBF))) << 4);
+}
+template <int K>
+constexpr bool area_f32_conflict_free()
+{
+    constexpr uint32_t NBF = GeomF32<K>::NBF;
+    for (uint32_t c = 0; c < 4u * NBF; ++c)
+        for (uint32_t t = 0; t < (uint32_t)K / 256u; ++t)
+            if (!lds::conflict_free_b128([=](uint32_t lane) { return area_f32_offset<K>(c, 64u * t + lane); }))
+                return false;
+    for (uint32_t f = 0; f < NBF; ++f)
+        for (uint32_t p = 0; p < 4; ++p)
+            for (uint32_t s = 0; s < (uint32_t)K / 16u; ++s)
+                if (!lds::conflict_free_b128_masked(
+                        [=](uint32_t lane) { return area_f32_offset<K>(NBF * (lane & 3u) + f, 4u * s + (lane >> 4)); },
+                        [=](uint32_t lane) { return ((lane & 15u) >> 2) == p; }))
+                    return false;
+    return true;
+}
+static_assert(area_f32_conflict_free<256>() && area_f32_conflict_free<512>() && area_f32_conflict_free<1024>(),
+              "an LDS access pattern of the fp32 prologue would serialise");
+
 template <int K>
 __global__ void __launch_bounds__(kThreads)
 fused_ht_gemm_xreg_f32_kernel(const float* __restrict__ W, const float* __restrict__ Xt,
                               float* __restrict__ C, uint32_t M, uint32_t N, uint32_t m_per_block,
                               uint32_t msplit, uint32_t mpx, uint32_t cgx, uint32_t nrect, float fscale)
 {
-    static_assert(K == 1024, "16 columns x K fp32 values = 256 registers per lane");
-    constexpr int KSTEPS = K / 16;        // 16-byte fragments (4 k per lane, 16 k per step) per column
-    constexpr int SPB = K / 128;          // W stages (64 rows x 128 k) per row block
-    constexpr int AHEAD = 3;              // stages the W stream runs ahead of the MFMAs
-    constexpr int NM = 16;                // MFMAs per K step: 4 row fragments x 4 k
-    constexpr uint32_t kCols = 64, CPW = 16;
-    static_assert(kSlots == 4 && AHEAD <= SPB && (SPB & 3) == 0, "stage g lives in buffer g % 4");
+    using G = GeomF32<K>;
+    constexpr int NBF = G::NBF, KSTEPS = G::KSTEPS, SPB = G::SPB, AHEAD = G::AHEAD, NM = G::NM;
+    constexpr uint32_t kCols = G::COLS, CPW = G::CPW;
+    static_assert(kSlots == 4 && AHEAD <= SPB && AHEAD >= 1, "stage g of the stream lives in buffer g % 4");
+    static_assert(G::RCOLS * K * 4 == kAreaBytes, "a round of columns fills the wavefront's LDS area");
     constexpr uint32_t ROW_BYTES = K * 4u;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -81,61 +122,92 @@ fused_ht_gemm_xreg_f32_kernel(const float* __restrict__ W, const float* __restri
     };
     set_voff(0);
 
-    // ---- prologue: fragment column lo of this wavefront = column n0 + 16 w + lo -------------------
-    // (scalars, not 4-vectors: an MFMA names one register, and the compiler keeps a vector's
-    // elements in the accumulation-register file only as a whole; with vectors it copied every
-    // element into one scratch register right before use, while the previous MFMA was still
-    // reading that register)
-    float yf[KSTEPS][4];
+    // ---- prologue: column f of lane (., lo) = column n0 + CPW w + NBF lo + f ------------------------
+    // The wavefront's columns pass through its LDS area in four rounds of 4 NBF columns = eight
+    // 512-element tiles (K = 1024: two tiles and one butterfly per column; K = 512: a tile per
+    // column; K = 256: two columns per tile, the tile's high index bit left alone).
+    // (yf is an array of scalars, not of 4-vectors: an MFMA names one register, and the compiler
+    // keeps a vector's elements in the accumulation-register file only as a whole; with vectors
+    // it copied every element into one scratch register right before use, while the previous MFMA
+    // was still reading that register)
+    float yf[NBF][KSTEPS][4];
     {
         unsigned char* area = lds + kAreaBase + wave * kAreaBytes;
         TileOperands<BF16> ops;
-        make_tile_operands<BF16, 4>(10, ops);
-        float in[4][2][8];
-        auto load_col = [&](int p4, int c) {
-            const uint32_t col = min(n0 + CPW * wave + (uint32_t)(4 * p4 + c), N - 1u);
+        make_tile_operands<BF16, 4>(K >= 512 ? 9 : 8, ops);
+        float in[8][8];
+        auto load_tile = [&](int p4, int i) {
 #pragma unroll
-            for (int tile = 0; tile < 2; ++tile)
+            for (int t = 0; t < 2; ++t) {
+                const uint32_t o = 512u * i + 256u * t;  // offset inside the round's columns
+                const uint32_t col = min(n0 + CPW * wave + (uint32_t)(G::RCOLS * p4) + o / K, N - 1u);
+                const f32x4 q = *reinterpret_cast<const f32x4*>(Xt + ((uint64_t)col * K + o % K + 4u * lane));
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    const f32x4 q = *reinterpret_cast<const f32x4*>(
-                        Xt + ((uint64_t)col * K + 512u * tile + 256u * t + 4u * lane));
+                for (int r = 0; r < 4; ++r) in[i][4 * t + r] = q[r];
+            }
+        };
+        auto w_first = [&](int i) {  // the first AHEAD stages of W, behind the last round of X
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) in[c][tile][4 * t + r] = q[r];
-                }
+            for (int u = 0; u < AHEAD; ++u) {
+                const int pc = AHEAD * i + u;
+                w_issue(pc >> 3, pc >> 3, pc & 7);
+            }
+        };
+        auto put = [&](uint32_t c, uint32_t q, f32x4 v) {
+            *reinterpret_cast<f32x4*>(area + area_f32_offset<K>(c, q)) = v * fscale;
         };
 #pragma unroll
-        for (int c = 0; c < 4; ++c) load_col(0, c);
+        for (int i = 0; i < 8; ++i) load_tile(0, i);
 #pragma unroll
         for (int p4 = 0; p4 < 4; ++p4) {
+            if constexpr (K == 1024) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                f32x4 a0[2], a1[2];
-                tile_transform_f32(in[c][0], ops, a0);
-                tile_transform_f32(in[c][1], ops, a1);
-                if (p4 + 1 < 4) load_col(p4 + 1, c);
-                if (p4 == 3) {  // the first AHEAD stages of W, behind the last X tile
+                for (int c = 0; c < 4; ++c) {
+                    f32x4 a0[2], a1[2];
+                    tile_transform_f32(in[2 * c], ops, a0);
+                    tile_transform_f32(in[2 * c + 1], ops, a1);
+                    if (p4 + 1 < 4) {
+                        load_tile(p4 + 1, 2 * c);
+                        load_tile(p4 + 1, 2 * c + 1);
+                    } else {
+                        w_first(2 * c);
+                        w_first(2 * c + 1);
+                    }
+                    // element 512 half + 256 t + 4 lane + r of the column = chunk 128 half + 64 t + lane
 #pragma unroll
-                    for (int u = 0; u < 2 * AHEAD; ++u) {
-                        const int pc = 2 * AHEAD * c + u;
-                        w_issue(pc >> 3, pc >> 3, pc & 7);
+                    for (int t = 0; t < 2; ++t) {
+                        put(c, 64u * t + lane, a0[t] + a1[t]);
+                        put(c, 128u + 64u * t + lane, a0[t] - a1[t]);
                     }
                 }
-                // element 512 half + 256 t + 4 lane + r of the column = chunk 128 half + 64 t + lane
+            } else {
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    *reinterpret_cast<f32x4*>(area + area4_offset(c, 64u * t + lane)) = (a0[t] + a1[t]) * fscale;
-                    *reinterpret_cast<f32x4*>(area + area4_offset(c, 128u + 64u * t + lane)) =
-                        (a0[t] - a1[t]) * fscale;
+                for (int i = 0; i < 8; ++i) {
+                    f32x4 a[2];
+                    tile_transform_f32(in[i], ops, a);
+                    if (p4 + 1 < 4)
+                        load_tile(p4 + 1, i);
+                    else
+                        w_first(i);
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        if constexpr (K == 512)
+                            put(i, 64u * t + lane, a[t]);  // element 256 t + 4 lane + r of column i
+                        else
+                            put(2 * i + t, lane, a[t]);    // element 4 lane + r of column 2 i + t
+                    }
                 }
             }
             if ((int)(lo >> 2) == p4) {
 #pragma unroll
-                for (int s = 0; s < KSTEPS; ++s) {
-                    const f32x4 q = *reinterpret_cast<const f32x4*>(area + area4_offset(lo & 3u, 4u * s + hi));
+                for (int f = 0; f < NBF; ++f)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) yf[s][e] = q[e];
-                }
+                    for (int s = 0; s < KSTEPS; ++s) {
+                        const f32x4 q = *reinterpret_cast<const f32x4*>(
+                            area + area_f32_offset<K>(NBF * (lo & 3u) + f, 4u * s + hi));
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) yf[f][s][e] = q[e];
+                    }
             }
         }
     }
@@ -155,38 +227,56 @@ fused_ht_gemm_xreg_f32_kernel(const float* __restrict__ W, const float* __restri
         fr[1][mb] = frag(0, mb, 1);
     }
 
-    // lane (hi, lo) of a row block owns rows 16 mb + 4 hi + r of column n0 + 16 w + lo
-    const uint32_t col = n0 + CPW * wave + lo;
-    const uint32_t lane_off = (4u * hi * N + col) * 4u;  // inside the row block, < 2^32
+    // lane (hi, lo) of a row block owns rows 16 mb + 4 hi + r of columns col0 .. col0 + NBF - 1
+    const uint32_t col0 = n0 + CPW * wave + NBF * lo;
+    const uint32_t lane_off = (4u * hi * N + col0) * 4u;  // inside the row block, < 2^32
     unsigned char* const Cb = reinterpret_cast<unsigned char*>(C);
-    const bool cols_full = n0 + kCols <= N;
-    auto store_one = [&](const f32x4 (&acc)[4][1], uint64_t block_base, int mb, int r)
+    const bool cols_full = n0 + kCols <= N && N % NBF == 0u;  // vector stores need aligned rows
+    auto store_one = [&](const f32x4 (&acc)[4][NBF], uint64_t block_base, int mb, int r)
         __attribute__((always_inline)) {
         unsigned char* row_ptr = Cb + (block_base + (uint64_t)((16u * mb + r) * N) * 4u);  // scalar
-        const float v = acc[mb][0][r];  // (a bit cast applied to the element expression itself reads element 0)
-        stream_store4(lane_off, __float_as_uint(v), row_ptr);
+        // (locals: a bit cast applied to a vector element expression itself reads element 0)
+        const float v0 = acc[mb][0][r];
+        if constexpr (NBF == 1) {
+            stream_store4(lane_off, __float_as_uint(v0), row_ptr);
+        } else if constexpr (NBF == 2) {
+            const float v1 = acc[mb][1][r];
+            stream_store8(lane_off, u32x2{__float_as_uint(v0), __float_as_uint(v1)}, row_ptr);
+        } else {
+            const float v1 = acc[mb][1][r], v2 = acc[mb][2][r], v3 = acc[mb][3][r];
+            stream_store16(lane_off,
+                           u32x4{__float_as_uint(v0), __float_as_uint(v1), __float_as_uint(v2), __float_as_uint(v3)},
+                           row_ptr);
+        }
     };
-    auto store_edge = [&](const f32x4 (&acc)[4][1], uint32_t row_base) __attribute__((always_inline)) {
-        if (col >= N) return;
+    auto store_edge = [&](const f32x4 (&acc)[4][NBF], uint32_t row_base) __attribute__((always_inline)) {
 #pragma unroll
-        for (int mb = 0; mb < 4; ++mb)
+        for (int f = 0; f < NBF; ++f) {
+            if (col0 + f >= N) continue;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const uint32_t row = row_base + 16u * mb + 4u * hi + r;
-                if (row < m_end) C[(uint64_t)row * N + col] = acc[mb][0][r];
-            }
+            for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint32_t row = row_base + 16u * mb + 4u * hi + r;
+                    if (row < m_end) C[(uint64_t)row * N + col0 + f] = acc[mb][f][r];
+                }
+        }
     };
 
-    auto row_block_body = [&](auto prev_tag, f32x4 (&acc)[4][1], const f32x4 (&prev)[4][1],
+    // One row block: SPB stages of 8 K steps of NM MFMAs.  `second`: the block is the odd one of a
+    // pair (its stages start at buffer SPB % 4).  `prev_full`: `prev` holds the finished previous
+    // block, stored behind the MFMAs of K step 6.
+    auto row_block_body = [&](auto prev_tag, auto second_tag, f32x4 (&acc)[4][NBF], const f32x4 (&prev)[4][NBF],
                               uint64_t prev_base, uint32_t rbi) __attribute__((always_inline)) {
         constexpr bool prev_full = decltype(prev_tag)::value;
+        constexpr int slot_base = decltype(second_tag)::value ? (SPB & 3) : 0;
         const bool last = rbi + 1u == nrb;
 #pragma unroll
         for (int kq = 0; kq < SPB; ++kq) {
             constexpr int kPieceAt[7] = {0, 2, 4, 5, 6, 7, 8};
-            // (everything below folds to constants once the loops are unrolled; SPB is a multiple
-            // of 4, so stage kq of every row block lives in buffer kq % 4)
-            const int cur_slot = kq & 3, next_slot = (kq + 1) & 3, fill_slot = (kq + AHEAD) & 3;
+            // (everything below folds to constants once the loops are unrolled)
+            const int cur_slot = (slot_base + kq) & 3, next_slot = (slot_base + kq + 1) & 3;
+            const int fill_slot = (slot_base + kq + AHEAD) & 3;
             const int fill_kq = (kq + AHEAD) % SPB;
             const bool fill_own_block = kq + AHEAD < SPB;
 #pragma unroll
@@ -195,24 +285,25 @@ fused_ht_gemm_xreg_f32_kernel(const float* __restrict__ W, const float* __restri
                 const int kk = kq * kStepsPerStage + ks;
 #pragma unroll
                 for (int m = 0; m < NM; ++m) {
-                    const int s = m >> 2, mb = m & 3;  // consecutive MFMAs go to different accumulators
+                    // consecutive MFMAs go to different accumulators
+                    const int s = m / (4 * NBF), mb = m & 3, f = (m >> 2) % NBF;
                     if (kk == 0 && s == 0)
-                        xmfma_f32_first(acc[mb][0], fr[ks & 3][mb][s], yf[0][s]);
+                        xmfma_f32_first(acc[mb][f], fr[ks & 3][mb][s], yf[f][0][s]);
                     else
-                        xmfma_f32_next(acc[mb][0], fr[ks & 3][mb][s], yf[kk][s]);
+                        xmfma_f32_next(acc[mb][f], fr[ks & 3][mb][s], yf[f][kk][s]);
                     // one memory instruction in the shadow of an MFMA: fragments two K steps ahead
-                    // (m = 12 .. 15: their registers were last read by the MFMAs of two steps ago),
-                    // up to two transfer pieces, the previous block's sixteen stores
-                    if (m >= 12)
-                        fr[(ks + 2) & 3][m - 12] =
-                            ks < 6 ? frag(cur_slot, m - 12, ks + 2) : frag(next_slot, m - 12, ks - 6);
+                    // (the last four MFMAs: their registers were last read by the MFMAs of two
+                    // steps ago), up to two transfer pieces, the previous block's sixteen stores
+                    if (m >= NM - 4)
+                        fr[(ks + 2) & 3][m - (NM - 4)] = ks < 6 ? frag(cur_slot, m - (NM - 4), ks + 2)
+                                                                : frag(next_slot, m - (NM - 4), ks - 6);
                     else if (m >= 4 && m < 6) {
                         if (ks < 6 && (fill_own_block || !last)) {
                             const int i = kPieceAt[ks] + (m - 4);
                             if (i < kPieceAt[ks + 1]) w_issue(fill_kq, fill_slot, i);
                         }
                     }
-                    if (prev_full && kk == 6) store_one(prev, prev_base, m >> 2, m & 3);
+                    if (prev_full && kk == 6 && m < 16) store_one(prev, prev_base, m >> 2, m & 3);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 // keep the previous step's fragment registers allocated while the matrix core may
@@ -233,24 +324,14 @@ fused_ht_gemm_xreg_f32_kernel(const float* __restrict__ W, const float* __restri
         }
     };
 
-    auto store_block = [&](f32x4 (&acc)[4][1], uint64_t base) __attribute__((always_inline)) {
+    auto store_block = [&](f32x4 (&acc)[4][NBF], uint64_t base) __attribute__((always_inline)) {
         drain_mfma(acc);
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
             for (int r = 0; r < 4; ++r) store_one(acc, base, mb, r);
     };
-    f32x4 accA[4][1], accB[4][1];
-    bool pend = false;        // accB holds a finished full row block that is not stored yet
-    uint64_t pend_base = 0;
-    auto run = [&](bool prev_full, f32x4 (&acc)[4][1], const f32x4 (&prev)[4][1], uint64_t prev_base,
-                   uint32_t rbi) __attribute__((always_inline)) {
-        if (prev_full)
-            row_block_body(std::true_type{}, acc, prev, prev_base, rbi);
-        else
-            row_block_body(std::false_type{}, acc, prev, prev_base, rbi);
-    };
-    auto finish = [&](f32x4 (&acc)[4][1], uint32_t rbi, bool& full, uint64_t& base)
+    auto finish = [&](f32x4 (&acc)[4][NBF], uint32_t rbi, bool& full, uint64_t& base)
         __attribute__((always_inline)) {
         const uint32_t row_base = m_begin + row_block(rbi) * kRows;
         full = cols_full && row_base + kRows <= m_end;
@@ -260,43 +341,85 @@ fused_ht_gemm_xreg_f32_kernel(const float* __restrict__ W, const float* __restri
             store_edge(acc, row_base);
         }
     };
+    if constexpr (NBF <= 2) {
+        // two accumulator sets: a finished block is stored behind the MFMAs of the next one
+        f32x4 accA[4][NBF], accB[4][NBF];
+        bool pend = false;        // accB holds a finished full row block that is not stored yet
+        uint64_t pend_base = 0;
+        auto run = [&](bool prev_full, auto second_tag, f32x4 (&acc)[4][NBF], const f32x4 (&prev)[4][NBF],
+                       uint64_t prev_base, uint32_t rbi) __attribute__((always_inline)) {
+            if (prev_full)
+                row_block_body(std::true_type{}, second_tag, acc, prev, prev_base, rbi);
+            else
+                row_block_body(std::false_type{}, second_tag, acc, prev, prev_base, rbi);
+        };
 #pragma unroll 1
-    for (uint32_t rbi = 0; rbi < nrb; rbi += 2u) {
-        run(pend, accA, accB, pend_base, rbi);
-        bool fullA;
-        uint64_t baseA;
-        finish(accA, rbi, fullA, baseA);
-        if (rbi + 1u < nrb) {
-            run(fullA, accB, accA, baseA, rbi + 1u);
-            finish(accB, rbi + 1u, pend, pend_base);
-        } else {
-            pend = false;
-            if (fullA) store_block(accA, baseA);
+        for (uint32_t rbi = 0; rbi < nrb; rbi += 2u) {
+            run(pend, std::false_type{}, accA, accB, pend_base, rbi);
+            bool fullA;
+            uint64_t baseA;
+            finish(accA, rbi, fullA, baseA);
+            if (rbi + 1u < nrb) {
+                run(fullA, std::true_type{}, accB, accA, baseA, rbi + 1u);
+                finish(accB, rbi + 1u, pend, pend_base);
+            } else {
+                pend = false;
+                if (fullA) store_block(accA, baseA);
+            }
+        }
+        if (pend) store_block(accB, pend_base);
+    } else {
+        // one accumulator set (the registers do not hold two): stored right after its block
+        f32x4 acc[4][NBF];
+        auto one = [&](auto second_tag, uint32_t rbi) __attribute__((always_inline)) {
+            row_block_body(std::false_type{}, second_tag, acc, acc, 0, rbi);
+            bool full;
+            uint64_t base;
+            finish(acc, rbi, full, base);
+            if (full) store_block(acc, base);
+        };
+#pragma unroll 1
+        for (uint32_t rbi = 0; rbi < nrb; rbi += 2u) {
+            one(std::false_type{}, rbi);
+            if (rbi + 1u < nrb) one(std::true_type{}, rbi + 1u);
         }
     }
-    if (pend) store_block(accB, pend_base);
 }
 
 }  // namespace xreg
 
-// Called by the fp32 dispatcher of mi_fused_ht_gemm for K = 1024 (arguments already validated).
-int fused_gemm_f32_xreg(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, uint32_t K,
-                        float scale, hipStream_t s)
+namespace {
+template <int K>
+int launch_xreg_f32(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, float scale, hipStream_t s)
 {
     using namespace xreg;
-    if (K != 1024u) return MI_ERR_SIZE;
-    // W and a row block of C are addressed with 32-bit byte offsets
-    if ((uint64_t)M * K * 4u > 0xffffffffull || (uint64_t)N * 4u * 64u > 0xffffffffull) return MI_ERR_SHAPE;
-    const int shift = tile_stage_shift<4>(10, false);
+    constexpr uint32_t log2k = K == 256 ? 8 : K == 512 ? 9 : 10;
+    const int shift = tile_stage_shift<4>(log2k, false);
     const float fscale = (float)((double)scale * (double)(1u << shift));
-    const Plan p = plan(M, N, 64u, 8u);
-    auto kern = fused_ht_gemm_xreg_f32_kernel<1024>;
+    const Plan p = plan(M, N, (uint32_t)GeomF32<K>::COLS, 8u);
+    auto kern = fused_ht_gemm_xreg_f32_kernel<K>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             kLdsBytes) != hipSuccess)
         return MI_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3(p.grid), dim3(kThreads), kLdsBytes, s, W, Xt, C, M, N, p.m_per_block,
                        p.msplit, p.mpx, p.cgx, p.nrect, fscale);
     return launch_status();
+}
+}  // namespace
+
+// Called by the fp32 dispatcher of mi_fused_ht_gemm for K = 256, 512, 1024 (arguments already
+// validated).
+int fused_gemm_f32_xreg(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, uint32_t K,
+                        float scale, hipStream_t s)
+{
+    // W and a row block of C are addressed with 32-bit byte offsets
+    if ((uint64_t)M * K * 4u > 0xffffffffull || (uint64_t)N * 4u * 64u > 0xffffffffull) return MI_ERR_SHAPE;
+    switch (K) {
+        case 256: return launch_xreg_f32<256>(W, Xt, C, M, N, scale, s);
+        case 512: return launch_xreg_f32<512>(W, Xt, C, M, N, scale, s);
+        case 1024: return launch_xreg_f32<1024>(W, Xt, C, M, N, scale, s);
+        default: return MI_ERR_SIZE;
+    }
 }
 
 }  // namespace mi
