@@ -227,8 +227,8 @@ int fused_gemm_f32(const float* W, const float* Xt, float* C, uint32_t M, uint32
         case 128: return launch<32, 0>(W, Xt, C, M, N, K, scale, s);
         case 256:
         case 512:
-        case 1024: return fused_gemm_f32_xreg(W, Xt, C, M, N, K, scale, s);
-        case 2048: return launch<16, 2>(W, Xt, C, M, N, K, scale, s);
+        case 1024:
+        case 2048: return fused_gemm_f32_xreg(W, Xt, C, M, N, K, scale, s);
         case 4096: return launch<16, 2, 2>(W, Xt, C, M, N, K, scale, s);  // two passes of K = 2048
         default: return MI_ERR_SIZE;
     }

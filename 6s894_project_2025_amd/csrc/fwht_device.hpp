@@ -176,9 +176,14 @@ __device__ __forceinline__ void split3(float x, __bf16& h, __bf16& m, __bf16& l)
     l = (__bf16)(r - (float)m);
 }
 
-// fp32 tile on the bf16 matrix cores: every stage multiplies the three bf16 pieces of its input
-// by the +-2^-k Hadamard operand and accumulates in fp32, so each product is exact and the only
-// rounding is the fp32 accumulation.  v[j] = the lane's 8 elements under TileMap<4>.
+// fp32 tile.  Stage 1 runs on the bf16 matrix cores: the three bf16 pieces of every input are
+// multiplied by the +-2^-k Hadamard operand and accumulated in fp32, so each product is exact and
+// the only rounding is the fp32 accumulation.  Stage 2 takes the fp32 sums as they are, as the A
+// operand of four v_mfma_f32_16x16x4_f32 (MFMA r contracts index 4 hi + r: A[lo][hi] = d1[r],
+// B[hi][lo] = G2[4 hi + r][lo]); again every product is exact.  That costs 128 matrix-core cycles
+// per half tile instead of 48, and saves the second three-way split, half of the vector
+// arithmetic of the tile, which is what bounds the callers that transform many tiles per
+// wavefront.  v[j] = the lane's 8 elements under TileMap<4>.
 // Result acc[t][r] = element 256t + 4*lane + r.
 __device__ __forceinline__ void tile_transform_f32(const float (&v)[8],
                                                    const TileOperands<BF16>& ops, f32x4 (&acc)[2])
@@ -192,24 +197,19 @@ __device__ __forceinline__ void tile_transform_f32(const float (&v)[8],
         m[j] = b;
         l[j] = c;
     }
+    float g2f[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) g2f[r] = (float)ops.g2[r];
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
         f32x4 d1 = BF16::mfma32(l, ops.g1[t], zero);
         d1 = BF16::mfma32(m, ops.g1[t], d1);
         d1 = BF16::mfma32(h, ops.g1[t], d1);
-        bf16x4 h2, m2, l2;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            __bf16 a, b, c;
-            split3(d1[r], a, b, c);
-            h2[r] = a;
-            m2[r] = b;
-            l2[r] = c;
-        }
-        f32x4 d2 = BF16::mfma16(l2, ops.g2, zero);
-        d2 = BF16::mfma16(m2, ops.g2, d2);
-        acc[t] = BF16::mfma16(h2, ops.g2, d2);
+        f32x4 d2 = __builtin_amdgcn_mfma_f32_16x16x4f32(d1[0], g2f[0], zero, 0, 0, 0);
+        d2 = __builtin_amdgcn_mfma_f32_16x16x4f32(d1[1], g2f[1], d2, 0, 0, 0);
+        d2 = __builtin_amdgcn_mfma_f32_16x16x4f32(d1[2], g2f[2], d2, 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(d1[3], g2f[3], d2, 0, 0, 0);
     }
 }
 
