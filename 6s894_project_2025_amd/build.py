@@ -6,7 +6,9 @@ hipcc cross-compiles without a GPU, so this works on a CPU-only machine.
 from __future__ import annotations
 
 import concurrent.futures
+import glob
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -39,6 +41,41 @@ PER_FILE_FLAGS = {
 }
 
 
+# The register-resident kernels issue their main-loop MFMAs as inline assembly with the B operand
+# named directly in the accumulation-register file.  If register pressure ever makes the compiler
+# keep part of that operand elsewhere, it copies the value into one accumulation register right
+# before each use - while the previous MFMA may still be reading that register, which silently
+# corrupts results.  The build therefore looks at the generated ISA of these files and fails when an
+# accumulation register is written anywhere after a kernel's first such MFMA.
+ISA_CHECKED = {"fused_gemm_xreg.hip", "fused_gemm_xreg_f32.hip"}
+_MFMA_B_IN_AGPR = re.compile(r"^\s*v_mfma_\S+\s+v\[[0-9:]+\], v\S+, a")
+_AGPR_WRITE = re.compile(r"^\s*v_accvgpr_(write|mov)")
+_LABEL = re.compile(r"^([A-Za-z_][\w$]*):")
+
+
+def check_register_resident_isa(asm_text: str, where: str) -> int:
+    """Raises if a kernel writes accumulation registers after its first MFMA that reads its B
+    operand from them; returns the number of kernels checked."""
+    kernels = 0
+    name, armed = None, False
+    for line in asm_text.splitlines():
+        label = _LABEL.match(line)
+        if label:  # a function (local labels start with a dot)
+            name, armed = label.group(1), False
+            continue
+        if name is None:
+            continue
+        if "s_endpgm" in line:
+            kernels += armed
+            name, armed = None, False
+        elif _MFMA_B_IN_AGPR.match(line):
+            armed = True
+        elif armed and _AGPR_WRITE.match(line):
+            raise RuntimeError(f"{where}: {name} writes an accumulation register inside its MFMA loop "
+                               f"({line.strip()}): the transformed operand no longer fits the register file")
+    return kernels
+
+
 def sources() -> list[str]:
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
@@ -51,15 +88,28 @@ def _hipcc() -> str:
 
 
 def _compile(src: str) -> str:
-    obj = os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, *PER_FILE_FLAGS.get(os.path.basename(src), []), "-c", src, "-o",
-           obj]
+    base = os.path.basename(src)
+    obj = os.path.join(OBJ_DIR, base[:-4] + ".o")
+    checked = base in ISA_CHECKED
+    cmd = [_hipcc(), *HIPCC_FLAGS, *PER_FILE_FLAGS.get(base, []), *(["-save-temps=obj"] if checked else []),
+           "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "recognized feature" not in l)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{err}")
     if err.strip():
         sys.stderr.write(err + "\n")
+    if checked:
+        temps = glob.glob(os.path.join(OBJ_DIR, base[:-4] + "-*")) + glob.glob(os.path.join(OBJ_DIR, base + "-*"))
+        isa = [t for t in temps if t.endswith(f"{ARCH}.s")]
+        if len(isa) != 1:
+            raise RuntimeError(f"no device assembly found for {src}")
+        with open(isa[0]) as f:
+            n = check_register_resident_isa(f.read(), base)
+        if n == 0:
+            raise RuntimeError(f"{base}: no register-resident MFMA loop found in the device assembly")
+        for t in temps:
+            os.remove(t)
     return obj
 
 

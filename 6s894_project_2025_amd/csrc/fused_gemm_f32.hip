@@ -228,8 +228,8 @@ int fused_gemm_f32(const float* W, const float* Xt, float* C, uint32_t M, uint32
         case 256:
         case 512:
         case 1024:
-        case 2048: return fused_gemm_f32_xreg(W, Xt, C, M, N, K, scale, s);
-        case 4096: return launch<16, 2, 2>(W, Xt, C, M, N, K, scale, s);  // two passes of K = 2048
+        case 2048:
+        case 4096: return fused_gemm_f32_xreg(W, Xt, C, M, N, K, scale, s);
         default: return MI_ERR_SIZE;
     }
 }

@@ -386,32 +386,48 @@ fused_ht_gemm_xreg_f32_kernel(const float* __restrict__ W, const float* __restri
     }
 }
 
-// ---- K = 2048: the K range split over pairs of wavefronts ----------------------------------------
+// ---- K = 2048, 4096: the K range split over pairs of wavefronts ---------------------------------
 // A wavefront's registers hold 16 columns x 1024 values and the matrix core is 16 columns wide, so
-// at K = 2048 wavefront (cs, kp) = (wave / 2, wave % 2) holds half kp of the transformed columns
-// 16 cs .. 16 cs + 15 (32 columns per workgroup): H_2048 x = [Ya + Yb; Ya - Yb] with Ya, Yb the
-// 1024-point transforms of the two halves of x.  W is streamed as two streams (k < 1024 and
-// k >= 1024), each through its own ring of four 16 KB stages (64 rows x 64 k); a wavefront reads
-// the fragments of its own stream only.  At the end of a row block each wavefront of a pair hands
-// the partner two of its four 16-row accumulator fragments through LDS and finishes (adds, stores)
-// the other two.
+// for larger K wavefront (cs, kp) = (wave / 2, wave % 2) holds one 1024-value quarter of the
+// transformed columns 16 cs .. 16 cs + 15 (32 columns per workgroup).  With T_i the 1024-point
+// transform of quarter i of a column x, H_K x has the quarters
+//     K = 2048:  Y_0 = T_0 + T_1,  Y_1 = T_0 - T_1
+//     K = 4096:  Y_j = sum_i (-1)^popcount(i & j) T_i
+// K = 4096 runs two phases, one launch each: in phase ph the pair holds Y_{2 ph} and Y_{2 ph + 1}
+// and walks all of its row blocks; phase 1 adds what phase 0 stored.  (One launch with a loop over
+// the phases made the compiler carry values of the prologue across the main loop, and with them
+// some of the transformed operand out of the accumulation registers.)
+// W is streamed as two streams (the K ranges of the pair's two quarters), each through its own
+// ring of four 16 KB stages (64 rows x 64 k); a wavefront reads the fragments of its own stream
+// only.  At the end of a row block each wavefront of a pair hands the partner two of its four
+// 16-row accumulator fragments through LDS and finishes (adds, stores) the other two.
+// The prologue is shared inside a pair: per round, wavefront kp transforms column 2 r + kp of the
+// set, all quarters of it, and writes the two quarters of this phase into the pair's LDS region;
+// after a barrier each wavefront reads its own quarter of both columns.
 namespace k2 {
 constexpr int kStage = 16 * 1024;      // 64 rows x 256 B
 constexpr int kSteps = 4;              // K steps of 16 per stage
 constexpr int SPB = 16;                // stages per row block and stream
 constexpr int AHEAD = 3;
-constexpr uint32_t kAreaBase = 8 * kStage;  // 128 KB: prologue areas (4 x 8 KB), later the exchange buffers
-constexpr uint32_t kAreaBytes = 8 * 1024;   // per wavefront: 2 columns x 1024 values
-static_assert(kAreaBase + 4 * kAreaBytes == (uint32_t)kLdsBytes, "rings and areas fill the 160 KB");
+// 128 KB: the prologue's regions [column set][quarter of the pair][column parity][4 KB], later the
+// exchange buffers
+constexpr uint32_t kAreaBase = 8 * kStage;
+static_assert(kAreaBase + 2 * 2 * 2 * 4096 == (uint32_t)kLdsBytes, "rings and regions fill the 160 KB");
 // LDS image of a stage: [64 rows][256 B], the 16-byte chunk q of row r stored at q ^ (r & 15)
 __host__ __device__ constexpr uint32_t stage_offset(uint32_t row, uint32_t q)
 {
     return row * 256u + ((q ^ (row & 15u)) << 4);
 }
-// prologue area: [2 columns][256 chunks], chunk q of column c stored at q ^ 2c
+// a quarter's two columns: [2 columns][256 chunks], chunk q of column c stored at q ^ 2c
 __host__ __device__ constexpr uint32_t area_offset(uint32_t c, uint32_t q) { return c * 4096u + ((q ^ (2u * c)) << 4); }
+// the same for q = 4 s + hi, hi < 4, as a base and a multiple of s: the swizzle leaves the bits of s alone
+__host__ __device__ constexpr uint32_t area_read_base(uint32_t c, uint32_t hi) { return c * 4096u + ((hi ^ (2u * c)) << 4); }
 constexpr bool patterns_conflict_free()
 {
+    for (uint32_t c = 0; c < 2; ++c)
+        for (uint32_t hi = 0; hi < 4; ++hi)
+            for (uint32_t s = 0; s < 64; ++s)
+                if (area_read_base(c, hi) + 64u * s != area_offset(c, 4u * s + hi)) return false;
     for (uint32_t mb = 0; mb < 4; ++mb)
         for (uint32_t ks = 0; ks < 4; ++ks)
             if (!lds::conflict_free_b128(
@@ -428,15 +444,18 @@ constexpr bool patterns_conflict_free()
                 return false;
     return true;
 }
-static_assert(patterns_conflict_free(), "an LDS access pattern of the K = 2048 fp32 kernel would serialise");
+static_assert(patterns_conflict_free(), "an LDS access pattern of the split-K fp32 kernel would serialise");
 }  // namespace k2
 
+template <int K>
 __global__ void __launch_bounds__(kThreads)
-fused_ht_gemm_xreg_f32_k2048_kernel(const float* __restrict__ W, const float* __restrict__ Xt,
-                                    float* __restrict__ C, uint32_t M, uint32_t N, uint32_t m_per_block,
-                                    uint32_t msplit, uint32_t mpx, uint32_t cgx, uint32_t nrect, float fscale)
+fused_ht_gemm_xreg_f32_ksplit_kernel(const float* __restrict__ W, const float* __restrict__ Xt,
+                                     float* __restrict__ C, uint32_t M, uint32_t N, uint32_t m_per_block,
+                                     uint32_t msplit, uint32_t mpx, uint32_t cgx, uint32_t nrect, float fscale,
+                                     uint32_t ph)
 {
-    constexpr int K = 2048, KSTEPS = 64, NM = 16;
+    static_assert(K == 2048 || K == 4096, "two or four quarters of 1024");
+    constexpr int NQ = K / 1024, PHASES = NQ / 2, KSTEPS = 64, NM = 16;
     constexpr int SPB = k2::SPB, AHEAD = k2::AHEAD;
     constexpr uint32_t kCols = 32;
     constexpr uint32_t ROW_BYTES = K * 4u;
@@ -444,7 +463,7 @@ fused_ht_gemm_xreg_f32_k2048_kernel(const float* __restrict__ W, const float* __
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t cs = wave >> 1, kp = wave & 1u;  // column set, K half
+    const uint32_t cs = wave >> 1, kp = wave & 1u;  // column set, quarter of the pair
     const uint32_t lo = lane & 15u, hi = lane >> 4;
 
     uint32_t cg, ms;
@@ -470,88 +489,6 @@ fused_ht_gemm_xreg_f32_k2048_kernel(const float* __restrict__ W, const float* __
             voff[i] = min(r0 + 4u * j, M - 1u) * ROW_BYTES + sp * 4096u + ((lq ^ (4u * j + lrow)) << 4);
         }
     };
-    auto w_issue = [&](uint32_t kq, int i) __attribute__((always_inline)) {
-        const uint32_t j = i & 3, sp = i >> 2;
-        global_to_lds16(voff[i], Wb + kq * 256u,
-                        lds_base + (sp * 4u + (kq & 3u)) * k2::kStage + (16u * wave + 4u * j) * 256u);
-    };
-    set_voff(0);
-
-    // ---- prologue: half kp of the transformed column n0 + 16 cs + lo, two columns per round through
-    // the wavefront's 8 KB area (both wavefronts of a pair transform the same columns)
-    float yf[KSTEPS][4];
-    {
-        unsigned char* area = lds + k2::kAreaBase + wave * k2::kAreaBytes;
-        TileOperands<BF16> ops;
-        make_tile_operands<BF16, 4>(9, ops);
-        const float sg = kp ? -1.0f : 1.0f;
-        float in[2][4][8];  // [buffer][tile][element]: tiles 0, 1 = x[0, 1024), tiles 2, 3 = x[1024, 2048)
-        auto load_col = [&](int buf, int ci) {
-            const uint32_t col = min(n0 + 16u * cs + (uint32_t)ci, N - 1u);
-#pragma unroll
-            for (int tile = 0; tile < 4; ++tile)
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    const f32x4 q = *reinterpret_cast<const f32x4*>(
-                        Xt + ((uint64_t)col * K + 512u * tile + 256u * t + 4u * lane));
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) in[buf][tile][4 * t + r] = q[r];
-                }
-        };
-        load_col(0, 0);
-#pragma unroll
-        for (int p8 = 0; p8 < 8; ++p8) {
-#pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                const int ci = 2 * p8 + c, buf = ci & 1;
-                if (ci + 1 < 16) load_col(buf ^ 1, ci + 1);
-                f32x4 a0[2], a1[2], b0[2], b1[2];
-                tile_transform_f32(in[buf][0], ops, a0);
-                tile_transform_f32(in[buf][1], ops, a1);
-                tile_transform_f32(in[buf][2], ops, b0);
-                tile_transform_f32(in[buf][3], ops, b1);
-                if (p8 >= 4) {  // the first AHEAD stage times of W, behind the last rounds of X
-#pragma unroll
-                    for (int u = 0; u < AHEAD; ++u) {
-                        const int pc = AHEAD * (ci - 8) + u;
-                        w_issue(pc >> 3, pc & 7);
-                    }
-                }
-                // element 512 h + 256 t + 4 lane + r of the half = chunk 128 h + 64 t + lane
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    const f32x4 ya0 = a0[t] + a1[t], ya1 = a0[t] - a1[t];
-                    const f32x4 yb0 = b0[t] + b1[t], yb1 = b0[t] - b1[t];
-                    *reinterpret_cast<f32x4*>(area + k2::area_offset(c, 64u * t + lane)) = (ya0 + yb0 * sg) * fscale;
-                    *reinterpret_cast<f32x4*>(area + k2::area_offset(c, 128u + 64u * t + lane)) =
-                        (ya1 + yb1 * sg) * fscale;
-                }
-            }
-            if ((int)(lo >> 1) == p8) {
-#pragma unroll
-                for (int s = 0; s < KSTEPS; ++s) {
-                    const f32x4 q = *reinterpret_cast<const f32x4*>(area + k2::area_offset(lo & 1u, 4u * s + hi));
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) yf[s][e] = q[e];
-                }
-            }
-        }
-    }
-
-    wait_vm(8 * (AHEAD - 1));
-    wait_lds();
-    __builtin_amdgcn_s_barrier();
-
-    const unsigned char* ring = lds + kp * 4u * k2::kStage;  // this wavefront's stream
-    auto frag = [&](uint32_t slot, int mb, int ks) __attribute__((always_inline)) -> f32x4 {
-        return *reinterpret_cast<const f32x4*>(ring + slot * k2::kStage + k2::stage_offset(16u * mb + lo, 4u * ks + hi));
-    };
-    f32x4 fr[4][4];  // [K step % 4][mb]
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
-        fr[0][mb] = frag(0, mb, 0);
-        fr[1][mb] = frag(0, mb, 1);
-    }
 
     // wavefront (cs, kp) finishes row fragments mb = 2 kp, 2 kp + 1: lane (hi, lo) owns rows
     // 16 mb + 4 hi + r of column n0 + 16 cs + lo
@@ -561,93 +498,223 @@ fused_ht_gemm_xreg_f32_k2048_kernel(const float* __restrict__ W, const float* __
     const bool cols_full = n0 + kCols <= N;
     unsigned char* const xb_mine = lds + k2::kAreaBase + wave * 2048u;
     const unsigned char* const xb_partner = lds + k2::kAreaBase + (wave ^ 1u) * 2048u;
+    const unsigned char* const ring = lds + kp * 4u * k2::kStage;  // this wavefront's stream
+    auto frag = [&](uint32_t slot, int mb, int ks) __attribute__((always_inline)) -> f32x4 {
+        return *reinterpret_cast<const f32x4*>(ring + slot * k2::kStage + k2::stage_offset(16u * mb + lo, 4u * ks + hi));
+    };
 
-    f32x4 acc[4][1];
-#pragma unroll 1
-    for (uint32_t rbi = 0; rbi < nrb; ++rbi) {
-        const bool last = rbi + 1u == nrb;
+    {
+        const unsigned char* Wph = Wb + (uint32_t)ph * 8192u;  // the pair's two quarters of every row
+        auto w_issue = [&](uint32_t kq, int i) __attribute__((always_inline)) {
+            const uint32_t j = i & 3, sp = i >> 2;
+            global_to_lds16(voff[i], Wph + kq * 256u,
+                            lds_base + (sp * 4u + (kq & 3u)) * k2::kStage + (16u * wave + 4u * j) * 256u);
+        };
+        set_voff(0);
+
+        // ---- prologue ----------------------------------------------------------------------------
+        float yf[KSTEPS][4];
+        {
+            unsigned char* const region = lds + k2::kAreaBase + cs * 16384u;  // [quarter of the pair][8 KB]
+            TileOperands<BF16> ops;
+            make_tile_operands<BF16, 4>(9, ops);
+            const float sigma = ph ? -1.0f : 1.0f;
+            float in[2 * NQ][8];  // tiles 2 i, 2 i + 1 = quarter i of the column
+            const float* Xp = Xt;
+            const uint32_t lane4 = 4u * lane;
+            auto load_tile = [&](int r, int i) {
+                const uint32_t c = min(n0 + 16u * cs + 2u * r + kp, N - 1u);
 #pragma unroll
-        for (int kq = 0; kq < SPB; ++kq) {
-            // (everything below folds to constants once the loops are unrolled; SPB is a multiple
-            // of 4, so stage kq of every row block lives in buffer kq % 4 of its stream)
-            const int cur_slot = kq & 3, next_slot = (kq + 1) & 3;
-            const int fill_kq = (kq + AHEAD) % SPB;
-            const bool fill_own_block = kq + AHEAD < SPB;
+                for (int t = 0; t < 2; ++t) {
+                    const f32x4 q = *reinterpret_cast<const f32x4*>(
+                        Xp + ((uint64_t)c * K + 512u * i + 256u * t + lane4));
 #pragma unroll
-            for (int ks = 0; ks < k2::kSteps; ++ks) {
-                if (kq == SPB - AHEAD && ks == 0 && !last) set_voff(rbi + 1u);
-                const int kk = kq * k2::kSteps + ks;
+                    for (int e = 0; e < 4; ++e) in[i][4 * t + e] = q[e];
+                }
+            };
 #pragma unroll
-                for (int m = 0; m < NM; ++m) {
-                    const int s = m >> 2, mb = m & 3;  // consecutive MFMAs go to different accumulators
-                    if (kk == 0 && s == 0)
-                        xmfma_f32_first(acc[mb][0], fr[ks & 3][mb][s], yf[0][s]);
-                    else
-                        xmfma_f32_next(acc[mb][0], fr[ks & 3][mb][s], yf[kk][s]);
-                    // one memory instruction in the shadow of an MFMA: fragments two K steps ahead,
-                    // the eight transfer pieces of this stage time in its first two steps
-                    if (m >= 12)
-                        fr[(ks + 2) & 3][m - 12] =
-                            ks < 2 ? frag(cur_slot, m - 12, ks + 2) : frag(next_slot, m - 12, ks - 2);
-                    else if (m >= 4 && m < 8) {
-                        if (ks < 2 && (fill_own_block || !last)) w_issue(fill_kq, 4 * ks + (m - 4));
+            for (int i = 0; i < 2 * NQ; ++i) load_tile(0, i);
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                // Y[h][g][t]: elements 512 g + 256 t + 4 lane + e of quarter h of this phase, summed
+                // over the quarters i of the input as their transforms arrive:
+                //   K = 2048: Y_0 = T_0 + T_1, Y_1 = T_0 - T_1
+                //   K = 4096: Y_{2 ph} = T_0 + T_1 + sigma (T_2 + T_3),
+                //             Y_{2 ph + 1} = T_0 - T_1 + sigma (T_2 - T_3),  sigma = (-1)^ph
+                f32x4 Y[2][2][2];
+#pragma unroll
+                for (int i = 0; i < NQ; ++i) {
+                    f32x4 a0[2], a1[2];
+                    tile_transform_f32(in[2 * i], ops, a0);
+                    tile_transform_f32(in[2 * i + 1], ops, a1);
+                    if (r + 1 < 8) {
+                        load_tile(r + 1, 2 * i);
+                        load_tile(r + 1, 2 * i + 1);
                     }
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        f32x4 u = a0[t] + a1[t], v = a0[t] - a1[t];  // the two halves of T_i
+                        if (i >= 2) {
+                            u = u * sigma;
+                            v = v * sigma;
+                        }
+                        if (i == 0) {
+                            Y[0][0][t] = u, Y[0][1][t] = v, Y[1][0][t] = u, Y[1][1][t] = v;
+                        } else {
+                            Y[0][0][t] = Y[0][0][t] + u;
+                            Y[0][1][t] = Y[0][1][t] + v;
+                            Y[1][0][t] = (i & 1) ? Y[1][0][t] - u : Y[1][0][t] + u;
+                            Y[1][1][t] = (i & 1) ? Y[1][1][t] - v : Y[1][1][t] + v;
+                        }
+                    }
+                    // (keeps the transforms of different quarters from being interleaved, which
+                    // would need more registers than there are)
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                // keep the previous step's fragment registers allocated while the matrix core may
-                // still be reading them (see the 16-bit kernel)
-                asm volatile("" ::"v"(fr[(ks + 3) & 3][0]), "v"(fr[(ks + 3) & 3][1]),
-                             "v"(fr[(ks + 3) & 3][2]), "v"(fr[(ks + 3) & 3][3]));
-                if (ks == 1) {
-                    const int later = SPB - kq - 2 < AHEAD - 1 ? SPB - kq - 2 : AHEAD - 1;
-                    const int after_last = kq == SPB - 1 ? -1 : 8 * (later > 0 ? later : 0);
-                    if (last)
-                        wait_vm(after_last);
-                    else
-                        wait_vm(8 * (AHEAD - 1));
-                    wait_lds();
-                    __builtin_amdgcn_s_barrier();
+                if (r >= 4) {  // the first AHEAD stage times of W, behind the last rounds of X
+#pragma unroll
+                    for (int u = 0; u < 2 * AHEAD; ++u) {
+                        const int pc = 2 * AHEAD * (r - 4) + u;
+                        w_issue(pc >> 3, pc & 7);
+                    }
+                }
+                // the partner has read the previous round's columns
+                wait_lds();
+                __builtin_amdgcn_s_barrier();
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        // element 512 g + 256 t + 4 lane + e of the quarter = chunk 128 g + 64 t + lane
+                        unsigned char* dst = region + h * 8192u;
+                        *reinterpret_cast<f32x4*>(dst + k2::area_offset(kp, 64u * t + lane)) = Y[h][0][t] * fscale;
+                        *reinterpret_cast<f32x4*>(dst + k2::area_offset(kp, 128u + 64u * t + lane)) =
+                            Y[h][1][t] * fscale;
+                    }
+                wait_lds();
+                __builtin_amdgcn_s_barrier();
+                if ((int)(lo >> 1) == r) {
+                    // chunk 4 s + hi of column lo % 2: one base address and constant offsets
+                    const unsigned char* src = region + kp * 8192u + k2::area_read_base(lo & 1u, hi);
+#pragma unroll
+                    for (int s = 0; s < KSTEPS; ++s) {
+                        const f32x4 q = *reinterpret_cast<const f32x4*>(src + 64u * s);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) yf[s][e] = q[e];
+                    }
                 }
             }
         }
-        // ---- the two K halves meet: hand over two fragments, finish the other two -------------------
-        drain_mfma(acc);
-        f32x4 keep[2], give[2];
-        if (kp) {
-            keep[0] = acc[2][0], keep[1] = acc[3][0], give[0] = acc[0][0], give[1] = acc[1][0];
-        } else {
-            keep[0] = acc[0][0], keep[1] = acc[1][0], give[0] = acc[2][0], give[1] = acc[3][0];
-        }
-#pragma unroll
-        for (int f = 0; f < 2; ++f) *reinterpret_cast<f32x4*>(xb_mine + f * 1024u + lane * 16u) = give[f];
+
+        wait_vm(8 * (AHEAD - 1));
         wait_lds();
         __builtin_amdgcn_s_barrier();
-        f32x4 sum[2];
+
+        f32x4 fr[4][4];  // [K step % 4][mb]
 #pragma unroll
-        for (int f = 0; f < 2; ++f) {
-            const f32x4 got = *reinterpret_cast<const f32x4*>(xb_partner + f * 1024u + lane * 16u);
-            sum[f] = kp ? got + keep[f] : keep[f] + got;  // always (k < 1024) + (k >= 1024)
+        for (int mb = 0; mb < 4; ++mb) {
+            fr[0][mb] = frag(0, mb, 0);
+            fr[1][mb] = frag(0, mb, 1);
         }
-        const uint32_t row_base = m_begin + rbi * kRows;
-        const bool full = cols_full && row_base + kRows <= m_end;
-        if (full) {
-            const uint64_t block_base = ((uint64_t)row_base + 32u * kp) * N * 4u;
+
+        f32x4 acc[4][1];
+#pragma unroll 1
+        for (uint32_t rbi = 0; rbi < nrb; ++rbi) {
+            const bool last = rbi + 1u == nrb;
+            const uint32_t row_base = m_begin + rbi * kRows;
+            const bool full = cols_full && row_base + kRows <= m_end;
+            f32x4 before[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};  // what phase 0 stored
 #pragma unroll
-            for (int f = 0; f < 2; ++f)
+            for (int kq = 0; kq < SPB; ++kq) {
+                // (everything below folds to constants once the loops are unrolled; SPB is a multiple
+                // of 4, so stage kq of every row block lives in buffer kq % 4 of its stream)
+                const int cur_slot = kq & 3, next_slot = (kq + 1) & 3;
+                const int fill_kq = (kq + AHEAD) % SPB;
+                const bool fill_own_block = kq + AHEAD < SPB;
+                if (PHASES > 1 && kq == SPB - 2 && ph > 0 && col < N) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    unsigned char* row_ptr = Cb + (block_base + (uint64_t)((16u * f + r) * N) * 4u);  // scalar
-                    const float v = sum[f][r];
-                    stream_store4(lane_off, __float_as_uint(v), row_ptr);
+                    for (int f = 0; f < 2; ++f)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const uint32_t row = row_base + 32u * kp + 16u * f + 4u * hi + r;
+                            if (row < m_end) before[f][r] = __builtin_nontemporal_load(&C[(uint64_t)row * N + col]);
+                        }
                 }
-        } else if (col < N) {
 #pragma unroll
-            for (int f = 0; f < 2; ++f)
+                for (int ks = 0; ks < k2::kSteps; ++ks) {
+                    if (kq == SPB - AHEAD && ks == 0 && !last) set_voff(rbi + 1u);
+                    const int kk = kq * k2::kSteps + ks;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const uint32_t row = row_base + 32u * kp + 16u * f + 4u * hi + r;
-                    if (row < m_end) C[(uint64_t)row * N + col] = sum[f][r];
+                    for (int m = 0; m < NM; ++m) {
+                        const int s = m >> 2, mb = m & 3;  // consecutive MFMAs go to different accumulators
+                        if (kk == 0 && s == 0)
+                            xmfma_f32_first(acc[mb][0], fr[ks & 3][mb][s], yf[0][s]);
+                        else
+                            xmfma_f32_next(acc[mb][0], fr[ks & 3][mb][s], yf[kk][s]);
+                        // one memory instruction in the shadow of an MFMA: fragments two K steps
+                        // ahead, the eight transfer pieces of this stage time in its first two steps
+                        if (m >= 12)
+                            fr[(ks + 2) & 3][m - 12] =
+                                ks < 2 ? frag(cur_slot, m - 12, ks + 2) : frag(next_slot, m - 12, ks - 2);
+                        else if (m >= 4 && m < 8) {
+                            if (ks < 2 && (fill_own_block || !last)) w_issue(fill_kq, 4 * ks + (m - 4));
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    // keep the previous step's fragment registers allocated while the matrix core
+                    // may still be reading them (see the 16-bit kernel)
+                    asm volatile("" ::"v"(fr[(ks + 3) & 3][0]), "v"(fr[(ks + 3) & 3][1]),
+                                 "v"(fr[(ks + 3) & 3][2]), "v"(fr[(ks + 3) & 3][3]));
+                    if (ks == 1) {
+                        const int later = SPB - kq - 2 < AHEAD - 1 ? SPB - kq - 2 : AHEAD - 1;
+                        const int after_last = kq == SPB - 1 ? -1 : 8 * (later > 0 ? later : 0);
+                        if (last)
+                            wait_vm(after_last);
+                        else
+                            wait_vm(8 * (AHEAD - 1));
+                        wait_lds();
+                        __builtin_amdgcn_s_barrier();
+                    }
                 }
+            }
+            // ---- the pair's two quarters meet: hand over two fragments, finish the other two --------
+            drain_mfma(acc);
+            f32x4 keep[2], give[2];
+            if (kp) {
+                keep[0] = acc[2][0], keep[1] = acc[3][0], give[0] = acc[0][0], give[1] = acc[1][0];
+            } else {
+                keep[0] = acc[0][0], keep[1] = acc[1][0], give[0] = acc[2][0], give[1] = acc[3][0];
+            }
+#pragma unroll
+            for (int f = 0; f < 2; ++f) *reinterpret_cast<f32x4*>(xb_mine + f * 1024u + lane * 16u) = give[f];
+            wait_lds();
+            __builtin_amdgcn_s_barrier();
+            f32x4 sum[2];
+#pragma unroll
+            for (int f = 0; f < 2; ++f) {
+                const f32x4 got = *reinterpret_cast<const f32x4*>(xb_partner + f * 1024u + lane * 16u);
+                sum[f] = kp ? got + keep[f] : keep[f] + got;  // always (lower quarter) + (upper quarter)
+                if (PHASES > 1) sum[f] = before[f] + sum[f];
+            }
+            if (full) {
+                const uint64_t block_base = ((uint64_t)row_base + 32u * kp) * N * 4u;
+#pragma unroll
+                for (int f = 0; f < 2; ++f)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        unsigned char* row_ptr = Cb + (block_base + (uint64_t)((16u * f + r) * N) * 4u);  // scalar
+                        const float v = sum[f][r];
+                        stream_store4(lane_off, __float_as_uint(v), row_ptr);
+                    }
+            } else if (col < N) {
+#pragma unroll
+                for (int f = 0; f < 2; ++f)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const uint32_t row = row_base + 32u * kp + 16u * f + 4u * hi + r;
+                        if (row < m_end) C[(uint64_t)row * N + col] = sum[f][r];
+                    }
+            }
         }
     }
 }
@@ -662,7 +729,7 @@ int launch_xreg_f32(const float* W, const float* Xt, float* C, uint32_t M, uint3
     constexpr uint32_t log2k = K == 256 ? 8 : K == 512 ? 9 : 10;
     const int shift = tile_stage_shift<4>(log2k, false);
     const float fscale = (float)((double)scale * (double)(1u << shift));
-    const Plan p = plan(M, N, (uint32_t)GeomF32<K>::COLS, 8u);
+    const Plan p = plan(M, N, (uint32_t)GeomF32<K>::COLS, 8u, 9u, 8u);
     auto kern = fused_ht_gemm_xreg_f32_kernel<K>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             kLdsBytes) != hipSuccess)
@@ -671,10 +738,25 @@ int launch_xreg_f32(const float* W, const float* Xt, float* C, uint32_t M, uint3
                        p.msplit, p.mpx, p.cgx, p.nrect, fscale);
     return launch_status();
 }
+template <int K>
+int launch_ksplit_f32(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, float scale, hipStream_t s)
+{
+    using namespace xreg;
+    const float fscale = (float)((double)scale * (double)(1u << tile_stage_shift<4>(9, false)));
+    const Plan p = plan(M, N, 32u, 8u, K == 4096 ? 18u : 9u, 8u);
+    auto kern = fused_ht_gemm_xreg_f32_ksplit_kernel<K>;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kLdsBytes) != hipSuccess)
+        return MI_ERR_LAUNCH;
+    for (uint32_t ph = 0; ph < (uint32_t)K / 2048u; ++ph)
+        hipLaunchKernelGGL(kern, dim3(p.grid), dim3(kThreads), kLdsBytes, s, W, Xt, C, M, N, p.m_per_block,
+                           p.msplit, p.mpx, p.cgx, p.nrect, fscale, ph);
+    return launch_status();
+}
 }  // namespace
 
-// Called by the fp32 dispatcher of mi_fused_ht_gemm for K = 256, 512, 1024, 2048 (arguments
-// already validated).
+// Called by the fp32 dispatcher of mi_fused_ht_gemm for K = 256 ... 4096 (arguments already
+// validated).
 int fused_gemm_f32_xreg(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, uint32_t K,
                         float scale, hipStream_t s)
 {
@@ -684,18 +766,8 @@ int fused_gemm_f32_xreg(const float* W, const float* Xt, float* C, uint32_t M, u
         case 256: return launch_xreg_f32<256>(W, Xt, C, M, N, scale, s);
         case 512: return launch_xreg_f32<512>(W, Xt, C, M, N, scale, s);
         case 1024: return launch_xreg_f32<1024>(W, Xt, C, M, N, scale, s);
-        case 2048: {
-            using namespace xreg;
-            const float fscale = (float)((double)scale * (double)(1u << tile_stage_shift<4>(9, false)));
-            const Plan p = plan(M, N, 32u, 8u);
-            auto kern = fused_ht_gemm_xreg_f32_k2048_kernel;
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess)
-                return MI_ERR_LAUNCH;
-            hipLaunchKernelGGL(kern, dim3(p.grid), dim3(kThreads), kLdsBytes, s, W, Xt, C, M, N, p.m_per_block,
-                               p.msplit, p.mpx, p.cgx, p.nrect, fscale);
-            return launch_status();
-        }
+        case 2048: return launch_ksplit_f32<2048>(W, Xt, C, M, N, scale, s);
+        case 4096: return launch_ksplit_f32<4096>(W, Xt, C, M, N, scale, s);
         default: return MI_ERR_SIZE;
     }
 }

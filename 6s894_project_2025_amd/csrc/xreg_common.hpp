@@ -159,16 +159,18 @@ __host__ __device__ inline bool tile_of_workgroup(uint32_t id, uint32_t msplit, 
 
 // How the (column group, M slice) grid is cut.  One workgroup fills a compute unit (all of its
 // registers and LDS), so the launch runs in rounds of 256 workgroups; a workgroup costs one prologue
-// (measured ~6.5 us) plus ~2.9 us per 64-row block (the same for both K: a row block is 64 rows x
-// 32768 / K columns x K).  The number of M slices is the one that
-// minimises rounds x (prologue + row blocks per slice) in those units (9 : 4): enough slices to
-// fill the chip, no more than that (every slice repeats the transform of its columns), and no
-// nearly empty last round.
+// plus a fixed time per 64-row block (16-bit kernel: measured ~6.5 us and ~2.9 us, the same for
+// every K: a row block is 64 rows x 131072 / K columns x K; fp32 kernels: ~15 us, twice that at
+// K = 4096, and 13.7 us).  The number of M slices is the one that minimises
+// rounds x (prologue + row blocks per slice) in those units (`pro_cost` : `block_cost`, 9 : 4 for
+// the 16-bit kernel): enough slices to fill the chip, no more than that (every slice repeats the
+// transform of its columns), and no nearly empty last round.
 struct Plan {
     uint32_t ngroups, msplit, m_per_block;
     uint32_t mpx, cgx, nrect, grid;  // XCD rectangles
 };
-inline Plan plan(uint32_t M, uint32_t N, uint32_t cols, uint32_t mpx_max)
+inline Plan plan(uint32_t M, uint32_t N, uint32_t cols, uint32_t mpx_max, uint32_t pro_cost = 9u,
+                 uint32_t block_cost = 4u)
 {
     Plan p{};
     p.ngroups = (N + cols - 1u) / cols;
@@ -179,7 +181,7 @@ inline Plan plan(uint32_t M, uint32_t N, uint32_t cols, uint32_t mpx_max)
         const uint32_t rb = (row_blocks + sp - 1u) / sp;
         const uint32_t slices = (row_blocks + rb - 1u) / rb;  // what sp really yields
         const uint64_t rounds = ((uint64_t)p.ngroups * slices + 255u) / 256u;
-        const uint64_t cost = rounds * (9u + 4u * (uint64_t)rb);
+        const uint64_t cost = rounds * (pro_cost + block_cost * (uint64_t)rb);
         if (cost < best) {
             best = cost;
             best_s = slices;

@@ -159,3 +159,33 @@ def test_fused_gemm_tiling_avoids_a_nearly_empty_last_round(libmod):
     # other K: rejected before anything else
     import ctypes
     assert lib.mi_debug_fused_gemm_tiling(64, 64, 4096, (ctypes.c_uint32 * 8)(), None, 0) != 0
+
+
+def test_build_rejects_accumulation_register_writes_inside_an_mfma_loop():
+    """The register-resident kernels name their B operand in the accumulation-register file from
+    inline assembly; the build reads the generated ISA and fails if the compiler writes such a
+    register after a kernel's first MFMA of that kind (a copy the matrix core may still be reading)."""
+    import importlib
+    build = importlib.import_module("6s894_project_2025_amd.build")
+    good = """
+_Zkernel_a: ; @_Zkernel_a
+	v_accvgpr_write_b32 a0, v1
+	;;#ASMSTART
+	v_mfma_f32_16x16x4_f32 v[28:31], v32, a252, 0
+	;;#ASMEND
+	v_add_u32_e32 v1, v2, v3
+	s_endpgm
+.Lfunc_end0:
+_Zkernel_b: ; @_Zkernel_b
+	v_accvgpr_write_b32 a5, v1
+	v_mfma_f32_16x16x32_bf16 v[0:3], v[8:11], a[4:7], v[0:3]
+	s_endpgm
+_Zplain: ; @_Zplain
+	v_accvgpr_write_b32 a5, v1
+	s_endpgm
+"""
+    assert build.check_register_resident_isa(good, "good") == 2
+    bad = good.replace("v_add_u32_e32 v1, v2, v3", "v_accvgpr_write_b32 a63, v229")
+    with pytest.raises(RuntimeError, match="_Zkernel_a writes an accumulation register"):
+        build.check_register_resident_isa(bad, "bad")
+    assert set(build.ISA_CHECKED) <= {os.path.basename(s) for s in build.sources()}

@@ -174,11 +174,12 @@ def test_gemm_k1024_launch_plans(pkg, oracle, M, N, K):
 
 
 # fp32 at K = 256, 512, 1024 runs the register-resident fp32 kernel: groups of 65536 / K columns,
-# 64-row blocks, one store of 1024 / K adjacent columns per lane and row; K = 2048 its variant
-# with the K range split over pairs of wavefronts (groups of 32 columns).  Shapes around every tile
+# 64-row blocks, one store of 1024 / K adjacent columns per lane and row; K = 2048 and 4096 its
+# variant with the K range split over pairs of wavefronts (groups of 32 columns; K = 4096 in two
+# phases, the second adding to what the first stored).  Shapes around every tile
 # boundary (edge store path, N that rules out vector stores, one row block, odd and even numbers of
 # row blocks), several scales, against the fp64 oracle at 1e-5.
-@pytest.mark.parametrize("K", [1024, 512, 256, 2048])
+@pytest.mark.parametrize("K", [1024, 512, 256, 2048, 4096])
 @pytest.mark.parametrize("M,N", [(1, 1), (31, 33), (63, 63), (64, 64), (65, 65), (128, 64), (129, 127), (192, 130),
                                  (128, 256), (320, 258), (577, 333), (130, 1000), (2048, 70), (700, 1023)])
 def test_gemm_f32_xreg_tile_boundaries(pkg, oracle, M, N, K):
@@ -194,10 +195,10 @@ def test_gemm_f32_xreg_tile_boundaries(pkg, oracle, M, N, K):
         assert err <= 1e-5, (M, N, scale, err)
 
 
-# fp32, K = 256 ... 2048, launch plans other than the benchmark's (ragged slices, more than one
+# fp32, K = 256 ... 4096, launch plans other than the benchmark's (ragged slices, more than one
 # round of workgroups, rectangles that leave workgroup ids without work): every element against the
 # product of W with the library's own fp32 transform, accumulated in fp64 on the device.
-@pytest.mark.parametrize("K", [1024, 512, 256, 2048])
+@pytest.mark.parametrize("K", [1024, 512, 256, 2048, 4096])
 @pytest.mark.parametrize("M,N", [(4096, 4096), (5000, 3000), (2048, 8192), (12288, 1536), (1000, 9000)])
 def test_gemm_f32_xreg_launch_plans(pkg, oracle, M, N, K):
     g = torch.Generator(device="cuda").manual_seed(M + N)
