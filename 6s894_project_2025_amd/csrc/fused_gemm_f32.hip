@@ -1,4 +1,6 @@
-// fp32 variant of the fused Hadamard -> GEMM (see fused_gemm.hip for the structure).
+// fp32 variant of the fused Hadamard -> GEMM for short transforms, K = 32, 64, 128 (see
+// fused_gemm.hip for the structure; K >= 256 runs the register-resident kernels of
+// fused_gemm_xreg_f32.hip).
 //
 // The transformed tile Y[BN][K] is kept in LDS as fp32; the prologue runs the fp32 transform on
 // the bf16 matrix cores with exact three-piece operands (tile_transform_f32), and the
@@ -11,7 +13,7 @@
 
 namespace mi {
 
-// K = 1024 with the transformed operand in registers: fused_gemm_xreg_f32.hip
+// K = 256 ... 4096 with the transformed operand in registers: fused_gemm_xreg_f32.hip
 int fused_gemm_f32_xreg(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, uint32_t K,
                         float scale, hipStream_t s);
 
@@ -28,18 +30,12 @@ __device__ __forceinline__ uint32_t y_off(uint32_t n, uint32_t q, uint32_t col_b
     return (n * (col_bytes >> 4) + (q ^ ((n >> LOG_NB) & swz_mask))) << 4;
 }
 
-// HALVES = 2 (K = 4096, whose fp32 tile does not fit in LDS): H_K = [[H, H], [H, -H]] with
-// H = H_{K/2}, so the kernel runs twice over half the K range, first with
-// Y = H (X_lo + X_hi) against W[:, :K/2], then with Y = H (X_lo - X_hi) against W[:, K/2:], the
-// accumulators staying in registers in between.  Each wavefront then owns exactly one 64-row
-// block (the launcher gives such workgroups 512 rows).
-template <int BN, int XB, int HALVES>
+template <int BN>
 __global__ void __launch_bounds__(kThreads)
 fused_ht_gemm_f32_kernel(const float* __restrict__ W, const float* __restrict__ Xt,
-                         float* __restrict__ C, uint32_t M, uint32_t N, uint32_t K_full,
-                         uint32_t logK_full, uint32_t m_per_block, float fscale)
+                         float* __restrict__ C, uint32_t M, uint32_t N, uint32_t K, uint32_t logK,
+                         uint32_t m_per_block, float fscale)
 {
-    const uint32_t K = K_full / HALVES, logK = logK_full - (HALVES == 2 ? 1u : 0u);
     constexpr int NB = BN / 16;
     constexpr int LOG_NB = NB == 4 ? 2 : (NB == 2 ? 1 : 0);
     extern __shared__ __attribute__((aligned(16))) unsigned char ylds[];
@@ -62,57 +58,42 @@ fused_ht_gemm_f32_kernel(const float* __restrict__ W, const float* __restrict__ 
     const uint32_t ksteps = K >> 4;
     f32x4 acc[NB][4];
 
-#pragma unroll 1
-    for (int half = 0; half < HALVES; ++half) {
-    if (half) __syncthreads();  // every wavefront is done with the first half's tile
     {
+        // a 512-element tile holds 512 / K whole columns (the operands leave the tile's upper index
+        // bits alone)
         TileOperands<BF16> ops;
         make_tile_operands<BF16, 4>(logK, ops);
-        constexpr int NT = 1 << XB;
         const uint32_t block_tiles = (BN * K) >> 9;
-        const uint64_t total = (uint64_t)N * K_full;
-        for (uint32_t t0 = wave * NT; t0 < block_tiles; t0 += kWaves * NT) {
-            float in[NT][8];
+        const uint64_t total = (uint64_t)N * K;
+        for (uint32_t t0 = wave; t0 < block_tiles; t0 += kWaves) {
+            float in[8];
 #pragma unroll
-            for (int c = 0; c < NT; ++c)
+            for (int t = 0; t < 2; ++t) {
+                // element e of the block's transformed tile: column e >> logK, k = e % K
+                const uint32_t e = t0 * 512u + 256u * t + 4u * lane;
+                const uint64_t off = (uint64_t)(n0 + (e >> logK)) * K + (e & (K - 1u));
+                f32x4 q = {0.f, 0.f, 0.f, 0.f};
+                if (off + 4u <= total) q = *reinterpret_cast<const f32x4*>(Xt + off);
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    // element e of the block's transformed tile: column e >> logK, k = e % K
-                    const uint32_t e = (t0 + c) * 512u + 256u * t + 4u * lane;
-                    const uint64_t off = (uint64_t)(n0 + (e >> logK)) * K_full + (e & (K - 1u));
-                    f32x4 q = {0.f, 0.f, 0.f, 0.f};
-                    if (off + 4u <= total) q = *reinterpret_cast<const f32x4*>(Xt + off);
-                    if (HALVES == 2 && off + K + 4u <= total) {
-                        const f32x4 u = *reinterpret_cast<const f32x4*>(Xt + off + K);
-                        q = half ? q - u : q + u;
-                    }
+                for (int r = 0; r < 4; ++r) in[4 * t + r] = q[r];
+            }
+            f32x4 y[2];
+            tile_transform_f32(in, ops, y);
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) in[c][4 * t + r] = q[r];
-                }
-            f32x4 acc[NT][2];
-#pragma unroll
-            for (int c = 0; c < NT; ++c) tile_transform_f32(in[c], ops, acc[c]);
-            cross_tile_butterflies<NT, XB>(acc);
-#pragma unroll
-            for (int c = 0; c < NT; ++c)
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    const uint32_t e = (t0 + c) * 512u + 256u * t + 4u * lane;
-                    const uint32_t n = e >> logK, q = (e & (K - 1u)) >> 2;
-                    *reinterpret_cast<f32x4*>(ylds + y_off<LOG_NB>(n, q, col_bytes, swz_mask)) =
-                        acc[c][t] * fscale;
-                }
+            for (int t = 0; t < 2; ++t) {
+                const uint32_t e = t0 * 512u + 256u * t + 4u * lane;
+                const uint32_t n = e >> logK, q = (e & (K - 1u)) >> 2;
+                *reinterpret_cast<f32x4*>(ylds + y_off<LOG_NB>(n, q, col_bytes, swz_mask)) = y[t] * fscale;
+            }
         }
     }
     __syncthreads();
 
     for (uint32_t mb = m_begin + wave * 64u; mb < m_end; mb += kWaves * 64u) {
-        if (half == 0) {
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
+        for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-                for (int mi = 0; mi < 4; ++mi) acc[nb][mi] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
+            for (int mi = 0; mi < 4; ++mi) acc[nb][mi] = f32x4{0.f, 0.f, 0.f, 0.f};
         // W goes global -> registers with four adjacent lanes on the 64 contiguous bytes a row
         // contributes to a K step (the pattern the L1 coalesces; one lane per row, which is what
         // the MFMA operand wants, runs at a third of the rate), then through a wavefront-private
@@ -123,7 +104,7 @@ fused_ht_gemm_f32_kernel(const float* __restrict__ W, const float* __restrict__ 
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
             const uint32_t m = min(mb + 16u * mi + (lane >> 2), M - 1u);
-            wsrc[mi] = W + (uint64_t)m * K_full + (uint32_t)half * K + 4u * (lane & 3u);
+            wsrc[mi] = W + (uint64_t)m * K + 4u * (lane & 3u);
         }
         // Software pipeline: while step kk is multiplied, the fragments of step kk+1 are already
         // on their way out of LDS and the W pieces of step kk+2 are in flight from memory.
@@ -169,7 +150,6 @@ fused_ht_gemm_f32_kernel(const float* __restrict__ W, const float* __restrict__ 
                                                                            acc[nb][mi], 0, 0, 0);
         }
 
-        if (half + 1 < HALVES) continue;  // the second half adds to the same accumulators
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
             const uint32_t m = mb + 16u * mi + lo;
@@ -185,15 +165,14 @@ fused_ht_gemm_f32_kernel(const float* __restrict__ W, const float* __restrict__ 
                     if ((uint32_t)(NB * r + nb) < ncols) p[NB * r + nb] = acc[nb][mi][r];
         }
     }
-    }  // half
 }
 
-template <int BN, int XB, int HALVES = 1>
+template <int BN>
 int launch(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, uint32_t K,
            float scale, hipStream_t s)
 {
     const uint32_t logK = ilog2(K);
-    const int shift = tile_stage_shift<4>(logK - (HALVES == 2 ? 1u : 0u), false);
+    const int shift = tile_stage_shift<4>(logK, false);
     const float fscale = (float)((double)scale * (double)(1u << shift));
     const uint32_t n_tiles = (N + BN - 1) / BN;
     const uint32_t row_blocks = (M + 511u) / 512u;
@@ -202,10 +181,9 @@ int launch(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, ui
     if (msplit < 1u) msplit = 1u;
     if (msplit > row_blocks) msplit = row_blocks;
     uint32_t m_per_block = ((row_blocks + msplit - 1u) / msplit) * 512u;
-    if (HALVES == 2) m_per_block = 512u;  // one row block per wavefront: accumulators stay put
     msplit = (M + m_per_block - 1u) / m_per_block;
-    const size_t lds = (size_t)BN * (K / HALVES) * 4u + (size_t)kWaves * kStageBytes;
-    auto kern = fused_ht_gemm_f32_kernel<BN, XB, HALVES>;
+    const size_t lds = (size_t)BN * K * 4u + (size_t)kWaves * kStageBytes;
+    auto kern = fused_ht_gemm_f32_kernel<BN>;
     if (lds > 64u * 1024u) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -224,7 +202,7 @@ int fused_gemm_f32(const float* W, const float* Xt, float* C, uint32_t M, uint32
     switch (K) {
         case 32:
         case 64:
-        case 128: return launch<32, 0>(W, Xt, C, M, N, K, scale, s);
+        case 128: return launch<32>(W, Xt, C, M, N, K, scale, s);
         case 256:
         case 512:
         case 1024:
