@@ -158,45 +158,50 @@ fused_ht_gemm_xreg_f32_kernel(const float* __restrict__ W, const float* __restri
         };
 #pragma unroll
         for (int i = 0; i < 8; ++i) load_tile(0, i);
+        // Pairs of tiles, software-pipelined by hand (one wavefront per SIMD hides nothing by
+        // itself): while the MFMA chains of pair p run, the vector unit splits pair p + 1 into its
+        // bf16 pieces, and the loads of the next round's pair p are already on their way.
+        SplitTileF32 cur[2], nxt[2];
+        split_tile_f32(in[0], cur[0]);
+        split_tile_f32(in[1], cur[1]);
 #pragma unroll
         for (int p4 = 0; p4 < 4; ++p4) {
-            if constexpr (K == 1024) {
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    f32x4 a0[2], a1[2];
-                    tile_transform_f32(in[2 * c], ops, a0);
-                    tile_transform_f32(in[2 * c + 1], ops, a1);
-                    if (p4 + 1 < 4) {
-                        load_tile(p4 + 1, 2 * c);
-                        load_tile(p4 + 1, 2 * c + 1);
+            for (int p = 0; p < 4; ++p) {
+                if (p4 + 1 < 4) {  // in[2 p], in[2 p + 1] are split already: refill them for the next round
+                    load_tile(p4 + 1, 2 * p);
+                    load_tile(p4 + 1, 2 * p + 1);
+                } else {
+                    w_first(2 * p);
+                    w_first(2 * p + 1);
+                }
+                // (the loads stay here, a round ahead of their use: left alone, the scheduler
+                // sinks them to the use and the wavefront waits out every one)
+                __builtin_amdgcn_sched_barrier(0);
+                if (!(p4 == 3 && p == 3)) {
+                    split_tile_f32(in[(2 * p + 2) & 7], nxt[0]);
+                    split_tile_f32(in[(2 * p + 3) & 7], nxt[1]);
+                }
+                f32x4 a[2][2];
+                tile_pair_mfma_f32(cur, ops, a);
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    if constexpr (K == 1024) {
+                        // column p: element 512 half + 256 t + 4 lane + r = chunk 128 half + 64 t + lane
+                        put(p, 64u * t + lane, a[0][t] + a[1][t]);
+                        put(p, 128u + 64u * t + lane, a[0][t] - a[1][t]);
+                    } else if constexpr (K == 512) {
+                        // columns 2 p, 2 p + 1: element 256 t + 4 lane + r
+                        put(2 * p, 64u * t + lane, a[0][t]);
+                        put(2 * p + 1, 64u * t + lane, a[1][t]);
                     } else {
-                        w_first(2 * c);
-                        w_first(2 * c + 1);
-                    }
-                    // element 512 half + 256 t + 4 lane + r of the column = chunk 128 half + 64 t + lane
-#pragma unroll
-                    for (int t = 0; t < 2; ++t) {
-                        put(c, 64u * t + lane, a0[t] + a1[t]);
-                        put(c, 128u + 64u * t + lane, a0[t] - a1[t]);
+                        // columns 4 p + 2 c + t: element 4 lane + r
+                        put(4 * p + t, lane, a[0][t]);
+                        put(4 * p + 2 + t, lane, a[1][t]);
                     }
                 }
-            } else {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    f32x4 a[2];
-                    tile_transform_f32(in[i], ops, a);
-                    if (p4 + 1 < 4)
-                        load_tile(p4 + 1, i);
-                    else
-                        w_first(i);
-#pragma unroll
-                    for (int t = 0; t < 2; ++t) {
-                        if constexpr (K == 512)
-                            put(i, 64u * t + lane, a[t]);  // element 256 t + 4 lane + r of column i
-                        else
-                            put(2 * i + t, lane, a[t]);    // element 4 lane + r of column 2 i + t
-                    }
-                }
+                cur[0] = nxt[0];
+                cur[1] = nxt[1];
             }
             if ((int)(lo >> 2) == p4) {
 #pragma unroll
@@ -534,6 +539,11 @@ fused_ht_gemm_xreg_f32_ksplit_kernel(const float* __restrict__ W, const float* _
             };
 #pragma unroll
             for (int i = 0; i < 2 * NQ; ++i) load_tile(0, i);
+            // Quarters (pairs of tiles) software-pipelined by hand, as in the kernel above: while
+            // the MFMA chains of one quarter run, the vector unit splits the next one.
+            SplitTileF32 cur[2], nxt[2];
+            split_tile_f32(in[0], cur[0]);
+            split_tile_f32(in[1], cur[1]);
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
                 // Y[h][g][t]: elements 512 g + 256 t + 4 lane + e of quarter h of this phase, summed
@@ -544,16 +554,22 @@ fused_ht_gemm_xreg_f32_ksplit_kernel(const float* __restrict__ W, const float* _
                 f32x4 Y[2][2][2];
 #pragma unroll
                 for (int i = 0; i < NQ; ++i) {
-                    f32x4 a0[2], a1[2];
-                    tile_transform_f32(in[2 * i], ops, a0);
-                    tile_transform_f32(in[2 * i + 1], ops, a1);
-                    if (r + 1 < 8) {
+                    if (r + 1 < 8) {  // tiles 2 i, 2 i + 1 are split already: refill them for the next round
                         load_tile(r + 1, 2 * i);
                         load_tile(r + 1, 2 * i + 1);
                     }
-#pragma unroll
+                    // (the loads stay here, a round ahead of their use: left alone, the scheduler
+                    // sinks them to the use and the wavefront waits out every one)
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (!(r == 7 && i == NQ - 1)) {
+                        split_tile_f32(in[(2 * i + 2) % (2 * NQ)], nxt[0]);
+                        split_tile_f32(in[(2 * i + 3) % (2 * NQ)], nxt[1]);
+                    }
+                    f32x4 a[2][2];
+                    tile_pair_mfma_f32(cur, ops, a);
+    #pragma unroll
                     for (int t = 0; t < 2; ++t) {
-                        f32x4 u = a0[t] + a1[t], v = a0[t] - a1[t];  // the two halves of T_i
+                        f32x4 u = a[0][t] + a[1][t], v = a[0][t] - a[1][t];  // the two halves of T_i
                         if (i >= 2) {
                             u = u * sigma;
                             v = v * sigma;
@@ -567,9 +583,8 @@ fused_ht_gemm_xreg_f32_ksplit_kernel(const float* __restrict__ W, const float* _
                             Y[1][1][t] = (i & 1) ? Y[1][1][t] - v : Y[1][1][t] + v;
                         }
                     }
-                    // (keeps the transforms of different quarters from being interleaved, which
-                    // would need more registers than there are)
-                    __builtin_amdgcn_sched_barrier(0);
+                    cur[0] = nxt[0];
+                    cur[1] = nxt[1];
                 }
                 if (r >= 4) {  // the first AHEAD stage times of W, behind the last rounds of X
 #pragma unroll

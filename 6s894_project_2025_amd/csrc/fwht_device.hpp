@@ -167,13 +167,37 @@ __device__ __forceinline__ void tile_transform(typename T16::V8 a, const TileOpe
     }
 }
 
-// Exact three-way split of fp32 into bf16 pieces (8 + 8 + 8 significand bits): x = h + m + l.
-__device__ __forceinline__ void split3(float x, __bf16& h, __bf16& m, __bf16& l)
+// Exact three-way split of fp32 values into bf16 pieces (8 + 8 + 8 significand bits), x = h + m + l,
+// for the eight elements of a tile operand.  By truncation: h = the upper 16 bits of x, m = the
+// upper 16 bits of x - h, l = x - h - m, which has at most eight significant bits left and is
+// therefore a bf16 value itself.  Every subtraction is exact; per value that is two ANDs, two
+// subtractions and one and a half byte permutes, all full-rate vector instructions (rounding
+// conversions to bf16 take three times as long).
+struct SplitTileF32 {
+    bf16x8 h, m, l;
+};
+__device__ __forceinline__ void split_tile_f32(const float (&v)[8], SplitTileF32& s)
 {
-    h = (__bf16)x;
-    const float r = x - (float)h;
-    m = (__bf16)r;
-    l = (__bf16)(r - (float)m);
+    u32x4 hp, mp, lp;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint32_t h[2], m[2], l[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const float x = v[2 * j + e];
+            h[e] = __float_as_uint(x) & 0xffff0000u;
+            const float r = x - __uint_as_float(h[e]);
+            m[e] = __float_as_uint(r) & 0xffff0000u;
+            l[e] = __float_as_uint(r - __uint_as_float(m[e]));
+        }
+        // upper halves of two values into one register, the first value in the lower half
+        hp[j] = __builtin_amdgcn_perm(h[1], h[0], 0x07060302u);
+        mp[j] = __builtin_amdgcn_perm(m[1], m[0], 0x07060302u);
+        lp[j] = __builtin_amdgcn_perm(l[1], l[0], 0x07060302u);
+    }
+    s.h = __builtin_bit_cast(bf16x8, hp);
+    s.m = __builtin_bit_cast(bf16x8, mp);
+    s.l = __builtin_bit_cast(bf16x8, lp);
 }
 
 // fp32 tile.  Stage 1 runs on the bf16 matrix cores: the three bf16 pieces of every input are
@@ -188,24 +212,17 @@ __device__ __forceinline__ void split3(float x, __bf16& h, __bf16& m, __bf16& l)
 __device__ __forceinline__ void tile_transform_f32(const float (&v)[8],
                                                    const TileOperands<BF16>& ops, f32x4 (&acc)[2])
 {
-    bf16x8 h, m, l;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        __bf16 a, b, c;
-        split3(v[j], a, b, c);
-        h[j] = a;
-        m[j] = b;
-        l[j] = c;
-    }
+    SplitTileF32 s;
+    split_tile_f32(v, s);
     float g2f[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) g2f[r] = (float)ops.g2[r];
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-        f32x4 d1 = BF16::mfma32(l, ops.g1[t], zero);
-        d1 = BF16::mfma32(m, ops.g1[t], d1);
-        d1 = BF16::mfma32(h, ops.g1[t], d1);
+        f32x4 d1 = BF16::mfma32(s.l, ops.g1[t], zero);
+        d1 = BF16::mfma32(s.m, ops.g1[t], d1);
+        d1 = BF16::mfma32(s.h, ops.g1[t], d1);
         f32x4 d2 = __builtin_amdgcn_mfma_f32_16x16x4f32(d1[0], g2f[0], zero, 0, 0, 0);
         d2 = __builtin_amdgcn_mfma_f32_16x16x4f32(d1[1], g2f[1], d2, 0, 0, 0);
         d2 = __builtin_amdgcn_mfma_f32_16x16x4f32(d1[2], g2f[2], d2, 0, 0, 0);
@@ -213,6 +230,48 @@ __device__ __forceinline__ void tile_transform_f32(const float (&v)[8],
     }
 }
 
+// The MFMA part of the same transform for a pair of tiles, for a caller that runs one wavefront
+// per SIMD and overlaps the pieces by hand: `split_tile_f32` is pure vector arithmetic (it can sit
+// in the shadow of another pair's MFMAs), `tile_pair_mfma_f32` issues the four MFMA chains of the
+// pair (2 tiles x 2 halves) round-robin, so that every MFMA depends on one issued four slots
+// earlier rather than on its predecessor.  (tile_transform_f32 called twice leaves the seven
+// MFMAs of each chain back to back, each waiting for the one before: about 1100 cycles per tile
+// on a lone wavefront.)  Results are bit-identical to tile_transform_f32.
+__device__ __forceinline__ void tile_pair_mfma_f32(const SplitTileF32 (&s)[2], const TileOperands<BF16>& ops,
+                                                   f32x4 (&acc)[2][2])
+{
+    // scheduling fence for MFMAs only: vector, scalar and memory instructions may cross it
+    constexpr int kKeepMfmaOrder = 0x3f6;
+    float g2f[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) g2f[r] = (float)ops.g2[r];
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    f32x4 d1[2][2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) d1[c][t] = BF16::mfma32(s[c].l, ops.g1[t], zero);
+    __builtin_amdgcn_sched_barrier(kKeepMfmaOrder);
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) d1[c][t] = BF16::mfma32(s[c].m, ops.g1[t], d1[c][t]);
+    __builtin_amdgcn_sched_barrier(kKeepMfmaOrder);
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) d1[c][t] = BF16::mfma32(s[c].h, ops.g1[t], d1[c][t]);
+    __builtin_amdgcn_sched_barrier(kKeepMfmaOrder);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+                acc[c][t] = __builtin_amdgcn_mfma_f32_16x16x4f32(d1[c][t][r], g2f[r], r ? acc[c][t] : zero, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(kKeepMfmaOrder);
+    }
+}
 // In-register butterflies over XB tile-index bits (element bits 9 .. 9+XB-1) of NT tiles.
 template <int NT, int XB>
 __device__ __forceinline__ void cross_tile_butterflies(f32x4 (&acc)[NT][2])

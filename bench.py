@@ -250,7 +250,24 @@ def main() -> int:
             "algorithmic_flops_per_step": flops,
             "roofline": roofline("mfma", tf, PEAK_TFLOPS["f32"], "TFLOP/s",
                                  traffic.get("fused_ht_gemm_f32"))}
+        u_ms, _ = steady_ms(lambda: torch.matmul(W, hada.hadamard_transform(Xt).t()), 10, 30.0)
+        others["fused_ht_gemm_f32"]["unfused_transform_then_library_gemm_us"] = round(u_ms * 1e3, 2)
+        others["fused_ht_gemm_f32"]["fused_over_unfused_speedup"] = round(u_ms / ms, 3)
         del W, Xt
+        # the other K of the reference's sweep at the same M = N (fp32 is the reference's precision)
+        if not only:
+            for Kx in (256, 512, 2048, 4096):
+                Wx = torch.randn(M, Kx, generator=torch.Generator().manual_seed(1)).to(dev)
+                Xx = torch.randn(N, Kx, generator=torch.Generator().manual_seed(0)).to(dev)
+                fx = 2 * M * N * Kx
+                f_ms, _ = steady_ms(lambda: hada.fused_ht_gemm(Wx, Xx), 10, 30.0)
+                u_ms, _ = steady_ms(lambda: torch.matmul(Wx, hada.hadamard_transform(Xx).t()), 10, 30.0)
+                others[f"fused_ht_gemm_f32_K{Kx}_M{M}_N{N}"] = {
+                    "us": round(f_ms * 1e3, 2), "algorithmic_flops": fx,
+                    "roofline": roofline("mfma", fx / f_ms / 1e9, PEAK_TFLOPS["f32"], "TFLOP/s", None),
+                    "unfused_transform_then_library_gemm_us": round(u_ms * 1e3, 2),
+                    "fused_over_unfused_speedup": round(u_ms / f_ms, 3)}
+                del Wx, Xx
 
     # ---- fused HT+GEMV and its unfused comparator (fwht_gemv_fusion.cu:323-363) ----------------------
     if want("gemv"):
