@@ -224,9 +224,19 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
         for (int i = 0; i < 8; ++i)
             voff[i] = min(r0 + 2u * i, M - 1u) * ROW_BYTES + ((lq ^ (2u * i + lrow)) << 4);
     };
-    auto w_issue = [&](uint32_t kq, uint32_t slot, int i) __attribute__((always_inline)) {
-        global_to_lds16(voff[i], Wb + kq * (kStageK * 2u),
-                        lds_base + slot * kStageBytes + (16u * wave + 2u * i) * 512u);
+    const uint32_t lds_wave_base = lds_base + 16u * wave * 512u;  // this wavefront's rows of a stage
+    auto w_issue = [&](int kq, int slot, int i) __attribute__((always_inline)) {
+        global_to_lds16(voff[i], Wb + kq * (kStageK * 2), lds_wave_base, slot * kStageBytes + 2 * i * 512);
+    };
+    // the same in two halves, one on either side of an MFMA of the main loop
+    auto w_target = [&](int slot, int i) __attribute__((always_inline)) {
+        lds_transfer_target(lds_wave_base, slot * kStageBytes + 2 * i * 512);
+    };
+    auto w_go = [&](bool always, uint32_t mask, int kq, int i) __attribute__((always_inline)) {
+        if (always)
+            lds_transfer_go(voff[i], Wb + kq * (kStageK * 2));
+        else
+            lds_transfer_go_if(mask, voff[i], Wb + kq * (kStageK * 2));
     };
     set_voff(0);
 
@@ -374,15 +384,30 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     wait_lds();
     __builtin_amdgcn_s_barrier();
 
-    auto frag = [&](uint32_t slot, int mb, int ks) __attribute__((always_inline)) -> V8 {
-        return *reinterpret_cast<const V8*>(lds + slot * kStageBytes +
-                                            stage_offset(16u * mb + lo, 4u * ks + hi));
+    // Fragment of row block mb, K step ks of a stage: row 16 mb + lo, chunk 4 ks + hi.  In the
+    // swizzled image that is (lane part) ^ (ks << 6) plus 8 KB per mb (frag_lane_offset), so one
+    // vector instruction per K step makes the address and the four reads differ by the constant in
+    // their offset field (which reaches 64 KB: buffers 2 and 3 have a lane part of their own).
+    // The instruction is opaque on purpose: left to itself the compiler keeps all the addresses of
+    // a stage in registers for the whole kernel, which this kernel does not have.
+    // (The dynamic LDS of these kernels starts at a multiple of 512, which the XOR relies on.)
+    const uint32_t frag_lane_lo = lds_base + frag_lane_offset(lo, hi);
+    const uint32_t frag_lane_hi = frag_lane_lo + 2u * kStageBytes;
+    auto frag_addr = [&](int slot, int ks) __attribute__((always_inline)) -> uint32_t {
+        uint32_t a;
+        asm volatile("v_xor_b32 %0, %2, %1" : "=v"(a) : "v"(slot >= 2 ? frag_lane_hi : frag_lane_lo), "i"(ks << 6));
+        return a;
+    };
+    auto frag_read = [&](V8& dst, uint32_t a, int slot, int mb) __attribute__((always_inline)) {
+        lds_read16(dst, a, (slot & 1) * kStageBytes + mb * 8192);
     };
     V8 fr[4][4];  // [K step % 4][mb]
+    {
+        const uint32_t a0 = frag_addr(0, 0), a1 = frag_addr(0, 1);
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
-        fr[0][mb] = frag(0, mb, 0);
-        fr[1][mb] = frag(0, mb, 1);
+        for (int mb = 0; mb < 4; ++mb) frag_read(fr[0][mb], a0, 0, mb);
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) frag_read(fr[1][mb], a1, 0, mb);
     }
 
     // ---- output addressing ------------------------------------------------------------------------
@@ -455,8 +480,11 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
         __attribute__((always_inline)) {
         constexpr bool prev_full = decltype(prev_tag)::value;
         constexpr int slot_base = decltype(second_tag)::value ? (SPB & 3) : 0;
-        // the last row block requests only its own remaining stages: nothing follows it
+        // the last row block requests only its own remaining stages: nothing follows it (its other
+        // transfers are masked off rather than branched around; the lane offsets of a block that
+        // does not exist are those of block 0, see row_block)
         const bool last = rbi + 1u == nrb;
+        const uint32_t next_block_mask = __builtin_amdgcn_readfirstlane(last ? 0u : ~0u);  // (a scalar register)
 #pragma unroll
         for (int kq = 0; kq < SPB; ++kq) {
             // pieces of stage g+AHEAD issued during K step ks of this stage (everything below folds to
@@ -471,28 +499,32 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
             for (int ks = 0; ks < kStepsPerStage; ++ks) {
                 // from the first stage whose transfers belong to the next row block on, the lane
                 // offsets are the next block's
-                if (kq == SPB - AHEAD && ks == 0 && !last) set_voff(rbi + 1u);
+                if (kq == SPB - AHEAD && ks == 0) set_voff(rbi + 1u);
                 const int kk = kq * kStepsPerStage + ks;
+                // This step's fragments were requested two steps ago; the four of the step between
+                // are the only younger reads.
+                wait_lds_all_but<4>();
+                // fragments two K steps ahead; the last two steps of a stage read the first two of
+                // the next stage, behind the barrier
+                const int read_slot = ks < 6 ? cur_slot : next_slot;
+                const uint32_t fa = frag_addr(read_slot, (ks + 2) & 7);
 #pragma unroll
                 for (int m = 0; m < NM; ++m) {
                     const int mb = m / NBF, nb = m % NBF;
+                    // up to two transfer pieces per K step: behind MFMAs 4 and 5 where a K step
+                    // has that many, else next to the fragment reads of MFMAs 1 and 3; the LDS
+                    // target goes into M0 in front of the MFMA, the transfer follows it
+                    const int piece = NM >= 6 ? m - 4 : (m == 1 ? 0 : (m == 3 ? 1 : -1));
+                    const int pi = piece >= 0 && piece < 2 && ks < 6 ? kPieceAt[ks] + piece : 99;
+                    const bool transfer = pi < kPieceAt[ks < 6 ? ks + 1 : 6];
+                    if (transfer) w_target(fill_slot, pi);
                     if (kk == 0)
                         XMfma<T16>::first(acc[mb][nb], fr[ks & 3][mb], yf[nb][0]);
                     else
                         XMfma<T16>::next(acc[mb][nb], fr[ks & 3][mb], yf[nb][kk]);
-                    // one memory instruction in the shadow of each MFMA
-                    if (m < 4) {
-                        // fragments two K steps ahead; the last two steps of a stage read the
-                        // first two of the next stage, behind the barrier
-                        fr[(ks + 2) & 3][m] = ks < 6 ? frag(cur_slot, m, ks + 2) : frag(next_slot, m, ks - 6);
-                    }
-                    // up to two transfer pieces: behind MFMAs 4 and 5 where a K step has that
-                    // many, else next to the fragment reads of MFMAs 1 and 3
-                    const int piece = NM >= 6 ? m - 4 : (m == 1 ? 0 : (m == 3 ? 1 : -1));
-                    if (piece >= 0 && piece < 2 && ks < 6 && (fill_own_block || !last)) {
-                        const int i = kPieceAt[ks] + piece;
-                        if (i < kPieceAt[ks + 1]) w_issue(fill_kq, fill_slot, i);
-                    }
+                    // memory instructions in the shadow of the MFMA
+                    if (m < 4) frag_read(fr[(ks + 2) & 3][m], fa, read_slot, m);
+                    if (transfer) w_go(fill_own_block, next_block_mask, fill_kq, pi);
                     // the previous block's sixteen stores, one behind each MFMA of the K steps
                     // that follow the first stage's barrier: they then have most of a stage to
                     // complete before the next barrier counts outstanding memory operations

@@ -117,8 +117,9 @@ fused_ht_gemm_xreg_f32_kernel(const float* __restrict__ W, const float* __restri
         for (int i = 0; i < 8; ++i)
             voff[i] = min(r0 + 2u * i, M - 1u) * ROW_BYTES + ((lq ^ (2u * i + lrow)) << 4);
     };
-    auto w_issue = [&](uint32_t kq, uint32_t slot, int i) __attribute__((always_inline)) {
-        global_to_lds16(voff[i], Wb + kq * 512u, lds_base + slot * kStageBytes + (16u * wave + 2u * i) * 512u);
+    const uint32_t lds_wave_base = lds_base + 16u * wave * 512u;  // this wavefront's rows of a stage
+    auto w_issue = [&](int kq, int slot, int i) __attribute__((always_inline)) {
+        global_to_lds16(voff[i], Wb + kq * 512, lds_wave_base, slot * kStageBytes + 2 * i * 512);
     };
     set_voff(0);
 
@@ -504,16 +505,16 @@ fused_ht_gemm_xreg_f32_ksplit_kernel(const float* __restrict__ W, const float* _
     unsigned char* const xb_mine = lds + k2::kAreaBase + wave * 2048u;
     const unsigned char* const xb_partner = lds + k2::kAreaBase + (wave ^ 1u) * 2048u;
     const unsigned char* const ring = lds + kp * 4u * k2::kStage;  // this wavefront's stream
+    const uint32_t lds_wave_base = lds_base + 16u * wave * 256u;     // this wavefront's rows of a stage
     auto frag = [&](uint32_t slot, int mb, int ks) __attribute__((always_inline)) -> f32x4 {
         return *reinterpret_cast<const f32x4*>(ring + slot * k2::kStage + k2::stage_offset(16u * mb + lo, 4u * ks + hi));
     };
 
     {
         const unsigned char* Wph = Wb + (uint32_t)ph * 8192u;  // the pair's two quarters of every row
-        auto w_issue = [&](uint32_t kq, int i) __attribute__((always_inline)) {
-            const uint32_t j = i & 3, sp = i >> 2;
-            global_to_lds16(voff[i], Wph + kq * 256u,
-                            lds_base + (sp * 4u + (kq & 3u)) * k2::kStage + (16u * wave + 4u * j) * 256u);
+        auto w_issue = [&](int kq, int i) __attribute__((always_inline)) {
+            const int j = i & 3, sp = i >> 2;
+            global_to_lds16(voff[i], Wph + kq * 256, lds_wave_base, (sp * 4 + (kq & 3)) * k2::kStage + 4 * j * 256);
         };
         set_voff(0);
 

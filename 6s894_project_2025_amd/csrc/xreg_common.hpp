@@ -38,8 +38,20 @@ __host__ __device__ constexpr uint32_t area4_offset(uint32_t c, uint32_t q)
 {
     return c * 4096u + ((q ^ (2u * c)) << 4);
 }
+// The lane part of a fragment address: row lo, chunk hi of a stage; the fragment of row block mb and
+// K step ks is at (frag_lane_offset ^ (ks << 6)) + 8192 mb (checked below).
+__host__ __device__ constexpr uint32_t frag_lane_offset(uint32_t lo, uint32_t hi)
+{
+    return lo * 512u + ((hi ^ lo) << 4);
+}
 constexpr bool lds_patterns_conflict_free()
 {
+    for (uint32_t lane = 0; lane < 64; ++lane)
+        for (uint32_t mb = 0; mb < 4; ++mb)
+            for (uint32_t ks = 0; ks < 8; ++ks)
+                if ((frag_lane_offset(lane & 15u, lane >> 4) ^ (ks << 6)) + 8192u * mb !=
+                    stage_offset(16u * mb + (lane & 15u), 4u * ks + (lane >> 4)))
+                    return false;
     // K = 2048: every lane writes chunk 64 t + lane of column c; in round p only the lanes with
     // lo / 4 == p read, chunk 4 s + hi of column lo % 4
     for (uint32_t c = 0; c < 4; ++c)
@@ -115,13 +127,57 @@ __device__ __forceinline__ void wait_vm(int n)
     }
 }
 
-// 16 bytes per lane from global memory straight into LDS: lane l's bytes land at lds_base + 16 l.
-// Scalar base + 32-bit lane offset form, so that no vector arithmetic is spent on addresses.
-// (M0 carries the LDS base of the transfer; nothing else in this kernel uses it.)
-__device__ __forceinline__ void global_to_lds16(uint32_t lane_off, const void* base, uint32_t lds_base)
+// A wavefront that has its SIMD to itself issues one instruction every four cycles, whatever the
+// instruction: between two 16-cycle MFMAs there is room for three others, waits and no-ops
+// included.  The statements below are therefore as few instructions as they can be, and are
+// placed by hand.
+//
+// 16 bytes per lane from global memory straight into LDS, in two statements so that an MFMA can
+// stand between them (M0 must be written one instruction before the transfer that uses it):
+// lane l's bytes come from base + lane_off and land at lds_wave_base + lds_imm + 16 l.  Scalar
+// base + 32-bit lane offset form, so that no vector arithmetic is spent on addresses; `lds_imm`
+// must fold to a constant (an immediate of the scalar add: a transfer then needs no scalar
+// register of its own).  The instruction's own offset field is left at zero: the hardware adds
+// it to the LDS address as well as to the global one.
+// (M0 carries the LDS base of the transfer; nothing else in these kernels uses it.)
+__device__ __forceinline__ void lds_transfer_target(uint32_t lds_wave_base, int lds_imm)
 {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :: "v"(lane_off), "s"(base), "s"(lds_base) : "memory");
+    asm volatile("s_add_i32 m0, %0, %1" :: "s"(lds_wave_base), "i"(lds_imm) : "memory", "scc");
+}
+__device__ __forceinline__ void lds_transfer_go(uint32_t lane_off, const void* base)
+{
+    asm volatile("global_load_lds_dwordx4 %0, %1" :: "v"(lane_off), "s"(base) : "memory");
+}
+// The same under a wavefront-uniform condition, without a branch: `mask` (all ones or zero) becomes
+// both halves of the execution mask for the one instruction.  (A branch costs the wavefront its
+// instruction prefetch.)  The caller runs with all 64 lanes active.
+__device__ __forceinline__ void lds_transfer_go_if(uint32_t mask, uint32_t lane_off, const void* base)
+{
+    mask = __builtin_amdgcn_readfirstlane(mask);  // (a scalar register whatever the caller's copy lives in)
+    asm volatile("s_mov_b32 exec_lo, %2\n\ts_mov_b32 exec_hi, %2\n\t"
+                 "global_load_lds_dwordx4 %0, %1\n\ts_mov_b64 exec, -1"
+                 :: "v"(lane_off), "s"(base), "s"(mask) : "memory");
+}
+// both statements at once, where nothing useful can stand between them
+__device__ __forceinline__ void global_to_lds16(uint32_t lane_off, const void* base, uint32_t lds_wave_base,
+                                                int lds_imm)
+{
+    asm volatile("s_add_i32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(lane_off), "s"(base), "s"(lds_wave_base), "i"(lds_imm) : "memory", "scc");
+}
+// A 16-byte LDS read as an opaque statement: address register + constant offset (below 64 KB), no
+// wait inserted by the compiler at the use: the caller waits with wait_lds_all_but.
+template <class V>
+__device__ __forceinline__ void lds_read16(V& dst, uint32_t addr, int offset)
+{
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(offset) : "memory");
+}
+// at most N LDS reads of this wavefront still outstanding (they complete in order)
+template <int N>
+__device__ __forceinline__ void wait_lds_all_but()
+{
+    static_assert(N >= 0 && N <= 15, "the counter has four bits");
+    asm volatile("s_waitcnt lgkmcnt(%0)" :: "n"(N) : "memory");
 }
 // streaming (non-temporal) stores, scalar base + 32-bit lane offset
 __device__ __forceinline__ void stream_store2(uint32_t lane_off, uint32_t v, void* base)

@@ -293,3 +293,21 @@ def test_fused_errors(pkg):
         pkg.fused_ht_gemm(z, torch.zeros(5, 24, device="cuda"))
     with pytest.raises(RuntimeError):
         pkg.fused_ht_gemm(torch.zeros(4, 64, device="cuda"), torch.zeros(5, 32, device="cuda"))
+
+
+def test_gemm_f32_k4096_does_not_depend_on_what_c_held(pkg, oracle):
+    # fp32 at K = 4096 is two kernels, the second adding to what the first stored in C: the first
+    # must overwrite whatever C held (NaN here), also in the masked edge blocks
+    import importlib
+    lib = importlib.import_module("6s894_project_2025_amd._lib")
+    K = 4096
+    for M, N in ((200, 70), (128, 64)):
+        W, Xt = oracle.inputs_gemm(M, N, K, torch.float32)
+        Wd, Xd = W.cuda(), Xt.cuda()
+        C = torch.full((M, N), float("nan"), device="cuda")
+        st = lib.load().mi_fused_ht_gemm(Wd.data_ptr(), Xd.data_ptr(), C.data_ptr(), M, N, K, lib.MI_F32,
+                                         lib.MI_F32, 1.0 / 64.0, torch.cuda.current_stream().cuda_stream)
+        assert st == 0
+        torch.cuda.synchronize()
+        want = oracle.fused_ht_gemm_f64_blas(W.double().numpy(), Xt.double().numpy(), 1.0 / 64.0)
+        assert _rel(oracle, C, want) <= 1e-5
