@@ -218,11 +218,13 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;  // LDS byte address of the array
     const uint32_t lrow = lane >> 5, lq = lane & 31u;
     uint32_t voff[8];  // byte offset of this lane's 16 bytes of piece i, K quarter 0, in W
-    auto set_voff = [&](uint32_t rbi) __attribute__((always_inline)) {
+    auto set_voff_piece = [&](uint32_t rbi, int i) __attribute__((always_inline)) {
         const uint32_t r0 = m_begin + row_block(rbi) * kRows + 16u * wave + lrow;
+        voff[i] = min(r0 + 2u * i, M - 1u) * ROW_BYTES + ((lq ^ (2u * i + lrow)) << 4);
+    };
+    auto set_voff = [&](uint32_t rbi) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-            voff[i] = min(r0 + 2u * i, M - 1u) * ROW_BYTES + ((lq ^ (2u * i + lrow)) << 4);
+        for (int i = 0; i < 8; ++i) set_voff_piece(rbi, i);
     };
     const uint32_t lds_wave_base = lds_base + 16u * wave * 512u;  // this wavefront's rows of a stage
     auto w_issue = [&](int kq, int slot, int i) __attribute__((always_inline)) {
@@ -497,9 +499,6 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
             const bool fill_own_block = kq + AHEAD < SPB;
 #pragma unroll
             for (int ks = 0; ks < kStepsPerStage; ++ks) {
-                // from the first stage whose transfers belong to the next row block on, the lane
-                // offsets are the next block's
-                if (kq == SPB - AHEAD && ks == 0) set_voff(rbi + 1u);
                 const int kk = kq * kStepsPerStage + ks;
                 // This step's fragments were requested two steps ago; the four of the step between
                 // are the only younger reads.
@@ -511,13 +510,19 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
 #pragma unroll
                 for (int m = 0; m < NM; ++m) {
                     const int mb = m / NBF, nb = m % NBF;
-                    // up to two transfer pieces per K step: behind MFMAs 4 and 5 where a K step
+                    // up to two transfer pieces per K step: behind MFMAs 4 and 6 where a K step
                     // has that many, else next to the fragment reads of MFMAs 1 and 3; the LDS
                     // target goes into M0 in front of the MFMA, the transfer follows it
-                    const int piece = NM >= 6 ? m - 4 : (m == 1 ? 0 : (m == 3 ? 1 : -1));
+                    const int piece = NM >= 6 ? (m == 4 ? 0 : (m == 6 ? 1 : -1)) : (m == 1 ? 0 : (m == 3 ? 1 : -1));
                     const int pi = piece >= 0 && piece < 2 && ks < 6 ? kPieceAt[ks] + piece : 99;
                     const bool transfer = pi < kPieceAt[ks < 6 ? ks + 1 : 6];
-                    if (transfer) w_target(fill_slot, pi);
+                    if (transfer) {
+                        // from the first stage whose transfers belong to the next row block on, the
+                        // lane offsets are the next block's: each is replaced right before its first
+                        // such use (three vector instructions in the shadow of the MFMA before)
+                        if (kq == SPB - AHEAD) set_voff_piece(rbi + 1u, pi);
+                        w_target(fill_slot, pi);
+                    }
                     if (kk == 0)
                         XMfma<T16>::first(acc[mb][nb], fr[ks & 3][mb], yf[nb][0]);
                     else
@@ -525,11 +530,11 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
                     // memory instructions in the shadow of the MFMA
                     if (m < 4) frag_read(fr[(ks + 2) & 3][m], fa, read_slot, m);
                     if (transfer) w_go(fill_own_block, next_block_mask, fill_kq, pi);
-                    // the previous block's sixteen stores, one behind each MFMA of the K steps
-                    // that follow the first stage's barrier: they then have most of a stage to
-                    // complete before the next barrier counts outstanding memory operations
-                    if (prev_full && kk >= 6 && kk < 6 + 16 / NM) {
-                        const int e = NM * (kk - 6) + m;
+                    // the previous block's sixteen stores, one per K step behind its last MFMA,
+                    // from the K step after the first stage's barrier on (a store costs the MFMA
+                    // stream about 16 cycles; two in a row cost more than twice that)
+                    if (prev_full && kk >= 6 && kk < 22 && m == NM - 1) {
+                        const int e = kk - 6;
                         store_pair(prev, prev_base, e >> 2, e & 3);
                     }
                     __builtin_amdgcn_sched_barrier(0);
@@ -575,6 +580,7 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     };
     if constexpr (NBF <= 2) {
         // Two accumulator sets take turns: a finished full block is stored during the next one.
+        static_assert(KSTEPS >= 22, "the sixteen stores take K steps 6 .. 21 of the next block");
         f32x4 accA[4][NBF], accB[4][NBF];
         bool pend = false;        // accB holds a finished full row block that is not stored yet
         uint64_t pend_base = 0;
