@@ -234,11 +234,8 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     auto w_target = [&](int slot, int i) __attribute__((always_inline)) {
         lds_transfer_target(lds_wave_base, slot * kStageBytes + 2 * i * 512);
     };
-    auto w_go = [&](bool always, uint32_t mask, int kq, int i) __attribute__((always_inline)) {
-        if (always)
-            lds_transfer_go(voff[i], Wb + kq * (kStageK * 2));
-        else
-            lds_transfer_go_if(mask, voff[i], Wb + kq * (kStageK * 2));
+    auto w_go = [&](int kq, int i) __attribute__((always_inline)) {
+        lds_transfer_go(voff[i], Wb + kq * (kStageK * 2));
     };
     set_voff(0);
 
@@ -477,16 +474,16 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     // when the tag says there is one) is stored one piece behind each MFMA of the K steps that follow
     // the first stage's barrier.  `second_tag`: the block is the second of its pair, whose stages
     // continue the ring where the first block's stopped (buffer (SPB + kq) % 4). -------------------
-    auto row_block_body = [&](auto prev_tag, auto second_tag, f32x4 (&acc)[4][NBF],
+    // `last_tag`: nothing follows the block, so it requests only its own remaining stages.  A tag
+    // rather than a run-time condition: a branch around a transfer costs the wavefront its
+    // instruction prefetch, and masking the transfer off through EXEC costs as much as the transfer
+    // (measured: 13 cycles of the MFMA stream each, 192 times per workgroup at the headline shape).
+    auto row_block_body = [&](auto prev_tag, auto second_tag, auto last_tag, f32x4 (&acc)[4][NBF],
                               const f32x4 (&prev)[4][NBF], uint64_t prev_base, uint32_t rbi)
         __attribute__((always_inline)) {
         constexpr bool prev_full = decltype(prev_tag)::value;
         constexpr int slot_base = decltype(second_tag)::value ? (SPB & 3) : 0;
-        // the last row block requests only its own remaining stages: nothing follows it (its other
-        // transfers are masked off rather than branched around; the lane offsets of a block that
-        // does not exist are those of block 0, see row_block)
-        const bool last = rbi + 1u == nrb;
-        const uint32_t next_block_mask = __builtin_amdgcn_readfirstlane(last ? 0u : ~0u);  // (a scalar register)
+        constexpr bool last = decltype(last_tag)::value;
 #pragma unroll
         for (int kq = 0; kq < SPB; ++kq) {
             // pieces of stage g+AHEAD issued during K step ks of this stage (everything below folds to
@@ -515,7 +512,7 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
                     // target goes into M0 in front of the MFMA, the transfer follows it
                     const int piece = NM >= 6 ? (m == 4 ? 0 : (m == 6 ? 1 : -1)) : (m == 1 ? 0 : (m == 3 ? 1 : -1));
                     const int pi = piece >= 0 && piece < 2 && ks < 6 ? kPieceAt[ks] + piece : 99;
-                    const bool transfer = pi < kPieceAt[ks < 6 ? ks + 1 : 6];
+                    const bool transfer = pi < kPieceAt[ks < 6 ? ks + 1 : 6] && (fill_own_block || !last);
                     if (transfer) {
                         // from the first stage whose transfers belong to the next row block on, the
                         // lane offsets are the next block's: each is replaced right before its first
@@ -529,7 +526,7 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
                         XMfma<T16>::next(acc[mb][nb], fr[ks & 3][mb], yf[nb][kk]);
                     // memory instructions in the shadow of the MFMA
                     if (m < 4) frag_read(fr[(ks + 2) & 3][m], fa, read_slot, m);
-                    if (transfer) w_go(fill_own_block, next_block_mask, fill_kq, pi);
+                    if (transfer) w_go(fill_kq, pi);
                     // the previous block's sixteen stores, one per K step behind its last MFMA,
                     // from the K step after the first stage's barrier on (a store costs the MFMA
                     // stream about 16 cycles; two in a row cost more than twice that)
@@ -554,10 +551,7 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
                     // stores can only make this wait longer, never shorter.
                     const int later = SPB - kq - 2 < AHEAD - 1 ? SPB - kq - 2 : AHEAD - 1;
                     const int after_last = kq == SPB - 1 ? -1 : 8 * (later > 0 ? later : 0);
-                    if (last)
-                        wait_vm(after_last);
-                    else
-                        wait_vm(8 * (AHEAD - 1));
+                    wait_vm(last ? after_last : 8 * (AHEAD - 1));
                     wait_lds();
                     __builtin_amdgcn_s_barrier();
                 }
@@ -586,10 +580,15 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
         uint64_t pend_base = 0;
         auto run = [&](bool prev_full, auto second_tag, f32x4 (&acc)[4][NBF], const f32x4 (&prev)[4][NBF],
                        uint64_t prev_base, uint32_t rbi) __attribute__((always_inline)) {
-            if (prev_full)
-                row_block_body(std::true_type{}, second_tag, acc, prev, prev_base, rbi);
+            const bool last = rbi + 1u == nrb;
+            if (prev_full && last)
+                row_block_body(std::true_type{}, second_tag, std::true_type{}, acc, prev, prev_base, rbi);
+            else if (prev_full)
+                row_block_body(std::true_type{}, second_tag, std::false_type{}, acc, prev, prev_base, rbi);
+            else if (last)
+                row_block_body(std::false_type{}, second_tag, std::true_type{}, acc, prev, prev_base, rbi);
             else
-                row_block_body(std::false_type{}, second_tag, acc, prev, prev_base, rbi);
+                row_block_body(std::false_type{}, second_tag, std::false_type{}, acc, prev, prev_base, rbi);
         };
         auto finish = [&](f32x4 (&acc)[4][NBF], uint32_t rbi, bool& full, uint64_t& base)
             __attribute__((always_inline)) {
@@ -622,7 +621,10 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
         // per K step the sixteen stores and the drain cost a few per cent of a block.
         f32x4 acc[4][NBF];
         auto one = [&](auto second_tag, uint32_t rbi) __attribute__((always_inline)) {
-            row_block_body(std::false_type{}, second_tag, acc, acc, 0, rbi);
+            if (rbi + 1u == nrb)
+                row_block_body(std::false_type{}, second_tag, std::true_type{}, acc, acc, 0, rbi);
+            else
+                row_block_body(std::false_type{}, second_tag, std::false_type{}, acc, acc, 0, rbi);
             bool full;
             uint64_t base;
             uint32_t row_base;

@@ -148,16 +148,6 @@ __device__ __forceinline__ void lds_transfer_go(uint32_t lane_off, const void* b
 {
     asm volatile("global_load_lds_dwordx4 %0, %1" :: "v"(lane_off), "s"(base) : "memory");
 }
-// The same under a wavefront-uniform condition, without a branch: `mask` (all ones or zero) becomes
-// both halves of the execution mask for the one instruction.  (A branch costs the wavefront its
-// instruction prefetch.)  The caller runs with all 64 lanes active.
-__device__ __forceinline__ void lds_transfer_go_if(uint32_t mask, uint32_t lane_off, const void* base)
-{
-    mask = __builtin_amdgcn_readfirstlane(mask);  // (a scalar register whatever the caller's copy lives in)
-    asm volatile("s_mov_b32 exec_lo, %2\n\ts_mov_b32 exec_hi, %2\n\t"
-                 "global_load_lds_dwordx4 %0, %1\n\ts_mov_b64 exec, -1"
-                 :: "v"(lane_off), "s"(base), "s"(mask) : "memory");
-}
 // both statements at once, where nothing useful can stand between them
 __device__ __forceinline__ void global_to_lds16(uint32_t lane_off, const void* base, uint32_t lds_wave_base,
                                                 int lds_imm)
