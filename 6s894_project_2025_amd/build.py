@@ -38,6 +38,7 @@ PER_FILE_FLAGS = {
     # the prologue's MFMA results feed VALU conversions; the main loop's MFMAs are inline assembly
     "fused_gemm_xreg.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "fused_gemm_xreg_f32.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "fused_gemm_xreg_k2048.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
 }
 
 
@@ -47,7 +48,7 @@ PER_FILE_FLAGS = {
 # before each use - while the previous MFMA may still be reading that register, which silently
 # corrupts results.  The build therefore looks at the generated ISA of these files and fails when an
 # accumulation register is written anywhere after a kernel's first such MFMA.
-ISA_CHECKED = {"fused_gemm_xreg.hip", "fused_gemm_xreg_f32.hip"}
+ISA_CHECKED = {"fused_gemm_xreg.hip", "fused_gemm_xreg_f32.hip", "fused_gemm_xreg_k2048.hip"}
 _MFMA_B_IN_AGPR = re.compile(r"^\s*v_mfma_\S+\s+v\[[0-9:]+\], v\S+, a")
 _AGPR_WRITE = re.compile(r"^\s*v_accvgpr_(write|mov)")
 _LABEL = re.compile(r"^([A-Za-z_][\w$]*):")

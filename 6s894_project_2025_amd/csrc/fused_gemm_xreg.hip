@@ -1,15 +1,16 @@
 // Fused Hadamard -> GEMM with the transformed operand held in registers, gfx950, 16-bit inputs:
-//     C[M,N] = W[M,K] * (scale * H_K * X[K,N]),  X given as Xt[N,K],  K = 512, 1024 or 2048.
+//     C[M,N] = W[M,K] * (scale * H_K * X[K,N]),  X given as Xt[N,K],  K = 512 or 1024
+// (K = 2048, with the K range split over pairs of wavefronts: fused_gemm_xreg_k2048.hip).
 //
 // One workgroup = four wavefronts, one per SIMD, each with the whole 512-register budget.
-//   prologue : wavefront w transforms 32768 / K columns of X (64, 32 or 16) on the
+//   prologue : wavefront w transforms 32768 / K columns of X (64 or 32) on the
 //              matrix cores (coalesced 16-byte loads, the two-stage tile transform of
 //              fwht_device.hpp; at K = 1024 the last butterfly is folded into the second stage),
 //              passes them once through a wavefront-private LDS area to get from "a lane owns 8
 //              consecutive k of one column" to MFMA operand order "lane (hi, lo) owns 8
 //              consecutive k of column lo", and keeps all 32768 values in the 256 accumulation
-//              registers for the rest of the kernel.  The workgroup therefore owns 256, 128 or
-//              64 columns, twice what fits in LDS.
+//              registers for the rest of the kernel.  The workgroup therefore owns 256 or 128
+//              columns, twice what fits in LDS.
 //   main loop: the workgroup walks its M range in 64-row blocks.  W is the only operand that
 //              moves: global -> LDS directly (no register hop), each wavefront fetching a quarter
 //              of a 64-row x 256-K stage as whole 512-byte row segments into a ring of four
@@ -21,7 +22,7 @@
 //              nothing hides an instruction that waits, so every memory instruction is issued in
 //              the shadow of a running MFMA.
 //   epilogue : D[row 4*hi + r][column lo] of the two column fragments is packed into pairs of
-//              adjacent columns and stored straight from registers, two stores per K step of the
+//              adjacent columns and stored straight from registers, one store per K step of the
 //              *next* row block (two accumulator sets take turns).
 // Per compute unit the kernel reads 128 columns of X once and a 1/msplit share of W once; the
 // register file, not LDS, decides how many columns a compute unit can keep.
@@ -32,6 +33,7 @@
 #include <type_traits>
 
 #include "xreg_common.hpp"
+#include "xreg_mfma16.hpp"
 
 namespace mi {
 namespace xreg {
@@ -41,8 +43,9 @@ namespace xreg {
 // registers (64 fragments of 16 columns x 32 k).
 template <int K>
 struct Geom {
-    static_assert(K == 512 || K == 1024 || K == 2048,
-                  "register budget: 16 NBF columns x K = 32768 values per wavefront");
+    static_assert(K == 512 || K == 1024,
+                  "register budget: 16 NBF columns x K = 32768 values per wavefront (K = 2048: "
+                  "fused_gemm_xreg_k2048.hip)");
     static constexpr int NBF = 2048 / K;            // 16-column fragments per wavefront
     static constexpr int CPW = 16 * NBF;            // columns per wavefront
     static constexpr int COLS = 4 * CPW;            // columns per workgroup
@@ -52,116 +55,6 @@ struct Geom {
     static constexpr int NM = 4 * NBF;              // MFMAs per K step
 };
 
-
-// acc (+)= A(16 x 32) * B(32 x 16) with B read straight from the accumulation-register file, where
-// the transformed operand lives for the whole kernel, and the accumulator in ordinary registers.
-// Inline assembly because the compiler, left to itself, copies register-file-resident operands
-// into ordinary registers before every use (v_accvgpr_read, four per fragment), and those copies
-// wait for the matrix-core pipeline.  What the compiler no longer sees: the result is written when
-// the instruction retires, not when it issues; readers of `c` other than the next accumulate must
-// come at least one more MFMA (or drain_mfma()) later.
-template <class T16>
-struct XMfma;
-template <>
-struct XMfma<BF16> {
-    static __device__ __forceinline__ void first(f32x4& c, bf16x8 a, bf16x8 b)
-    {
-        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "a"(b));
-    }
-    static __device__ __forceinline__ void next(f32x4& c, bf16x8 a, bf16x8 b)
-    {
-        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
-    }
-};
-template <>
-struct XMfma<F16> {
-    static __device__ __forceinline__ void first(f32x4& c, f16x8 a, f16x8 b)
-    {
-        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "a"(b));
-    }
-    static __device__ __forceinline__ void next(f32x4& c, f16x8 a, f16x8 b)
-    {
-        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
-    }
-};
-
-// A column = two 512-element tiles.  Stage 1 as in tile_transform; stage 2 contracts the two
-// tiles' stage-1 results together (K = 32: 16 stage-2 inputs of each tile) against [G2; +G2] and
-// [G2; -G2], which yields the transform of the first and of the second half of the column (the
-// butterfly over element bit 9) without any vector arithmetic.
-template <class T16>
-struct PairOperands {
-    typename T16::V8 g1[2];
-    typename T16::V8 g2s, g2d;
-};
-
-template <class T16>
-__device__ __forceinline__ void make_pair_operands(PairOperands<T16>& po, int exp2)
-{
-    TileOperands<T16> ops;
-    make_tile_operands<T16, 2>(10, ops, exp2);
-    po.g1[0] = ops.g1[0];
-    po.g1[1] = ops.g1[1];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        po.g2s[j] = ops.g2[j];
-        po.g2s[4 + j] = ops.g2[j];
-        po.g2d[j] = ops.g2[j];
-        po.g2d[4 + j] = -ops.g2[j];
-    }
-}
-
-// lo_half / hi_half: lane l's elements 8l .. 8l+7 of H_1024 (x) restricted to k < 512 / k >= 512
-template <class T16>
-__device__ __forceinline__ void column_transform(typename T16::V8 t0, typename T16::V8 t1,
-                                                 const PairOperands<T16>& po,
-                                                 typename T16::V8& lo_half, typename T16::V8& hi_half)
-{
-    using E = typename T16::E;
-    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const f32x4 d0 = T16::mfma32(t0, po.g1[h], zero);
-        const f32x4 d1 = T16::mfma32(t1, po.g1[h], zero);
-        typename T16::V8 a2;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            a2[r] = (E)d0[r];
-            a2[4 + r] = (E)d1[r];
-        }
-        const f32x4 s = T16::mfma32(a2, po.g2s, zero);
-        const f32x4 d = T16::mfma32(a2, po.g2d, zero);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            lo_half[4 * h + r] = (E)s[r];
-            hi_half[4 * h + r] = (E)d[r];
-        }
-    }
-}
-
-// The same without the final rounding: s[h] / d[h] hold elements 4h .. 4h+3 of the lane's eight for
-// the first / second half (K = 2048 adds one more butterfly, between two such pairs, in fp32).
-template <class T16>
-__device__ __forceinline__ void column_pair_f32(typename T16::V8 t0, typename T16::V8 t1,
-                                                const PairOperands<T16>& po, f32x4 (&s)[2],
-                                                f32x4 (&d)[2])
-{
-    using E = typename T16::E;
-    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const f32x4 d0 = T16::mfma32(t0, po.g1[h], zero);
-        const f32x4 d1 = T16::mfma32(t1, po.g1[h], zero);
-        typename T16::V8 a2;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            a2[r] = (E)d0[r];
-            a2[4 + r] = (E)d1[r];
-        }
-        s[h] = T16::mfma32(a2, po.g2s, zero);
-        d[h] = T16::mfma32(a2, po.g2d, zero);
-    }
-}
 
 template <class T16, int K, bool OUT_F32>
 __global__ void __launch_bounds__(kThreads)
@@ -293,57 +186,6 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
                     yf[nb][KSTEPS / 2 + s] =
                         *reinterpret_cast<const V8*>(area + area_offset(lo, 4u * s + hi));
             }
-        } else if constexpr (K == 2048) {
-            // A column is four tiles: two pairs through the pair transform, one fp32 butterfly
-            // between them (H_2048 = [[H, H], [H, -H]] over the halves).  Sixteen columns do not
-            // fit the area at once: four rounds of four columns; in round p only the lanes whose
-            // fragment column lo belongs to the round (lo / 4 == p) read their column back.
-            PairOperands<T16> po;
-            make_pair_operands<T16>(po, exp2);
-            V8 in[4][4];
-            auto load_col = [&](int p4, int c) {
-                const uint32_t col = min(n0 + CPW * wave + (uint32_t)(4 * p4 + c), N - 1u);
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    in[c][t] = *reinterpret_cast<const V8*>(Xt + ((uint64_t)col * K + 512u * t + 8u * lane));
-            };
-#pragma unroll
-            for (int c = 0; c < 4; ++c) load_col(0, c);
-#pragma unroll
-            for (int p4 = 0; p4 < 4; ++p4) {
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    f32x4 sa[2], da[2], sb[2], db[2];
-                    column_pair_f32<T16>(in[c][0], in[c][1], po, sa, da);
-                    column_pair_f32<T16>(in[c][2], in[c][3], po, sb, db);
-                    if (p4 + 1 < 4) load_col(p4 + 1, c);
-                    if (p4 == 3) {  // the first AHEAD stages of W: 8 AHEAD pieces over four columns
-#pragma unroll
-                        for (int u = 0; u < 2 * AHEAD; ++u) {
-                            const int pc = 2 * AHEAD * c + u;
-                            w_issue(pc >> 3, pc >> 3, pc & 7);
-                        }
-                    }
-                    V8 o[4];  // k quarters: A_lo + B_lo, A_hi + B_hi, A_lo - B_lo, A_hi - B_hi
-#pragma unroll
-                    for (int h = 0; h < 2; ++h)
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            o[0][4 * h + r] = (E)(sa[h][r] + sb[h][r]);
-                            o[1][4 * h + r] = (E)(da[h][r] + db[h][r]);
-                            o[2][4 * h + r] = (E)(sa[h][r] - sb[h][r]);
-                            o[3][4 * h + r] = (E)(da[h][r] - db[h][r]);
-                        }
-#pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        *reinterpret_cast<V8*>(area + area4_offset(c, 64u * t + lane)) = o[t];
-                }
-                if ((int)(lo >> 2) == p4) {
-#pragma unroll
-                    for (int s = 0; s < KSTEPS; ++s)
-                        yf[0][s] = *reinterpret_cast<const V8*>(area + area4_offset(lo & 3u, 4u * s + hi));
-                }
-            }
         } else {  // K = 512: a column is one tile
             TileOperands<T16> ops;
             make_tile_operands<T16, 2>(9, ops, exp2);
@@ -427,13 +269,7 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
         // streaming stores: C is not read again, and keeping it out of the L2 leaves the cache to
         // the operands
         unsigned char* row_ptr = Cb + (block_base + (uint64_t)((16u * mb + r) * N) * esize);  // scalar
-        if constexpr (NBF == 1) {
-            const float v0 = acc[mb][0][r] * mult;
-            if (OUT_F32)
-                stream_store4(lane_off, __builtin_bit_cast(uint32_t, v0), row_ptr);
-            else
-                stream_store2(lane_off, (uint32_t)__builtin_bit_cast(uint16_t, (E)v0), row_ptr);
-        } else if constexpr (NBF == 2) {
+        if constexpr (NBF == 2) {
             const float v0 = acc[mb][0][r] * mult, v1 = acc[mb][1][r] * mult;
             if (OUT_F32)
                 stream_store8(lane_off, u32x2{__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1)}, row_ptr);
@@ -507,10 +343,9 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
 #pragma unroll
                 for (int m = 0; m < NM; ++m) {
                     const int mb = m / NBF, nb = m % NBF;
-                    // up to two transfer pieces per K step: behind MFMAs 4 and 6 where a K step
-                    // has that many, else next to the fragment reads of MFMAs 1 and 3; the LDS
-                    // target goes into M0 in front of the MFMA, the transfer follows it
-                    const int piece = NM >= 6 ? (m == 4 ? 0 : (m == 6 ? 1 : -1)) : (m == 1 ? 0 : (m == 3 ? 1 : -1));
+                    // up to two transfer pieces per K step, behind MFMAs 4 and 6; the LDS target
+                    // goes into M0 in front of the MFMA, the transfer follows it
+                    const int piece = m == 4 ? 0 : (m == 6 ? 1 : -1);
                     const int pi = piece >= 0 && piece < 2 && ks < 6 ? kPieceAt[ks] + piece : 99;
                     const bool transfer = pi < kPieceAt[ks < 6 ? ks + 1 : 6] && (fill_own_block || !last);
                     if (transfer) {
@@ -674,6 +509,10 @@ int launch(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, int o
 
 }  // namespace xreg
 
+// K = 2048: fused_gemm_xreg_k2048.hip
+int fused_gemm16_xreg_k2048(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, int in_dtype,
+                            int out_f32, float scale, hipStream_t s);
+
 // Called by the dispatcher of mi_fused_ht_gemm for K = 512, 1024 and 2048 (arguments already
 // validated there).
 int fused_gemm16_xreg(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
@@ -689,8 +528,7 @@ int fused_gemm16_xreg(const void* W, const void* Xt, void* C, uint32_t M, uint32
         if (in_dtype == MI_BF16) return xreg::launch<BF16, 512>(W, Xt, C, M, N, out_f32, scale, 8u, s);
         if (in_dtype == MI_F16) return xreg::launch<F16, 512>(W, Xt, C, M, N, out_f32, scale, 8u, s);
     } else if (K == 2048u) {
-        if (in_dtype == MI_BF16) return xreg::launch<BF16, 2048>(W, Xt, C, M, N, out_f32, scale, 8u, s);
-        if (in_dtype == MI_F16) return xreg::launch<F16, 2048>(W, Xt, C, M, N, out_f32, scale, 8u, s);
+        return fused_gemm16_xreg_k2048(W, Xt, C, M, N, in_dtype, out_f32, scale, s);
     } else {
         return MI_ERR_SIZE;
     }

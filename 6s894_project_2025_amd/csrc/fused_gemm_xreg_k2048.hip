@@ -1,0 +1,417 @@
+// Fused Hadamard -> GEMM with the transformed operand held in registers, gfx950, 16-bit inputs,
+// K = 2048, with the K range split over pairs of wavefronts:
+//     C[M,N] = W[M,K] * (scale * H_K * X[K,N]),  X given as Xt[N,K].
+//
+// A wavefront's 256 accumulation registers hold 32768 16-bit values.  With all of K = 2048 per
+// wavefront that is 16 columns: every W fragment read from LDS then feeds one MFMA, and the LDS
+// (16 KB of fragment reads per K step of four MFMAs) bounds the loop at half the matrix-core rate.
+// Here wavefront (cs, kp) = (wave / 2, wave % 2) holds half kp of the K range of 32 columns (the
+// geometry of the K = 1024 kernel of fused_gemm_xreg.hip: two MFMAs per fragment):
+//     H_2048 x = [Ya + Yb; Ya - Yb],  Ya, Yb = the 1024-point transforms of the halves of x.
+// W is streamed as two streams (k < 1024 and k >= 1024), each through its own ring of four 16 KB
+// stages (64 rows x 128 k; a stage is four K steps); a wavefront reads the fragments of its own
+// stream only.  At the end of a row block each wavefront of a pair hands the partner the
+// accumulators of two of the four 16-row fragments through LDS and finishes (adds, stores) the
+// other two, always as (k < 1024) + (k >= 1024).
+// The prologue is shared inside a pair: per round, each wavefront transforms two of the pair's next
+// four columns, all of K, and writes both halves into the pair's LDS region; after a barrier each
+// wavefront reads its own half of the four columns.
+//
+// Main-loop statements are the hand-placed single instructions of xreg_common.hpp (see the
+// K = 1024 kernel for the reasons).
+//
+// Behaviour replaced: fused_ht_gemm_pipelined, fused_ht/fusion_pipelined.cu:306-563.
+#include <type_traits>
+
+#include "xreg_common.hpp"
+#include "xreg_mfma16.hpp"
+
+namespace mi {
+namespace xreg {
+namespace k2h {
+
+constexpr int kStage = 16 * 1024;  // 64 rows x 256 B (128 k)
+constexpr int kSteps = 4;          // K steps of 32 per stage
+constexpr int SPB = 8;             // stages per row block and stream
+constexpr int AHEAD = 3;
+constexpr int KSTEPS = 32;         // K steps per row block and wavefront
+// behind the two rings: the prologue's regions [column set][half][4 columns][2 KB], later the
+// exchange buffers [wavefront][4 KB]
+constexpr uint32_t kRegionBase = 8 * kStage;
+static_assert(kRegionBase + 2 * 2 * 4 * 2048 == (uint32_t)kLdsBytes, "rings and regions fill the 160 KB");
+
+// LDS image of a stage: [64 rows][256 B], the 16-byte chunk q of row r stored at q ^ (r & 15)
+__host__ __device__ constexpr uint32_t stage_offset(uint32_t row, uint32_t q)
+{
+    return row * 256u + ((q ^ (row & 15u)) << 4);
+}
+// lane part of a fragment address (row lo, chunk hi): the fragment of row block mb and K step ks of
+// the stage is at (frag_lane ^ (ks << 6)) + 4096 mb
+__host__ __device__ constexpr uint32_t frag_lane(uint32_t lo, uint32_t hi) { return lo * 256u + ((hi ^ lo) << 4); }
+// a half's four columns in the prologue region: [4 columns][128 chunks], chunk q of column c stored
+// at q ^ 2 (c / 2); for q = 4 s + hi that is region_read_base(c, hi) + 64 s
+__host__ __device__ constexpr uint32_t region_offset(uint32_t c, uint32_t q)
+{
+    return c * 2048u + ((q ^ (2u * (c >> 1))) << 4);
+}
+__host__ __device__ constexpr uint32_t region_read_base(uint32_t c, uint32_t hi)
+{
+    return c * 2048u + ((hi ^ (2u * (c >> 1))) << 4);
+}
+constexpr bool patterns_ok()
+{
+    for (uint32_t lane = 0; lane < 64; ++lane)
+        for (uint32_t mb = 0; mb < 4; ++mb)
+            for (uint32_t ks = 0; ks < 4; ++ks)
+                if ((frag_lane(lane & 15u, lane >> 4) ^ (ks << 6)) + 4096u * mb !=
+                    stage_offset(16u * mb + (lane & 15u), 4u * ks + (lane >> 4)))
+                    return false;
+    for (uint32_t mb = 0; mb < 4; ++mb)
+        for (uint32_t ks = 0; ks < 4; ++ks)
+            if (!lds::conflict_free_b128(
+                    [=](uint32_t lane) { return stage_offset(16u * mb + (lane & 15u), 4u * ks + (lane >> 4)); }))
+                return false;
+    for (uint32_t c = 0; c < 4; ++c)
+        for (uint32_t hi = 0; hi < 4; ++hi)
+            for (uint32_t s = 0; s < 32; ++s)
+                if (region_read_base(c, hi) + 64u * s != region_offset(c, 4u * s + hi)) return false;
+    // every lane writes chunk 64 t + lane of a column; in round r the lanes with lo / 2 == r read
+    // chunk 4 s + hi of column 2 (lo % 2) + nb
+    for (uint32_t c = 0; c < 4; ++c)
+        for (uint32_t t = 0; t < 2; ++t)
+            if (!lds::conflict_free_b128([=](uint32_t lane) { return region_offset(c, 64u * t + lane); })) return false;
+    for (uint32_t nb = 0; nb < 2; ++nb)
+        for (uint32_t r = 0; r < 8; ++r)
+            for (uint32_t s = 0; s < 32; ++s)
+                if (!lds::conflict_free_b128_masked(
+                        [=](uint32_t lane) { return region_offset(2u * (lane & 1u) + nb, 4u * s + (lane >> 4)); },
+                        [=](uint32_t lane) { return ((lane & 15u) >> 1) == r; }))
+                    return false;
+    return true;
+}
+static_assert(patterns_ok(), "an LDS access pattern of the split-K 16-bit kernel would serialise");
+
+}  // namespace k2h
+
+template <class T16, bool OUT_F32>
+__global__ void __launch_bounds__(kThreads)
+fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typename T16::E* __restrict__ Xt,
+                                void* __restrict__ C, uint32_t M, uint32_t N, uint32_t m_per_block,
+                                uint32_t msplit, uint32_t mpx, uint32_t cgx, uint32_t nrect, int exp2,
+                                float mult)
+{
+    using E = typename T16::E;
+    using V8 = typename T16::V8;
+    typedef E V2 __attribute__((ext_vector_type(2)));
+    constexpr int K = 2048, NBF = 2, NM = 8;
+    constexpr int SPB = k2h::SPB, AHEAD = k2h::AHEAD, KSTEPS = k2h::KSTEPS;
+    constexpr uint32_t kCols = 64;
+    constexpr uint32_t ROW_BYTES = K * 2u;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t cs = wave >> 1, kp = wave & 1u;  // column set, K half
+    const uint32_t lo = lane & 15u, hi = lane >> 4;
+
+    uint32_t cg, ms;
+    if (!tile_of_workgroup(blockIdx.x, msplit, mpx, cgx, nrect, cg, ms)) return;  // uniform, before any barrier
+    const uint32_t n0 = cg * kCols;
+    const uint32_t m_begin = ms * m_per_block;
+    if (m_begin >= M || n0 >= N) return;  // workgroup-uniform, before any barrier
+    const uint32_t m_end = min(M, m_begin + m_per_block);
+    const uint32_t nrb = (m_end - m_begin + kRows - 1u) / kRows;
+    auto row_block = [&](uint32_t rbi) __attribute__((always_inline)) { return rbi < nrb ? rbi : 0u; };
+
+    // ---- W streams: per stage time a wavefront moves rows 16 w .. 16 w + 15 of both streams' stages,
+    // eight pieces of 4 rows x 256 B (piece i: stream i / 4, rows 4 (i % 4) .. + 3)
+    const unsigned char* Wb = reinterpret_cast<const unsigned char*>(W);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;
+    const uint32_t lrow = lane >> 4, lq = lane & 15u;
+    uint32_t voff[8];
+    auto set_voff_piece = [&](uint32_t rbi, int i) __attribute__((always_inline)) {
+        const uint32_t r0 = m_begin + row_block(rbi) * kRows + 16u * wave + lrow;
+        const uint32_t j = i & 3, sp = i >> 2;
+        voff[i] = min(r0 + 4u * j, M - 1u) * ROW_BYTES + sp * 2048u + ((lq ^ (4u * j + lrow)) << 4);
+    };
+    const uint32_t lds_wave_base = lds_base + 16u * wave * 256u;  // this wavefront's rows of a stage
+    auto lds_piece = [](int kq, int i) constexpr { return ((i >> 2) * 4 + (kq & 3)) * k2h::kStage + 4 * (i & 3) * 256; };
+    auto w_issue = [&](int kq, int i) __attribute__((always_inline)) {
+        global_to_lds16(voff[i], Wb + kq * 256, lds_wave_base, lds_piece(kq, i));
+    };
+#pragma unroll
+    for (int i = 0; i < 8; ++i) set_voff_piece(0, i);
+
+    // ---- prologue: column nb of lane (., lo) = column n0 + 32 cs + 2 lo + nb, its half kp -------------
+    V8 yf[NBF][KSTEPS];
+    {
+        unsigned char* const region = lds + k2h::kRegionBase + cs * 16384u;  // [half][4 columns][2 KB]
+        PairOperands<T16> po;
+        make_pair_operands<T16>(po, exp2);
+        V8 in[2][4];  // [column of this wavefront in the round][tile]
+        auto load_col = [&](int r, int j) {  // the wavefront's column j of round r: 4 r + 2 j + kp of the set
+            const uint32_t col = min(n0 + 32u * cs + (uint32_t)(4 * r + 2 * j) + kp, N - 1u);
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                in[j][t] = *reinterpret_cast<const V8*>(Xt + ((uint64_t)col * K + 512u * t + 8u * lane));
+        };
+        load_col(0, 0);
+        load_col(0, 1);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            V8 o[2][4];  // [column][k quarter]: A_lo + B_lo, A_hi + B_hi, A_lo - B_lo, A_hi - B_hi
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                f32x4 sa[2], da[2], sb[2], db[2];
+                column_pair_f32<T16>(in[j][0], in[j][1], po, sa, da);
+                column_pair_f32<T16>(in[j][2], in[j][3], po, sb, db);
+                if (r + 1 < 8) load_col(r + 1, j);
+                // (the loads stay here, a round ahead of their use)
+                __builtin_amdgcn_sched_barrier(0);
+                if (r >= 4) {  // W stages 0 .. 2 and the first half of stage 3, behind the last rounds of X
+#pragma unroll
+                    for (int u = 0; u < (j ? 3 : 4); ++u) {
+                        const int pc = 7 * (r - 4) + 4 * j + u;
+                        w_issue(pc >> 3, pc & 7);
+                    }
+                }
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        o[j][0][4 * h + e] = (E)(sa[h][e] + sb[h][e]);
+                        o[j][1][4 * h + e] = (E)(da[h][e] + db[h][e]);
+                        o[j][2][4 * h + e] = (E)(sa[h][e] - sb[h][e]);
+                        o[j][3][4 * h + e] = (E)(da[h][e] - db[h][e]);
+                    }
+            }
+            // the partner has read the previous round's columns
+            wait_lds();
+            __builtin_amdgcn_s_barrier();
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)  // quarter q = half q / 2, chunks 64 (q % 2) + lane of it
+                    *reinterpret_cast<V8*>(region + (q >> 1) * 8192u +
+                                           k2h::region_offset(2u * j + kp, 64u * (q & 1) + lane)) = o[j][q];
+            wait_lds();
+            __builtin_amdgcn_s_barrier();
+            if ((int)(lo >> 1) == r) {
+#pragma unroll
+                for (int nb = 0; nb < NBF; ++nb) {
+                    const unsigned char* src = region + kp * 8192u + k2h::region_read_base(2u * (lo & 1u) + nb, hi);
+#pragma unroll
+                    for (int s = 0; s < KSTEPS; ++s) yf[nb][s] = *reinterpret_cast<const V8*>(src + 64u * s);
+                }
+            }
+        }
+    }
+
+    wait_vm(8 * (AHEAD - 1) + 4);  // stage 0 has landed (stages 1, 2 and half of 3 are younger)
+    wait_lds();
+    __builtin_amdgcn_s_barrier();
+
+    // ---- fragments of this wavefront's stream ----------------------------------------------------
+    const uint32_t frag_lane = lds_base + kp * 4u * k2h::kStage + k2h::frag_lane(lo, hi);
+    auto frag_addr = [&](int ks) __attribute__((always_inline)) -> uint32_t {
+        uint32_t a;
+        asm volatile("v_xor_b32 %0, %2, %1" : "=v"(a) : "v"(frag_lane), "i"(ks << 6));
+        return a;
+    };
+    auto frag_read = [&](V8& dst, uint32_t a, int slot, int mb) __attribute__((always_inline)) {
+        lds_read16(dst, a, slot * k2h::kStage + mb * 4096);
+    };
+    V8 fr[4][4];  // [K step % 4][mb]
+    {
+        const uint32_t a0 = frag_addr(0), a1 = frag_addr(1);
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) frag_read(fr[0][mb], a0, 0, mb);
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) frag_read(fr[1][mb], a1, 0, mb);
+    }
+
+    // ---- output: wavefront (cs, kp) finishes row fragments mb = 2 kp, 2 kp + 1; lane (hi, lo) owns
+    // rows 16 mb + 4 hi + r of the adjacent columns n0 + 32 cs + 2 lo, + 1
+    constexpr uint32_t esize = OUT_F32 ? 4u : 2u;
+    const uint32_t col = n0 + 32u * cs + 2u * lo;
+    const uint32_t lane_off = (4u * hi * N + col) * esize;  // inside the row block, < 2^32
+    unsigned char* const Cb = static_cast<unsigned char*>(C);
+    const bool cols_full = n0 + kCols <= N && (N & 1u) == 0u;
+    unsigned char* const xb_mine = lds + k2h::kRegionBase + wave * 4096u;
+    const unsigned char* const xb_partner = lds + k2h::kRegionBase + (wave ^ 1u) * 4096u;
+
+    // Transfers: two pieces per K step (behind MFMAs 4 and 6), every K step.  The stage whose reads
+    // end with the barrier of K step 1 is refilled from K step 2 on: during K steps 2, 3 of stage kq
+    // the first four pieces of stage kq + 4 go out (into the buffer of stage kq), during K steps 0, 1
+    // of stage kq + 1 its other four.  At the barrier of stage kq the pieces of stages kq + 2 and
+    // kq + 3 are the sixteen youngest, so the wait for stage kq + 1 is the same constant everywhere.
+    f32x4 acc[4][NBF];
+    f32x4 out[2][NBF];  // the finished half of the previous row block, stored during this one
+    uint64_t out_base = 0;
+    auto store_out = [&](int f, int r) __attribute__((always_inline)) {
+        unsigned char* row_ptr = Cb + (out_base + (uint64_t)((16u * f + r) * N) * esize);  // scalar
+        const float v0 = out[f][0][r], v1 = out[f][1][r];
+        if (OUT_F32)
+            stream_store8(lane_off, u32x2{__float_as_uint(v0), __float_as_uint(v1)}, row_ptr);
+        else
+            stream_store4(lane_off, __builtin_bit_cast(uint32_t, V2{(E)v0, (E)v1}), row_ptr);
+    };
+    auto row_block_body = [&](auto last_tag, auto out_tag, uint32_t rbi) __attribute__((always_inline)) {
+        constexpr bool last = decltype(last_tag)::value;
+        constexpr bool out_full = decltype(out_tag)::value;
+#pragma unroll
+        for (int kq = 0; kq < SPB; ++kq) {
+            // (everything below folds to constants once the loops are unrolled; SPB is a multiple of
+            // 4, so stage kq of every row block lives in buffer kq % 4 of its stream)
+            const int cur_slot = kq & 3, next_slot = (kq + 1) & 3;
+#pragma unroll
+            for (int ks = 0; ks < k2h::kSteps; ++ks) {
+                const int kk = kq * k2h::kSteps + ks;
+                // this step's fragments were requested two steps ago; the four of the step between
+                // are the only younger reads
+                wait_lds_all_but<4>();
+                const int read_slot = ks < 2 ? cur_slot : next_slot;
+                const uint32_t fa = frag_addr((ks + 2) & 3);
+                const int fill_stage = ks < 2 ? kq + AHEAD : kq + AHEAD + 1;  // may lie in the next row block
+                const int fill_kq = fill_stage % SPB;
+#pragma unroll
+                for (int m = 0; m < NM; ++m) {
+                    const int mb = m >> 1, nb = m & 1;
+                    const int pi = (ks < 2 ? 4 : 0) + 2 * (ks & 1) + (m == 6 ? 1 : 0);
+                    const bool transfer = (m == 4 || m == 6) && (fill_stage < SPB || !last);
+                    if (transfer) {
+                        // the lane offsets of the next row block replace this one's right before
+                        // their first use (three vector instructions in the shadow of an MFMA)
+                        if (fill_stage == SPB) set_voff_piece(rbi + 1u, pi);
+                        lds_transfer_target(lds_wave_base, lds_piece(fill_kq, pi));
+                    }
+                    if (kk == 0)
+                        XMfma<T16>::first(acc[mb][nb], fr[ks & 3][mb], yf[nb][0]);
+                    else
+                        XMfma<T16>::next(acc[mb][nb], fr[ks & 3][mb], yf[nb][kk]);
+                    if (m < 4) frag_read(fr[(ks + 2) & 3][m], fa, read_slot, m);
+                    if (transfer) lds_transfer_go(voff[pi], Wb + fill_kq * 256);
+                    // the previous block's eight stores, one per K step from K step 2 on
+                    if (out_full && kk >= 2 && kk < 10 && m == NM - 1) store_out((kk - 2) >> 2, (kk - 2) & 3);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                // keep the previous step's fragment registers allocated while the matrix core may
+                // still be reading them (see the K = 1024 kernel)
+                asm volatile("" ::"v"(fr[(ks + 3) & 3][0]), "v"(fr[(ks + 3) & 3][1]),
+                             "v"(fr[(ks + 3) & 3][2]), "v"(fr[(ks + 3) & 3][3]));
+                if (ks == 1) {
+                    // stage kq + 1 has landed: loads complete in order, and what was requested after
+                    // its pieces are the pieces of stages kq + 2 and kq + 3 (those that exist, in the
+                    // last row block); pending stores can only make this wait longer
+                    const int younger = (kq + 2 < SPB ? 8 : 0) + (kq + 3 < SPB ? 8 : 0);
+                    wait_vm(last ? (kq + 1 < SPB ? younger : -1) : 16);
+                    wait_lds();
+                    __builtin_amdgcn_s_barrier();
+                }
+            }
+        }
+    };
+
+    bool out_pending = false;
+#pragma unroll 1
+    for (uint32_t rbi = 0; rbi < nrb; ++rbi) {
+        const bool last_block = rbi + 1u == nrb;
+        if (last_block && out_pending)
+            row_block_body(std::true_type{}, std::true_type{}, rbi);
+        else if (last_block)
+            row_block_body(std::true_type{}, std::false_type{}, rbi);
+        else if (out_pending)
+            row_block_body(std::false_type{}, std::true_type{}, rbi);
+        else
+            row_block_body(std::false_type{}, std::false_type{}, rbi);
+        // ---- the two K halves meet: hand over two row fragments, finish the other two -------------
+        drain_mfma(acc);
+        f32x4 keep[2][NBF], give[2][NBF];
+#pragma unroll
+        for (int f = 0; f < 2; ++f)
+#pragma unroll
+            for (int nb = 0; nb < NBF; ++nb) {
+                keep[f][nb] = kp ? acc[2 + f][nb] : acc[f][nb];
+                give[f][nb] = kp ? acc[f][nb] : acc[2 + f][nb];
+            }
+#pragma unroll
+        for (int f = 0; f < 2; ++f)
+#pragma unroll
+            for (int nb = 0; nb < NBF; ++nb)
+                *reinterpret_cast<f32x4*>(xb_mine + (2 * f + nb) * 1024u + lane * 16u) = give[f][nb];
+        wait_lds();
+        __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int f = 0; f < 2; ++f)
+#pragma unroll
+            for (int nb = 0; nb < NBF; ++nb) {
+                const f32x4 got = *reinterpret_cast<const f32x4*>(xb_partner + (2 * f + nb) * 1024u + lane * 16u);
+                out[f][nb] = (kp ? got + keep[f][nb] : keep[f][nb] + got) * mult;  // (k < 1024) + (k >= 1024)
+            }
+        const uint32_t row_base = m_begin + rbi * kRows;
+        const bool full = cols_full && row_base + kRows <= m_end;
+        out_base = ((uint64_t)row_base + 32u * kp) * N * esize;
+        out_pending = full && !last_block;  // stored behind the MFMAs of the next row block
+        if (full && last_block) {
+#pragma unroll
+            for (int f = 0; f < 2; ++f)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) store_out(f, r);
+        } else if (!full) {
+#pragma unroll
+            for (int f = 0; f < 2; ++f)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint32_t row = row_base + 32u * kp + 16u * f + 4u * hi + r;
+                    if (row >= m_end) continue;
+#pragma unroll
+                    for (int nb = 0; nb < NBF; ++nb) {
+                        if (col + nb >= N) continue;
+                        const float v = out[f][nb][r];
+                        const uint64_t at = (uint64_t)row * N + col + nb;
+                        if (OUT_F32)
+                            static_cast<float*>(C)[at] = v;
+                        else
+                            static_cast<E*>(C)[at] = (E)v;
+                    }
+                }
+        }
+    }
+    // Every transfer into LDS was waited for at the barrier of the stage before the one that read
+    // it, so none is in flight when the workgroup's LDS is released.
+}
+
+namespace {
+template <class T16, bool OUT_F32>
+int launch_k2048(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, float scale, hipStream_t s)
+{
+    const OutputScale os = split_output_scale((double)scale, tile_stage_shift<2>(11u, kNarrowRange<T16>));
+    const Plan p = plan(M, N, 64u, 8u);
+    auto kern = fused_ht_gemm_xreg_k2048_kernel<T16, OUT_F32>;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kLdsBytes) != hipSuccess)
+        return MI_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(p.grid), dim3(kThreads), kLdsBytes, s, static_cast<const typename T16::E*>(W),
+                       static_cast<const typename T16::E*>(Xt), C, M, N, p.m_per_block, p.msplit, p.mpx, p.cgx,
+                       p.nrect, os.exp2, os.mult);
+    return launch_status();
+}
+}  // namespace
+
+}  // namespace xreg
+
+// Called by fused_gemm16_xreg for K = 2048 (arguments already validated).
+int fused_gemm16_xreg_k2048(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, int in_dtype,
+                            int out_f32, float scale, hipStream_t s)
+{
+    using namespace xreg;
+    if (in_dtype == MI_BF16)
+        return out_f32 ? launch_k2048<BF16, true>(W, Xt, C, M, N, scale, s)
+                       : launch_k2048<BF16, false>(W, Xt, C, M, N, scale, s);
+    if (in_dtype == MI_F16)
+        return out_f32 ? launch_k2048<F16, true>(W, Xt, C, M, N, scale, s)
+                       : launch_k2048<F16, false>(W, Xt, C, M, N, scale, s);
+    return MI_ERR_DTYPE;
+}
+
+}  // namespace mi

@@ -32,12 +32,6 @@ __host__ __device__ constexpr uint32_t area_offset(uint32_t j, uint32_t q)
 {
     return j * 1024u + ((q ^ j) << 4);
 }
-// The same area at K = 2048, four columns at a time: [4 columns][256 chunks], chunk q of column c
-// stored at q ^ 2c.
-__host__ __device__ constexpr uint32_t area4_offset(uint32_t c, uint32_t q)
-{
-    return c * 4096u + ((q ^ (2u * c)) << 4);
-}
 // The lane part of a fragment address: row lo, chunk hi of a stage; the fragment of row block mb and
 // K step ks is at (frag_lane_offset ^ (ks << 6)) + 8192 mb (checked below).
 __host__ __device__ constexpr uint32_t frag_lane_offset(uint32_t lo, uint32_t hi)
@@ -52,18 +46,6 @@ constexpr bool lds_patterns_conflict_free()
                 if ((frag_lane_offset(lane & 15u, lane >> 4) ^ (ks << 6)) + 8192u * mb !=
                     stage_offset(16u * mb + (lane & 15u), 4u * ks + (lane >> 4)))
                     return false;
-    // K = 2048: every lane writes chunk 64 t + lane of column c; in round p only the lanes with
-    // lo / 4 == p read, chunk 4 s + hi of column lo % 4
-    for (uint32_t c = 0; c < 4; ++c)
-        for (uint32_t t = 0; t < 4; ++t)
-            if (!lds::conflict_free_b128([=](uint32_t lane) { return area4_offset(c, 64u * t + lane); }))
-                return false;
-    for (uint32_t p = 0; p < 4; ++p)
-        for (uint32_t s = 0; s < 64; ++s)
-            if (!lds::conflict_free_b128_masked(
-                    [=](uint32_t lane) { return area4_offset(lane & 3u, 4u * s + (lane >> 4)); },
-                    [=](uint32_t lane) { return ((lane & 15u) >> 2) == p; }))
-                return false;
     // fragment read of row block mb, K step ks: lane (hi, lo) takes row 16 mb + lo, chunk 4 ks + hi
     for (uint32_t mb = 0; mb < 4; ++mb)
         for (uint32_t ks = 0; ks < 8; ++ks)
@@ -121,8 +103,11 @@ __device__ __forceinline__ void wait_vm(int n)
 {
     switch (n) {
         case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+        case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
         case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+        case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
         case 16: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
+        case 20: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
         default: break;  // nothing to wait for
     }
 }
@@ -170,10 +155,6 @@ __device__ __forceinline__ void wait_lds_all_but()
     asm volatile("s_waitcnt lgkmcnt(%0)" :: "n"(N) : "memory");
 }
 // streaming (non-temporal) stores, scalar base + 32-bit lane offset
-__device__ __forceinline__ void stream_store2(uint32_t lane_off, uint32_t v, void* base)
-{
-    asm volatile("global_store_short %0, %1, %2 nt" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
-}
 __device__ __forceinline__ void stream_store4(uint32_t lane_off, uint32_t v, void* base)
 {
     asm volatile("global_store_dword %0, %1, %2 nt" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
