@@ -104,8 +104,9 @@ def test_gemm_against_oracle(pkg, oracle, M, N, K, dt, tol):
         assert _rel(oracle, C16, want) <= tol
 
 
-# K = 512, 1024 and 2048 run the register-resident kernel: groups of 131072 / K columns, 64-row
-# blocks, results stored while the next row block is multiplied or (K = 512) right after it.
+# K = 512, 1024 and 2048 run the register-resident kernels (K = 2048 its own, with K split over
+# wavefront pairs): groups of 131072 / K columns, 64-row blocks, results stored while the next row
+# block is multiplied or (K = 512) right after it.
 # Shapes around every tile boundary, a single row block, N not a multiple of the columns a lane
 # stores together (no vector stores), a scale that is not a power of two (separate store path),
 # both 16-bit types and both output types.
