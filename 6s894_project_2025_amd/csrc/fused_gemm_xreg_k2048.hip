@@ -128,19 +128,19 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
     const unsigned char* Wb = reinterpret_cast<const unsigned char*>(W);
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;
     const uint32_t lrow = lane >> 4, lq = lane & 15u;
-    uint32_t voff[8];
-    auto set_voff_piece = [&](uint32_t rbi, int i) __attribute__((always_inline)) {
+    uint32_t voff[4];  // lane offset of rows 4 j .. 4 j + 3 (the second stream's 2048 bytes go into the scalar base)
+    auto set_voff_piece = [&](uint32_t rbi, int j) __attribute__((always_inline)) {
         const uint32_t r0 = m_begin + row_block(rbi) * kRows + 16u * wave + lrow;
-        const uint32_t j = i & 3, sp = i >> 2;
-        voff[i] = min(r0 + 4u * j, M - 1u) * ROW_BYTES + sp * 2048u + ((lq ^ (4u * j + lrow)) << 4);
+        voff[j] = min(r0 + 4u * j, M - 1u) * ROW_BYTES + ((lq ^ (4u * j + lrow)) << 4);
     };
     const uint32_t lds_wave_base = lds_base + 16u * wave * 256u;  // this wavefront's rows of a stage
     auto lds_piece = [](int kq, int i) constexpr { return ((i >> 2) * 4 + (kq & 3)) * k2h::kStage + 4 * (i & 3) * 256; };
+    auto w_base = [&](int kq, int i) __attribute__((always_inline)) { return Wb + (kq * 256 + (i >> 2) * 2048); };
     auto w_issue = [&](int kq, int i) __attribute__((always_inline)) {
-        global_to_lds16(voff[i], Wb + kq * 256, lds_wave_base, lds_piece(kq, i));
+        global_to_lds16(voff[i & 3], w_base(kq, i), lds_wave_base, lds_piece(kq, i));
     };
 #pragma unroll
-    for (int i = 0; i < 8; ++i) set_voff_piece(0, i);
+    for (int j = 0; j < 4; ++j) set_voff_piece(0, j);
 
     // ---- prologue: column nb of lane (., lo) = column n0 + 32 cs + 2 lo + nb, its half kp -------------
     V8 yf[NBF][KSTEPS];
@@ -148,33 +148,37 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
         unsigned char* const region = lds + k2h::kRegionBase + cs * 16384u;  // [half][4 columns][2 KB]
         PairOperands<T16> po;
         make_pair_operands<T16>(po, exp2);
-        V8 in[2][4];  // [column of this wavefront in the round][tile]
+        // X tiles are requested kXAhead rounds before their use: one round of transforms is far
+        // shorter than a trip to memory
+        constexpr int kXAhead = 2;
+        V8 in[kXAhead][2][4];  // [round % kXAhead][column of this wavefront in the round][tile]
         auto load_col = [&](int r, int j) {  // the wavefront's column j of round r: 4 r + 2 j + kp of the set
             const uint32_t col = min(n0 + 32u * cs + (uint32_t)(4 * r + 2 * j) + kp, N - 1u);
 #pragma unroll
             for (int t = 0; t < 4; ++t)
-                in[j][t] = *reinterpret_cast<const V8*>(Xt + ((uint64_t)col * K + 512u * t + 8u * lane));
+                in[r % kXAhead][j][t] = *reinterpret_cast<const V8*>(Xt + ((uint64_t)col * K + 512u * t + 8u * lane));
         };
-        load_col(0, 0);
-        load_col(0, 1);
+        // W stages 0 .. 2 and the first half of stage 3 go out before any X: vector memory
+        // operations complete in order and the compiler's waits for X count only the loads it knows
+        // of, so a transfer requested between two X tiles would be waited for with the older tile
+#pragma unroll
+        for (int pc = 0; pc < 28; ++pc) w_issue(pc >> 3, pc & 7);
+#pragma unroll
+        for (int r = 0; r < kXAhead; ++r) {
+            load_col(r, 0);
+            load_col(r, 1);
+        }
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
             V8 o[2][4];  // [column][k quarter]: A_lo + B_lo, A_hi + B_hi, A_lo - B_lo, A_hi - B_hi
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 f32x4 sa[2], da[2], sb[2], db[2];
-                column_pair_f32<T16>(in[j][0], in[j][1], po, sa, da);
-                column_pair_f32<T16>(in[j][2], in[j][3], po, sb, db);
-                if (r + 1 < 8) load_col(r + 1, j);
-                // (the loads stay here, a round ahead of their use)
+                column_pair_f32<T16>(in[r % kXAhead][j][0], in[r % kXAhead][j][1], po, sa, da);
+                column_pair_f32<T16>(in[r % kXAhead][j][2], in[r % kXAhead][j][3], po, sb, db);
+                if (r + kXAhead < 8) load_col(r + kXAhead, j);
+                // (the loads stay here, kXAhead rounds ahead of their use)
                 __builtin_amdgcn_sched_barrier(0);
-                if (r >= 4) {  // W stages 0 .. 2 and the first half of stage 3, behind the last rounds of X
-#pragma unroll
-                    for (int u = 0; u < (j ? 3 : 4); ++u) {
-                        const int pc = 7 * (r - 4) + 4 * j + u;
-                        w_issue(pc >> 3, pc & 7);
-                    }
-                }
 #pragma unroll
                 for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -212,41 +216,49 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
     __builtin_amdgcn_s_barrier();
 
     // ---- fragments of this wavefront's stream ----------------------------------------------------
+    // Wavefront (cs, kp) takes the block's four row fragments in the order 2 kp, 2 kp + 1, then the
+    // other two: accumulators 0 and 1 are the ones it finishes, 2 and 3 the ones it hands over.
     const uint32_t frag_lane = lds_base + kp * 4u * k2h::kStage + k2h::frag_lane(lo, hi);
-    auto frag_addr = [&](int ks) __attribute__((always_inline)) -> uint32_t {
+    const uint32_t frag_lane_own = frag_lane + kp * 8192u, frag_lane_other = frag_lane - kp * 8192u;
+    auto frag_addr = [&](uint32_t lane_part, int ks) __attribute__((always_inline)) -> uint32_t {
         uint32_t a;
-        asm volatile("v_xor_b32 %0, %2, %1" : "=v"(a) : "v"(frag_lane), "i"(ks << 6));
+        asm volatile("v_xor_b32 %0, %2, %1" : "=v"(a) : "v"(lane_part), "i"(ks << 6));
         return a;
     };
     auto frag_read = [&](V8& dst, uint32_t a, int slot, int mb) __attribute__((always_inline)) {
         lds_read16(dst, a, slot * k2h::kStage + mb * 4096);
     };
     V8 fr[4][4];  // [K step % 4][mb]
-    {
-        const uint32_t a0 = frag_addr(0), a1 = frag_addr(1);
 #pragma unroll
-        for (int mb = 0; mb < 4; ++mb) frag_read(fr[0][mb], a0, 0, mb);
+    for (int ks = 0; ks < 2; ++ks) {
+        const uint32_t a_own = frag_addr(frag_lane_own, ks), a_other = frag_addr(frag_lane_other, ks);
 #pragma unroll
-        for (int mb = 0; mb < 4; ++mb) frag_read(fr[1][mb], a1, 0, mb);
+        for (int mb = 0; mb < 4; ++mb) frag_read(fr[ks][mb], mb < 2 ? a_own : a_other, 0, mb);
     }
 
-    // ---- output: wavefront (cs, kp) finishes row fragments mb = 2 kp, 2 kp + 1; lane (hi, lo) owns
-    // rows 16 mb + 4 hi + r of the adjacent columns n0 + 32 cs + 2 lo, + 1
+    // ---- output: wavefront (cs, kp) finishes rows 32 kp .. 32 kp + 31 of a block; lane (hi, lo) owns
+    // rows 16 f + 4 hi + r of them in the adjacent columns n0 + 32 cs + 2 lo, + 1
     constexpr uint32_t esize = OUT_F32 ? 4u : 2u;
     const uint32_t col = n0 + 32u * cs + 2u * lo;
     const uint32_t lane_off = (4u * hi * N + col) * esize;  // inside the row block, < 2^32
     unsigned char* const Cb = static_cast<unsigned char*>(C);
     const bool cols_full = n0 + kCols <= N && (N & 1u) == 0u;
-    unsigned char* const xb_mine = lds + k2h::kRegionBase + wave * 4096u;
-    const unsigned char* const xb_partner = lds + k2h::kRegionBase + (wave ^ 1u) * 4096u;
+    // where the two K halves meet: 4 KB per wavefront, fragment i = 2 f + nb at 1024 i + 16 lane
+    const uint32_t xb_mine = lds_base + k2h::kRegionBase + wave * 4096u + lane * 16u;
+    const uint32_t xb_partner = lds_base + k2h::kRegionBase + (wave ^ 1u) * 4096u + lane * 16u;
 
     // Transfers: two pieces per K step (behind MFMAs 4 and 6), every K step.  The stage whose reads
     // end with the barrier of K step 1 is refilled from K step 2 on: during K steps 2, 3 of stage kq
     // the first four pieces of stage kq + 4 go out (into the buffer of stage kq), during K steps 0, 1
     // of stage kq + 1 its other four.  At the barrier of stage kq the pieces of stages kq + 2 and
     // kq + 3 are the sixteen youngest, so the wait for stage kq + 1 is the same constant everywhere.
-    f32x4 acc[4][NBF];
-    f32x4 out[2][NBF];  // the finished half of the previous row block, stored during this one
+    //
+    // The halves of a finished block meet while the next block is being multiplied: two accumulator
+    // sets take turns, the fragments to hand over are written to LDS behind the MFMAs of K step 0,
+    // become visible with the stage barrier after K step 1, are read behind the MFMAs of K step 2,
+    // added and scaled in K step 4 and stored one row per K step from K step 5 on.
+    f32x4 acc[2][4][NBF];
+    f32x4 out[2][NBF];  // the partner's partial sums, then the finished values
     uint64_t out_base = 0;
     auto store_out = [&](int f, int r) __attribute__((always_inline)) {
         unsigned char* row_ptr = Cb + (out_base + (uint64_t)((16u * f + r) * N) * esize);  // scalar
@@ -256,9 +268,10 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
         else
             stream_store4(lane_off, __builtin_bit_cast(uint32_t, V2{(E)v0, (E)v1}), row_ptr);
     };
-    auto row_block_body = [&](auto last_tag, auto out_tag, uint32_t rbi) __attribute__((always_inline)) {
+    auto row_block_body = [&](auto last_tag, auto pending_tag, auto set_tag, uint32_t rbi) __attribute__((always_inline)) {
         constexpr bool last = decltype(last_tag)::value;
-        constexpr bool out_full = decltype(out_tag)::value;
+        constexpr bool pending = decltype(pending_tag)::value;  // the previous block awaits its other half
+        constexpr int cur = decltype(set_tag)::value, prev = cur ^ 1;
 #pragma unroll
         for (int kq = 0; kq < SPB; ++kq) {
             // (everything below folds to constants once the loops are unrolled; SPB is a multiple of
@@ -268,10 +281,14 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
             for (int ks = 0; ks < k2h::kSteps; ++ks) {
                 const int kk = kq * k2h::kSteps + ks;
                 // this step's fragments were requested two steps ago; the four of the step between
-                // are the only younger reads
+                // are the only younger reads (in K step 3 of a block also the four reads of the
+                // partner's sums, which K step 4 then finds complete)
                 wait_lds_all_but<4>();
+                if (pending && kk == 4)
+                    asm volatile("" : "+v"(out[0][0]), "+v"(out[0][1]), "+v"(out[1][0]), "+v"(out[1][1]));
                 const int read_slot = ks < 2 ? cur_slot : next_slot;
-                const uint32_t fa = frag_addr((ks + 2) & 3);
+                const uint32_t fa_own = frag_addr(frag_lane_own, (ks + 2) & 3);
+                const uint32_t fa_other = frag_addr(frag_lane_other, (ks + 2) & 3);
                 const int fill_stage = ks < 2 ? kq + AHEAD : kq + AHEAD + 1;  // may lie in the next row block
                 const int fill_kq = fill_stage % SPB;
 #pragma unroll
@@ -282,17 +299,21 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
                     if (transfer) {
                         // the lane offsets of the next row block replace this one's right before
                         // their first use (three vector instructions in the shadow of an MFMA)
-                        if (fill_stage == SPB) set_voff_piece(rbi + 1u, pi);
+                        if (fill_stage == SPB && pi < 4) set_voff_piece(rbi + 1u, pi);
                         lds_transfer_target(lds_wave_base, lds_piece(fill_kq, pi));
                     }
                     if (kk == 0)
-                        XMfma<T16>::first(acc[mb][nb], fr[ks & 3][mb], yf[nb][0]);
+                        XMfma<T16>::first(acc[cur][mb][nb], fr[ks & 3][mb], yf[nb][0]);
                     else
-                        XMfma<T16>::next(acc[mb][nb], fr[ks & 3][mb], yf[nb][kk]);
-                    if (m < 4) frag_read(fr[(ks + 2) & 3][m], fa, read_slot, m);
-                    if (transfer) lds_transfer_go(voff[pi], Wb + fill_kq * 256);
-                    // the previous block's eight stores, one per K step from K step 2 on
-                    if (out_full && kk >= 2 && kk < 10 && m == NM - 1) store_out((kk - 2) >> 2, (kk - 2) & 3);
+                        XMfma<T16>::next(acc[cur][mb][nb], fr[ks & 3][mb], yf[nb][kk]);
+                    if (m < 4) frag_read(fr[(ks + 2) & 3][m], m < 2 ? fa_own : fa_other, read_slot, m);
+                    if (transfer) lds_transfer_go(voff[pi & 3], w_base(fill_kq, pi));
+                    if (pending) {
+                        if (kk == 0 && m >= 4) lds_write16(xb_mine, acc[prev][2 + ((m - 4) >> 1)][m & 1], (m - 4) * 1024);
+                        if (kk == 2 && m >= 4) lds_read16(out[(m - 4) >> 1][m & 1], xb_partner, (m - 4) * 1024);
+                        if (kk == 4 && m < 4) out[m >> 1][m & 1] = (acc[prev][m >> 1][m & 1] + out[m >> 1][m & 1]) * mult;
+                        if (kk >= 5 && kk < 13 && m == NM - 1) store_out((kk - 5) >> 2, (kk - 5) & 3);
+                    }
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 // keep the previous step's fragment registers allocated while the matrix core may
@@ -310,54 +331,60 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
                 }
             }
         }
+        // the last MFMAs retire before anything else touches their accumulators
+        drain_mfma(acc[cur]);
     };
-
-    bool out_pending = false;
-#pragma unroll 1
-    for (uint32_t rbi = 0; rbi < nrb; ++rbi) {
-        const bool last_block = rbi + 1u == nrb;
-        if (last_block && out_pending)
-            row_block_body(std::true_type{}, std::true_type{}, rbi);
-        else if (last_block)
-            row_block_body(std::true_type{}, std::false_type{}, rbi);
-        else if (out_pending)
-            row_block_body(std::false_type{}, std::true_type{}, rbi);
-        else
-            row_block_body(std::false_type{}, std::false_type{}, rbi);
-        // ---- the two K halves meet: hand over two row fragments, finish the other two -------------
-        drain_mfma(acc);
-        f32x4 keep[2][NBF], give[2][NBF];
+    // the same meeting of the halves with nothing to hide it behind: the last block of a workgroup,
+    // and blocks whose stores need bounds checks
+    auto meet_now = [&](auto set_tag) __attribute__((always_inline)) {
+        constexpr int cur = decltype(set_tag)::value;
 #pragma unroll
-        for (int f = 0; f < 2; ++f)
-#pragma unroll
-            for (int nb = 0; nb < NBF; ++nb) {
-                keep[f][nb] = kp ? acc[2 + f][nb] : acc[f][nb];
-                give[f][nb] = kp ? acc[f][nb] : acc[2 + f][nb];
-            }
-#pragma unroll
-        for (int f = 0; f < 2; ++f)
-#pragma unroll
-            for (int nb = 0; nb < NBF; ++nb)
-                *reinterpret_cast<f32x4*>(xb_mine + (2 * f + nb) * 1024u + lane * 16u) = give[f][nb];
+        for (int i = 0; i < 4; ++i) lds_write16(xb_mine, acc[cur][2 + (i >> 1)][i & 1], i * 1024);
         wait_lds();
         __builtin_amdgcn_s_barrier();
 #pragma unroll
-        for (int f = 0; f < 2; ++f)
+        for (int i = 0; i < 4; ++i) lds_read16(out[i >> 1][i & 1], xb_partner, i * 1024);
+        wait_lds();
+        asm volatile("" : "+v"(out[0][0]), "+v"(out[0][1]), "+v"(out[1][0]), "+v"(out[1][1]));
 #pragma unroll
-            for (int nb = 0; nb < NBF; ++nb) {
-                const f32x4 got = *reinterpret_cast<const f32x4*>(xb_partner + (2 * f + nb) * 1024u + lane * 16u);
-                out[f][nb] = (kp ? got + keep[f][nb] : keep[f][nb] + got) * mult;  // (k < 1024) + (k >= 1024)
-            }
+        for (int i = 0; i < 4; ++i) out[i >> 1][i & 1] = (acc[cur][i >> 1][i & 1] + out[i >> 1][i & 1]) * mult;
+    };
+
+    bool pending = false;
+#pragma unroll 1
+    for (uint32_t rbi = 0; rbi < nrb; ++rbi) {
+        const bool last_block = rbi + 1u == nrb;
+        const bool odd = rbi & 1u;
+        using T = std::true_type;
+        using F = std::false_type;
+        using S0 = std::integral_constant<int, 0>;
+        using S1 = std::integral_constant<int, 1>;
+        if (!odd) {
+            if (last_block && pending) row_block_body(T{}, T{}, S0{}, rbi);
+            else if (last_block) row_block_body(T{}, F{}, S0{}, rbi);
+            else if (pending) row_block_body(F{}, T{}, S0{}, rbi);
+            else row_block_body(F{}, F{}, S0{}, rbi);
+        } else {
+            if (last_block && pending) row_block_body(T{}, T{}, S1{}, rbi);
+            else if (last_block) row_block_body(T{}, F{}, S1{}, rbi);
+            else if (pending) row_block_body(F{}, T{}, S1{}, rbi);
+            else row_block_body(F{}, F{}, S1{}, rbi);
+        }
         const uint32_t row_base = m_begin + rbi * kRows;
         const bool full = cols_full && row_base + kRows <= m_end;
         out_base = ((uint64_t)row_base + 32u * kp) * N * esize;
-        out_pending = full && !last_block;  // stored behind the MFMAs of the next row block
-        if (full && last_block) {
+        pending = full && !last_block;  // its halves meet behind the MFMAs of the next row block
+        if (pending) continue;
+        if (odd)
+            meet_now(S1{});
+        else
+            meet_now(S0{});
+        if (full) {
 #pragma unroll
             for (int f = 0; f < 2; ++f)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) store_out(f, r);
-        } else if (!full) {
+        } else {
 #pragma unroll
             for (int f = 0; f < 2; ++f)
 #pragma unroll

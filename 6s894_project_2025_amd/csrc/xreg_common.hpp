@@ -147,6 +147,13 @@ __device__ __forceinline__ void lds_read16(V& dst, uint32_t addr, int offset)
 {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(offset) : "memory");
 }
+// One 16-byte LDS write per lane, equally opaque; the data registers must stay as they are until
+// the write has been waited for.
+template <class V>
+__device__ __forceinline__ void lds_write16(uint32_t addr, V v, int offset)
+{
+    asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(addr), "v"(v), "i"(offset) : "memory");
+}
 // at most N LDS reads of this wavefront still outstanding (they complete in order)
 template <int N>
 __device__ __forceinline__ void wait_lds_all_but()
