@@ -13,9 +13,11 @@
 // stream only.  At the end of a row block each wavefront of a pair hands the partner the
 // accumulators of two of the four 16-row fragments through LDS and finishes (adds, stores) the
 // other two, always as (k < 1024) + (k >= 1024).
-// The prologue is shared inside a pair: per round, each wavefront transforms two of the pair's next
-// four columns, all of K, and writes both halves into the pair's LDS region; after a barrier each
-// wavefront reads its own half of the four columns.
+// The prologue is shared inside a pair: in each of four rounds the pair transforms eight columns of
+// its set, all of K (four columns per wavefront), and writes both halves into the pair's LDS area;
+// after a barrier each wavefront reads its own half of the eight columns in operand order (the half
+// of the lanes whose columns these are).  The area is the ring's fourth buffers plus the 32 KB behind
+// the ring, so the first three stage times of W are on their way meanwhile.
 //
 // Main-loop statements are the hand-placed single instructions of xreg_common.hpp (see the
 // K = 1024 kernel for the reasons).
@@ -35,10 +37,17 @@ constexpr int kSteps = 4;          // K steps of 32 per stage
 constexpr int SPB = 8;             // stages per row block and stream
 constexpr int AHEAD = 3;
 constexpr int KSTEPS = 32;         // K steps per row block and wavefront
-// behind the two rings: the prologue's regions [column set][half][4 columns][2 KB], later the
-// exchange buffers [wavefront][4 KB]
+// Ring: buffer b (= stage % 4) of stream t at (4 t + b) kStage (fragment reads reach every buffer of
+// a stream with a 16-bit offset).  Behind the ring 32 KB.  The prologue's area, four blocks
+// [8 columns][2 KB], one per column set and K half, is the fourth buffer of either stream (set 0) and
+// those 32 KB (set 1); later the 32 KB hold the hand-over buffers [wavefront][4 KB].
 constexpr uint32_t kRegionBase = 8 * kStage;
-static_assert(kRegionBase + 2 * 2 * 4 * 2048 == (uint32_t)kLdsBytes, "rings and regions fill the 160 KB");
+static_assert(kRegionBase + 32 * 1024 == (uint32_t)kLdsBytes, "ring and the 32 KB behind it fill the 160 KB");
+static_assert(8 * 2048 == kStage, "an area block is a stage buffer");
+__host__ __device__ constexpr uint32_t area_block(uint32_t cs, uint32_t half)
+{
+    return cs ? kRegionBase + half * (uint32_t)kStage : (3u + 4u * half) * (uint32_t)kStage;
+}
 
 // LDS image of a stage: [64 rows][256 B], the 16-byte chunk q of row r stored at q ^ (r & 15)
 __host__ __device__ constexpr uint32_t stage_offset(uint32_t row, uint32_t q)
@@ -48,15 +57,12 @@ __host__ __device__ constexpr uint32_t stage_offset(uint32_t row, uint32_t q)
 // lane part of a fragment address (row lo, chunk hi): the fragment of row block mb and K step ks of
 // the stage is at (frag_lane ^ (ks << 6)) + 4096 mb
 __host__ __device__ constexpr uint32_t frag_lane(uint32_t lo, uint32_t hi) { return lo * 256u + ((hi ^ lo) << 4); }
-// a half's four columns in the prologue region: [4 columns][128 chunks], chunk q of column c stored
-// at q ^ 2 (c / 2); for q = 4 s + hi that is region_read_base(c, hi) + 64 s
-__host__ __device__ constexpr uint32_t region_offset(uint32_t c, uint32_t q)
+// a half's eight columns in the prologue area: [8 columns][128 chunks], chunk q of column c stored
+// at q ^ c; for q = 4 s + hi that is area_read_base(c, hi) + 64 (s ^ (c / 4))
+__host__ __device__ constexpr uint32_t area_offset(uint32_t c, uint32_t q) { return c * 2048u + ((q ^ c) << 4); }
+__host__ __device__ constexpr uint32_t area_read_base(uint32_t c, uint32_t hi)
 {
-    return c * 2048u + ((q ^ (2u * (c >> 1))) << 4);
-}
-__host__ __device__ constexpr uint32_t region_read_base(uint32_t c, uint32_t hi)
-{
-    return c * 2048u + ((hi ^ (2u * (c >> 1))) << 4);
+    return c * 2048u + ((hi ^ (c & 3u)) << 4);
 }
 constexpr bool patterns_ok()
 {
@@ -71,22 +77,21 @@ constexpr bool patterns_ok()
             if (!lds::conflict_free_b128(
                     [=](uint32_t lane) { return stage_offset(16u * mb + (lane & 15u), 4u * ks + (lane >> 4)); }))
                 return false;
-    for (uint32_t c = 0; c < 4; ++c)
+    for (uint32_t c = 0; c < 8; ++c)
         for (uint32_t hi = 0; hi < 4; ++hi)
             for (uint32_t s = 0; s < 32; ++s)
-                if (region_read_base(c, hi) + 64u * s != region_offset(c, 4u * s + hi)) return false;
-    // every lane writes chunk 64 t + lane of a column; in round r the lanes with lo / 2 == r read
-    // chunk 4 s + hi of column 2 (lo % 2) + nb
-    for (uint32_t c = 0; c < 4; ++c)
+                if (area_read_base(c, hi) + 64u * (s ^ (c >> 2)) != area_offset(c, 4u * s + hi)) return false;
+    // every lane writes chunk 64 t + lane of a column; in rounds 2 h, 2 h + 1 the lanes with
+    // lo / 8 == h read chunk 4 s + hi of column lo % 8
+    for (uint32_t c = 0; c < 8; ++c)
         for (uint32_t t = 0; t < 2; ++t)
-            if (!lds::conflict_free_b128([=](uint32_t lane) { return region_offset(c, 64u * t + lane); })) return false;
-    for (uint32_t nb = 0; nb < 2; ++nb)
-        for (uint32_t r = 0; r < 8; ++r)
-            for (uint32_t s = 0; s < 32; ++s)
-                if (!lds::conflict_free_b128_masked(
-                        [=](uint32_t lane) { return region_offset(2u * (lane & 1u) + nb, 4u * s + (lane >> 4)); },
-                        [=](uint32_t lane) { return ((lane & 15u) >> 1) == r; }))
-                    return false;
+            if (!lds::conflict_free_b128([=](uint32_t lane) { return area_offset(c, 64u * t + lane); })) return false;
+    for (uint32_t h = 0; h < 2; ++h)
+        for (uint32_t s = 0; s < 32; ++s)
+            if (!lds::conflict_free_b128_masked(
+                    [=](uint32_t lane) { return area_offset(lane & 7u, 4u * s + (lane >> 4)); },
+                    [=](uint32_t lane) { return ((lane & 15u) >> 3) == h; }))
+                return false;
     return true;
 }
 static_assert(patterns_ok(), "an LDS access pattern of the split-K 16-bit kernel would serialise");
@@ -143,77 +148,77 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
     for (int j = 0; j < 4; ++j) set_voff_piece(0, j);
 
     // ---- prologue: column nb of lane (., lo) = column n0 + 32 cs + 2 lo + nb, its half kp -------------
+    // Round R = 2 h + nb: the set's columns 2 (8 h + i) + nb, i = 0 .. 7; wavefront kp of the pair
+    // transforms i = 4 kp .. 4 kp + 3, and the lanes with lo / 8 == h read back column i = lo % 8.
     V8 yf[NBF][KSTEPS];
     {
-        unsigned char* const region = lds + k2h::kRegionBase + cs * 16384u;  // [half][4 columns][2 KB]
         PairOperands<T16> po;
         make_pair_operands<T16>(po, exp2);
-        // X tiles are requested kXAhead rounds before their use: one round of transforms is far
-        // shorter than a trip to memory
-        constexpr int kXAhead = 2;
-        V8 in[kXAhead][2][4];  // [round % kXAhead][column of this wavefront in the round][tile]
-        auto load_col = [&](int r, int j) {  // the wavefront's column j of round r: 4 r + 2 j + kp of the set
-            const uint32_t col = min(n0 + 32u * cs + (uint32_t)(4 * r + 2 * j) + kp, N - 1u);
+        // The first three stage times of W go out before any X: vector memory operations complete in
+        // order and the compiler's waits for X count only the loads it knows of, so a transfer
+        // requested between two X tiles would be waited for with the older tile.
+#pragma unroll
+        for (int pc = 0; pc < 8 * AHEAD; ++pc) w_issue(pc >> 3, pc & 7);
+        // X tiles are requested a round before their use
+        V8 in[4][4];  // [column of the wavefront in its round][tile]
+        auto load_col = [&](int R, int jj) {
+            const uint32_t i = 4u * kp + (uint32_t)jj;
+            const uint32_t col = min(n0 + 32u * cs + 2u * (8u * (uint32_t)(R >> 1) + i) + (uint32_t)(R & 1), N - 1u);
 #pragma unroll
             for (int t = 0; t < 4; ++t)
-                in[r % kXAhead][j][t] = *reinterpret_cast<const V8*>(Xt + ((uint64_t)col * K + 512u * t + 8u * lane));
+                in[jj][t] = *reinterpret_cast<const V8*>(Xt + ((uint64_t)col * K + 512u * t + 8u * lane));
         };
-        // W stages 0 .. 2 and the first half of stage 3 go out before any X: vector memory
-        // operations complete in order and the compiler's waits for X count only the loads it knows
-        // of, so a transfer requested between two X tiles would be waited for with the older tile
 #pragma unroll
-        for (int pc = 0; pc < 28; ++pc) w_issue(pc >> 3, pc & 7);
+        for (int jj = 0; jj < 4; ++jj) load_col(0, jj);
+        const uint32_t cl = lo & 7u;
+        const unsigned char* const src = lds + k2h::area_block(cs, kp) + k2h::area_read_base(cl, hi);
+        const unsigned char* const src_even = src + 64u * (cl >> 2);  // K step s: + 64 (s ^ (cl / 4))
+        const unsigned char* const src_odd = src - 64u * (cl >> 2);
 #pragma unroll
-        for (int r = 0; r < kXAhead; ++r) {
-            load_col(r, 0);
-            load_col(r, 1);
-        }
+        for (int R = 0; R < 4; ++R) {
+            if (R > 0) {  // the partner has read the previous round's columns
+                wait_lds();
+                __builtin_amdgcn_s_barrier();
+            }
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
-            V8 o[2][4];  // [column][k quarter]: A_lo + B_lo, A_hi + B_hi, A_lo - B_lo, A_hi - B_hi
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
+            for (int jj = 0; jj < 4; ++jj) {
                 f32x4 sa[2], da[2], sb[2], db[2];
-                column_pair_f32<T16>(in[r % kXAhead][j][0], in[r % kXAhead][j][1], po, sa, da);
-                column_pair_f32<T16>(in[r % kXAhead][j][2], in[r % kXAhead][j][3], po, sb, db);
-                if (r + kXAhead < 8) load_col(r + kXAhead, j);
-                // (the loads stay here, kXAhead rounds ahead of their use)
+                column_pair_f32<T16>(in[jj][0], in[jj][1], po, sa, da);
+                column_pair_f32<T16>(in[jj][2], in[jj][3], po, sb, db);
+                if (R + 1 < 4) load_col(R + 1, jj);
+                // (the loads stay here, a round ahead of their use)
                 __builtin_amdgcn_sched_barrier(0);
+                V8 o[4];  // k quarters: A_lo + B_lo, A_hi + B_hi, A_lo - B_lo, A_hi - B_hi
 #pragma unroll
                 for (int h = 0; h < 2; ++h)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        o[j][0][4 * h + e] = (E)(sa[h][e] + sb[h][e]);
-                        o[j][1][4 * h + e] = (E)(da[h][e] + db[h][e]);
-                        o[j][2][4 * h + e] = (E)(sa[h][e] - sb[h][e]);
-                        o[j][3][4 * h + e] = (E)(da[h][e] - db[h][e]);
+                        o[0][4 * h + e] = (E)(sa[h][e] + sb[h][e]);
+                        o[1][4 * h + e] = (E)(da[h][e] + db[h][e]);
+                        o[2][4 * h + e] = (E)(sa[h][e] - sb[h][e]);
+                        o[3][4 * h + e] = (E)(da[h][e] - db[h][e]);
                     }
-            }
-            // the partner has read the previous round's columns
-            wait_lds();
-            __builtin_amdgcn_s_barrier();
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
 #pragma unroll
                 for (int q = 0; q < 4; ++q)  // quarter q = half q / 2, chunks 64 (q % 2) + lane of it
-                    *reinterpret_cast<V8*>(region + (q >> 1) * 8192u +
-                                           k2h::region_offset(2u * j + kp, 64u * (q & 1) + lane)) = o[j][q];
+                    *reinterpret_cast<V8*>(lds + k2h::area_block(cs, q >> 1) +
+                                           k2h::area_offset(4u * kp + (uint32_t)jj, 64u * (q & 1) + lane)) = o[q];
+            }
             wait_lds();
             __builtin_amdgcn_s_barrier();
-            if ((int)(lo >> 1) == r) {
+            if ((int)(lo >> 3) == (R >> 1)) {
 #pragma unroll
-                for (int nb = 0; nb < NBF; ++nb) {
-                    const unsigned char* src = region + kp * 8192u + k2h::region_read_base(2u * (lo & 1u) + nb, hi);
-#pragma unroll
-                    for (int s = 0; s < KSTEPS; ++s) yf[nb][s] = *reinterpret_cast<const V8*>(src + 64u * s);
-                }
+                for (int s = 0; s < KSTEPS; ++s)
+                    yf[R & 1][s] = *reinterpret_cast<const V8*>(((s & 1) ? src_odd : src_even) + 64u * s);
             }
         }
     }
-
-    wait_vm(8 * (AHEAD - 1) + 4);  // stage 0 has landed (stages 1, 2 and half of 3 are younger)
+    // stage 0 of W has landed (stages 1 and 2 are younger), everybody is done with the area: its
+    // part inside the ring can take the first half of stage 3
+    wait_vm(8 * (AHEAD - 1));
     wait_lds();
     __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w_issue(AHEAD, i);
 
     // ---- fragments of this wavefront's stream ----------------------------------------------------
     // Wavefront (cs, kp) takes the block's four row fragments in the order 2 kp, 2 kp + 1, then the
