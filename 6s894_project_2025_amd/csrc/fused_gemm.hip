@@ -1,9 +1,11 @@
 // Fused Hadamard -> GEMM (mi_fused_ht_gemm), gfx950:  C[M,N] = W[M,K] * (scale * H_K * X[K,N]),
 // X given as Xt[N,K].  The transformed operand lives only in LDS.
 //
-// This file: the dispatcher and the LDS-resident variant, used for K = 32 .. 512, 2048 and 4096.
-// K = 1024 goes to the register-resident variant in fused_gemm_xreg.hip, which holds twice as many
-// columns per compute unit.
+// This file: the dispatcher and the LDS-resident variant, used for K = 32 .. 256 (64 columns per
+// workgroup, a column at most one tile; the kernel is written for any BN and for columns of several
+// tiles, which larger K used before the register-resident kernels took them over).  K >= 512 goes to
+// the register-resident variants in fused_gemm_xreg.hip and fused_gemm_xreg_k2048.hip, which hold
+// more columns per compute unit.
 //
 // Structure ("X-stationary"): a workgroup owns BN columns of X for the whole K extent.
 //   prologue : its wavefronts transform those BN rows of Xt on the matrix cores (tile_transform,
@@ -32,7 +34,7 @@
 
 namespace mi {
 
-// K = 512, 1024 and 2048 with the transformed operand in registers: fused_gemm_xreg.hip
+// K = 512 ... 4096 with the transformed operand in registers: fused_gemm_xreg.hip
 int fused_gemm16_xreg(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
                       int in_dtype, int out_f32, float scale, hipStream_t s);
 
@@ -457,8 +459,8 @@ int dispatch_gemm16(const void* W, const void* Xt, void* C, uint32_t M, uint32_t
         case 256: return launch_gemm16<T16, 64, 0, 0>(W, Xt, C, M, N, K, out_f32, scale, s);
         case 512:
         case 1024:
-        case 2048: return fused_gemm16_xreg(W, Xt, C, M, N, K, T16::kCode, out_f32, scale, s);
-        case 4096: return launch_gemm16<T16, 16, 3, 0>(W, Xt, C, M, N, K, out_f32, scale, s);
+        case 2048:
+        case 4096: return fused_gemm16_xreg(W, Xt, C, M, N, K, T16::kCode, out_f32, scale, s);
         default: return MI_ERR_SIZE;
     }
 }

@@ -509,12 +509,12 @@ int launch(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, int o
 
 }  // namespace xreg
 
-// K = 2048: fused_gemm_xreg_k2048.hip
-int fused_gemm16_xreg_k2048(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, int in_dtype,
-                            int out_f32, float scale, hipStream_t s);
+// K = 2048 and 4096: fused_gemm_xreg_k2048.hip
+int fused_gemm16_xreg_k2048(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
+                            int in_dtype, int out_f32, float scale, hipStream_t s);
 
-// Called by the dispatcher of mi_fused_ht_gemm for K = 512, 1024 and 2048 (arguments already
-// validated there).
+// Called by the dispatcher of mi_fused_ht_gemm for K = 512 ... 4096 (arguments already validated
+// there).
 int fused_gemm16_xreg(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
                       int in_dtype, int out_f32, float scale, hipStream_t s)
 {
@@ -527,8 +527,8 @@ int fused_gemm16_xreg(const void* W, const void* Xt, void* C, uint32_t M, uint32
     } else if (K == 512u) {
         if (in_dtype == MI_BF16) return xreg::launch<BF16, 512>(W, Xt, C, M, N, out_f32, scale, 8u, s);
         if (in_dtype == MI_F16) return xreg::launch<F16, 512>(W, Xt, C, M, N, out_f32, scale, 8u, s);
-    } else if (K == 2048u) {
-        return fused_gemm16_xreg_k2048(W, Xt, C, M, N, in_dtype, out_f32, scale, s);
+    } else if (K == 2048u || K == 4096u) {
+        return fused_gemm16_xreg_k2048(W, Xt, C, M, N, K, in_dtype, out_f32, scale, s);
     } else {
         return MI_ERR_SIZE;
     }

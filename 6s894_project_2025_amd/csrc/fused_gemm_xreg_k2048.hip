@@ -98,7 +98,11 @@ static_assert(patterns_ok(), "an LDS access pattern of the split-K 16-bit kernel
 
 }  // namespace k2h
 
-template <class T16, bool OUT_F32>
+// KTOT = 2048: the whole contraction.  KTOT = 4096: one of two passes; pass 0 (ACCUM = false)
+// contracts W[:, :2048] with the first half of H_4096 x = [H_2048 a + H_2048 b; H_2048 a - H_2048 b]
+// (a, b the halves of a column) and stores, pass 1 (ACCUM = true) contracts W[:, 2048:] with the
+// second half and adds to what pass 0 stored.
+template <class T16, bool OUT_F32, int KTOT, bool ACCUM>
 __global__ void __launch_bounds__(kThreads)
 fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typename T16::E* __restrict__ Xt,
                                 void* __restrict__ C, uint32_t M, uint32_t N, uint32_t m_per_block,
@@ -108,7 +112,9 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
     using E = typename T16::E;
     using V8 = typename T16::V8;
     typedef E V2 __attribute__((ext_vector_type(2)));
-    constexpr int K = 2048, NBF = 2, NM = 8;
+    static_assert(KTOT == 2048 || (KTOT == 4096), "K = 2048, or one half of K = 4096");
+    static_assert(KTOT == 4096 || !ACCUM, "a single pass stores");
+    constexpr int K = KTOT, NBF = 2, NM = 8;  // K: row length of W and Xt
     constexpr int SPB = k2h::SPB, AHEAD = k2h::AHEAD, KSTEPS = k2h::KSTEPS;
     constexpr uint32_t kCols = 64;
     constexpr uint32_t ROW_BYTES = K * 2u;
@@ -130,7 +136,7 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
 
     // ---- W streams: per stage time a wavefront moves rows 16 w .. 16 w + 15 of both streams' stages,
     // eight pieces of 4 rows x 256 B (piece i: stream i / 4, rows 4 (i % 4) .. + 3)
-    const unsigned char* Wb = reinterpret_cast<const unsigned char*>(W);
+    const unsigned char* Wb = reinterpret_cast<const unsigned char*>(W) + (ACCUM ? 4096u : 0u);  // the pass's 2048 k
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;
     const uint32_t lrow = lane >> 4, lq = lane & 15u;
     uint32_t voff[4];  // lane offset of rows 4 j .. 4 j + 3 (the second stream's 2048 bytes go into the scalar base)
@@ -159,17 +165,18 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
         // requested between two X tiles would be waited for with the older tile.
 #pragma unroll
         for (int pc = 0; pc < 8 * AHEAD; ++pc) w_issue(pc >> 3, pc & 7);
-        // X tiles are requested a round before their use
-        V8 in[4][4];  // [column of the wavefront in its round][tile]
-        auto load_col = [&](int R, int jj) {
-            const uint32_t i = 4u * kp + (uint32_t)jj;
-            const uint32_t col = min(n0 + 32u * cs + 2u * (8u * (uint32_t)(R >> 1) + i) + (uint32_t)(R & 1), N - 1u);
+        // X tiles are requested kAhead columns before their use (a round at K = 2048)
+        constexpr int NT = KTOT / 512, kAhead = 16 / NT;
+        V8 in[kAhead][NT];  // [column of the wavefront % kAhead][tile]
+        auto load_col = [&](int c) {  // the wavefront's column c = 4 R + jj
+            const uint32_t i = 4u * kp + (uint32_t)(c & 3);
+            const uint32_t col = min(n0 + 32u * cs + 2u * (8u * (uint32_t)(c >> 3) + i) + (uint32_t)((c >> 2) & 1), N - 1u);
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
-                in[jj][t] = *reinterpret_cast<const V8*>(Xt + ((uint64_t)col * K + 512u * t + 8u * lane));
+            for (int t = 0; t < NT; ++t)
+                in[c % kAhead][t] = *reinterpret_cast<const V8*>(Xt + ((uint64_t)col * K + 512u * t + 8u * lane));
         };
 #pragma unroll
-        for (int jj = 0; jj < 4; ++jj) load_col(0, jj);
+        for (int c = 0; c < kAhead; ++c) load_col(c);
         const uint32_t cl = lo & 7u;
         const unsigned char* const src = lds + k2h::area_block(cs, kp) + k2h::area_read_base(cl, hi);
         const unsigned char* const src_even = src + 64u * (cl >> 2);  // K step s: + 64 (s ^ (cl / 4))
@@ -182,22 +189,51 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
             }
 #pragma unroll
             for (int jj = 0; jj < 4; ++jj) {
-                f32x4 sa[2], da[2], sb[2], db[2];
-                column_pair_f32<T16>(in[jj][0], in[jj][1], po, sa, da);
-                column_pair_f32<T16>(in[jj][2], in[jj][3], po, sb, db);
-                if (R + 1 < 4) load_col(R + 1, jj);
-                // (the loads stay here, a round ahead of their use)
-                __builtin_amdgcn_sched_barrier(0);
-                V8 o[4];  // k quarters: A_lo + B_lo, A_hi + B_hi, A_lo - B_lo, A_hi - B_hi
+                const int c = 4 * R + jj, e = c % kAhead;
+                // the lane's eight values of each k quarter of the 2048 transformed values this
+                // pass keeps, [quarter][4 h .. 4 h + 3]
+                f32x4 qv[4][2];
+                {
+                    f32x4 sa[2], da[2], sb[2], db[2];
+                    column_pair_f32<T16>(in[e][0], in[e][1], po, sa, da);
+                    column_pair_f32<T16>(in[e][2], in[e][3], po, sb, db);
 #pragma unroll
-                for (int h = 0; h < 2; ++h)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        o[0][4 * h + e] = (E)(sa[h][e] + sb[h][e]);
-                        o[1][4 * h + e] = (E)(da[h][e] + db[h][e]);
-                        o[2][4 * h + e] = (E)(sa[h][e] - sb[h][e]);
-                        o[3][4 * h + e] = (E)(da[h][e] - db[h][e]);
+                    for (int h = 0; h < 2; ++h) {  // A_lo + B_lo, A_hi + B_hi, A_lo - B_lo, A_hi - B_hi
+                        qv[0][h] = sa[h] + sb[h];
+                        qv[1][h] = da[h] + db[h];
+                        qv[2][h] = sa[h] - sb[h];
+                        qv[3][h] = da[h] - db[h];
                     }
+                }
+                if constexpr (KTOT == 4096) {  // the same of the column's second half, added or subtracted
+                    f32x4 sa[2], da[2], sb[2], db[2];
+                    column_pair_f32<T16>(in[e][4], in[e][5], po, sa, da);
+                    column_pair_f32<T16>(in[e][6], in[e][7], po, sb, db);
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        if (ACCUM) {
+                            qv[0][h] -= sa[h] + sb[h];
+                            qv[1][h] -= da[h] + db[h];
+                            qv[2][h] -= sa[h] - sb[h];
+                            qv[3][h] -= da[h] - db[h];
+                        } else {
+                            qv[0][h] += sa[h] + sb[h];
+                            qv[1][h] += da[h] + db[h];
+                            qv[2][h] += sa[h] - sb[h];
+                            qv[3][h] += da[h] - db[h];
+                        }
+                    }
+                }
+                if (c + kAhead < 16) load_col(c + kAhead);
+                // (the loads stay here, kAhead columns ahead of their use)
+                __builtin_amdgcn_sched_barrier(0);
+                V8 o[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+#pragma unroll
+                        for (int el = 0; el < 4; ++el) o[q][4 * h + el] = (E)qv[q][h][el];
 #pragma unroll
                 for (int q = 0; q < 4; ++q)  // quarter q = half q / 2, chunks 64 (q % 2) + lane of it
                     *reinterpret_cast<V8*>(lds + k2h::area_block(cs, q >> 1) +
@@ -268,10 +304,20 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
     auto store_out = [&](int f, int r) __attribute__((always_inline)) {
         unsigned char* row_ptr = Cb + (out_base + (uint64_t)((16u * f + r) * N) * esize);  // scalar
         const float v0 = out[f][0][r], v1 = out[f][1][r];
-        if (OUT_F32)
+        if (ACCUM) {
+            // second pass: every element has one owner and the first pass has completed, so the
+            // addition needs no ordering; done in the L2, it spares the loop a wait for loaded values
+            if (OUT_F32) {
+                add_f32_to_memory(lane_off, v0, row_ptr, 0);
+                add_f32_to_memory(lane_off, v1, row_ptr, 4);
+            } else {
+                XMfma<T16>::add_pair_to_memory(lane_off, __builtin_bit_cast(uint32_t, V2{(E)v0, (E)v1}), row_ptr);
+            }
+        } else if (OUT_F32) {
             stream_store8(lane_off, u32x2{__float_as_uint(v0), __float_as_uint(v1)}, row_ptr);
-        else
+        } else {
             stream_store4(lane_off, __builtin_bit_cast(uint32_t, V2{(E)v0, (E)v1}), row_ptr);
+        }
     };
     auto row_block_body = [&](auto last_tag, auto pending_tag, auto set_tag, uint32_t rbi) __attribute__((always_inline)) {
         constexpr bool last = decltype(last_tag)::value;
@@ -402,9 +448,9 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
                         const float v = out[f][nb][r];
                         const uint64_t at = (uint64_t)row * N + col + nb;
                         if (OUT_F32)
-                            static_cast<float*>(C)[at] = v;
+                            static_cast<float*>(C)[at] = ACCUM ? static_cast<float*>(C)[at] + v : v;
                         else
-                            static_cast<E*>(C)[at] = (E)v;
+                            static_cast<E*>(C)[at] = ACCUM ? (E)((float)static_cast<E*>(C)[at] + v) : (E)v;
                     }
                 }
         }
@@ -414,12 +460,11 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
 }
 
 namespace {
-template <class T16, bool OUT_F32>
-int launch_k2048(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, float scale, hipStream_t s)
+template <class T16, bool OUT_F32, int KTOT, bool ACCUM>
+int launch_pass(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, const Plan& p, OutputScale os,
+                hipStream_t s)
 {
-    const OutputScale os = split_output_scale((double)scale, tile_stage_shift<2>(11u, kNarrowRange<T16>));
-    const Plan p = plan(M, N, 64u, 8u);
-    auto kern = fused_ht_gemm_xreg_k2048_kernel<T16, OUT_F32>;
+    auto kern = fused_ht_gemm_xreg_k2048_kernel<T16, OUT_F32, KTOT, ACCUM>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             kLdsBytes) != hipSuccess)
         return MI_ERR_LAUNCH;
@@ -428,21 +473,38 @@ int launch_k2048(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N,
                        p.nrect, os.exp2, os.mult);
     return launch_status();
 }
+
+template <class T16, bool OUT_F32>
+int launch_ksplit16(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K, float scale,
+                    hipStream_t s)
+{
+    const OutputScale os = split_output_scale((double)scale, tile_stage_shift<2>(11u, kNarrowRange<T16>));
+    if (K == 2048u) return launch_pass<T16, OUT_F32, 2048, false>(W, Xt, C, M, N, plan(M, N, 64u, 8u), os, s);
+    // K = 4096: a workgroup transforms twice as much per column as at K = 2048 for the same main loop
+    const Plan p = plan(M, N, 64u, 8u, 18u, 4u);
+    const int rc = launch_pass<T16, OUT_F32, 4096, false>(W, Xt, C, M, N, p, os, s);
+    if (rc != MI_OK) return rc;
+    return launch_pass<T16, OUT_F32, 4096, true>(W, Xt, C, M, N, p, os, s);
+}
 }  // namespace
 
 }  // namespace xreg
 
-// Called by fused_gemm16_xreg for K = 2048 (arguments already validated).
-int fused_gemm16_xreg_k2048(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, int in_dtype,
-                            int out_f32, float scale, hipStream_t s)
+// Called by fused_gemm16_xreg for K = 2048 and by the dispatcher of mi_fused_ht_gemm for K = 4096
+// (arguments already validated).
+int fused_gemm16_xreg_k2048(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
+                            int in_dtype, int out_f32, float scale, hipStream_t s)
 {
     using namespace xreg;
+    if (K != 2048u && K != 4096u) return MI_ERR_SIZE;
+    // W and a row block of C are addressed with 32-bit byte offsets
+    if ((uint64_t)M * K * 2u > 0xffffffffull || (uint64_t)N * 4u * 64u > 0xffffffffull) return MI_ERR_SHAPE;
     if (in_dtype == MI_BF16)
-        return out_f32 ? launch_k2048<BF16, true>(W, Xt, C, M, N, scale, s)
-                       : launch_k2048<BF16, false>(W, Xt, C, M, N, scale, s);
+        return out_f32 ? launch_ksplit16<BF16, true>(W, Xt, C, M, N, K, scale, s)
+                       : launch_ksplit16<BF16, false>(W, Xt, C, M, N, K, scale, s);
     if (in_dtype == MI_F16)
-        return out_f32 ? launch_k2048<F16, true>(W, Xt, C, M, N, scale, s)
-                       : launch_k2048<F16, false>(W, Xt, C, M, N, scale, s);
+        return out_f32 ? launch_ksplit16<F16, true>(W, Xt, C, M, N, K, scale, s)
+                       : launch_ksplit16<F16, false>(W, Xt, C, M, N, K, scale, s);
     return MI_ERR_DTYPE;
 }
 

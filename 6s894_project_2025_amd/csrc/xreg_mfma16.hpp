@@ -26,6 +26,11 @@ struct XMfma<BF16> {
     {
         asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
     }
+    // adds a pair of adjacent 16-bit values to memory (performed in the L2, nothing returned)
+    static __device__ __forceinline__ void add_pair_to_memory(uint32_t lane_off, uint32_t v, void* base)
+    {
+        asm volatile("global_atomic_pk_add_bf16 %0, %1, %2" ::"v"(lane_off), "v"(v), "s"(base) : "memory");
+    }
 };
 template <>
 struct XMfma<F16> {
@@ -37,7 +42,16 @@ struct XMfma<F16> {
     {
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
     }
+    static __device__ __forceinline__ void add_pair_to_memory(uint32_t lane_off, uint32_t v, void* base)
+    {
+        asm volatile("global_atomic_pk_add_f16 %0, %1, %2" ::"v"(lane_off), "v"(v), "s"(base) : "memory");
+    }
 };
+// the same for one fp32 value, `offset` bytes behind the lane's address
+__device__ __forceinline__ void add_f32_to_memory(uint32_t lane_off, float v, void* base, int offset)
+{
+    asm volatile("global_atomic_add_f32 %0, %1, %2 offset:%3" ::"v"(lane_off), "v"(v), "s"(base), "i"(offset) : "memory");
+}
 
 // A column = two 512-element tiles.  Stage 1 as in tile_transform; stage 2 contracts the two
 // tiles' stage-1 results together (K = 32: 16 stage-2 inputs of each tile) against [G2; +G2] and

@@ -104,13 +104,14 @@ def test_gemm_against_oracle(pkg, oracle, M, N, K, dt, tol):
         assert _rel(oracle, C16, want) <= tol
 
 
-# K = 512, 1024 and 2048 run the register-resident kernels (K = 2048 its own, with K split over
-# wavefront pairs): groups of 131072 / K columns, 64-row blocks, results stored while the next row
-# block is multiplied or (K = 512) right after it.
+# K = 512 ... 4096 run the register-resident kernels (K = 2048 its own, with K split over wavefront
+# pairs; K = 4096 the same kernel in two passes, the second adding to what the first stored): groups
+# of 131072 / K columns (64 at K = 4096), 64-row blocks, results stored while the next row block is
+# multiplied or (K = 512) right after it.
 # Shapes around every tile boundary, a single row block, N not a multiple of the columns a lane
 # stores together (no vector stores), a scale that is not a power of two (separate store path),
 # both 16-bit types and both output types.
-@pytest.mark.parametrize("K", [1024, 512, 2048])
+@pytest.mark.parametrize("K", [1024, 512, 2048, 4096])
 @pytest.mark.parametrize("M,N", [(1, 1), (63, 127), (64, 128), (65, 129), (128, 256), (129, 257),
                                  (577, 1333), (130, 2000), (4096, 130), (700, 4095), (200, 514)])
 def test_gemm_k1024_tile_boundaries(pkg, oracle, M, N, K):
@@ -131,12 +132,12 @@ def test_gemm_k1024_tile_boundaries(pkg, oracle, M, N, K):
             assert err <= 2e-2, (M, N, K, dt, scale, od)
 
 
-@pytest.mark.parametrize("K", [1024, 512, 2048])
+@pytest.mark.parametrize("K", [1024, 512, 2048, 4096])
 def test_gemm_k1024_every_output_written_once(pkg, oracle, K):
     # size-independent check on the full benchmark shape, both output types: C against the
     # unfused product computed on the device from the library's own transform, every element
     M = N = 4096
-    s2 = {512: 1.0 / 16.0, 1024: 1.0 / 32.0, 2048: 1.0 / 32.0}[K]   # a power of two
+    s2 = {512: 1.0 / 16.0, 1024: 1.0 / 32.0, 2048: 1.0 / 32.0, 4096: 1.0 / 64.0}[K]   # a power of two
     W, Xt = oracle.inputs_gemm(M, N, K, torch.bfloat16)
     Wd, Xd = W.cuda(), Xt.cuda()
     Y = pkg.hadamard_transform(Xd, s2)                  # bf16, same rounding as the fused operand
@@ -154,11 +155,11 @@ def test_gemm_k1024_every_output_written_once(pkg, oracle, K):
 # evenly (workgroup ids without work), M slices that are not a power of two, more than one round of
 # workgroups, a ragged last slice and last column group.  Every element against the unfused
 # product computed on the device from the library's own transform.
-@pytest.mark.parametrize("K", [1024, 512, 2048])
+@pytest.mark.parametrize("K", [1024, 512, 2048, 4096])
 @pytest.mark.parametrize("M,N", [(5000, 3000), (6144, 6144), (2048, 8192), (12288, 1536), (1000, 9000)])
 def test_gemm_k1024_launch_plans(pkg, oracle, M, N, K):
     g = torch.Generator(device="cuda").manual_seed(M + N)
-    s2 = {512: 1.0 / 16.0, 1024: 1.0 / 32.0, 2048: 1.0 / 32.0}[K]   # a power of two
+    s2 = {512: 1.0 / 16.0, 1024: 1.0 / 32.0, 2048: 1.0 / 32.0, 4096: 1.0 / 64.0}[K]   # a power of two
     Wd = torch.randn(M, K, generator=g, device="cuda").to(torch.bfloat16)
     Xd = torch.randn(N, K, generator=g, device="cuda").to(torch.bfloat16)
     Y = pkg.hadamard_transform(Xd, s2)
@@ -312,3 +313,24 @@ def test_gemm_f32_k4096_does_not_depend_on_what_c_held(pkg, oracle):
         torch.cuda.synchronize()
         want = oracle.fused_ht_gemm_f64_blas(W.double().numpy(), Xt.double().numpy(), 1.0 / 64.0)
         assert _rel(oracle, C, want) <= 1e-5
+
+
+def test_gemm16_k4096_does_not_depend_on_what_c_held(pkg, oracle):
+    # the same for 16-bit inputs (two passes of the split-K kernel, the second adding in the L2), all
+    # four type combinations, shapes with and without edge blocks, twice in a row into the same C
+    import importlib
+    lib = importlib.import_module("6s894_project_2025_amd._lib")
+    K = 4096
+    for dt, code in ((torch.bfloat16, lib.MI_BF16), (torch.float16, lib.MI_F16)):
+        for M, N in ((200, 70), (128, 64), (640, 256)):
+            W, Xt = oracle.inputs_gemm(M, N, K, dt)
+            Wd, Xd = W.cuda(), Xt.cuda()
+            want = oracle.fused_ht_gemm_f64_blas(W.double().numpy(), Xt.double().numpy(), 1.0 / 64.0)
+            for od, ocode in ((torch.float32, lib.MI_F32), (dt, code)):
+                C = torch.full((M, N), float("nan"), device="cuda", dtype=od)
+                for _ in range(2):
+                    st = lib.load().mi_fused_ht_gemm(Wd.data_ptr(), Xd.data_ptr(), C.data_ptr(), M, N, K, code,
+                                                     ocode, 1.0 / 64.0, torch.cuda.current_stream().cuda_stream)
+                    assert st == 0
+                torch.cuda.synchronize()
+                assert _rel(oracle, C, want) <= 2e-2, (dt, od, M, N)
