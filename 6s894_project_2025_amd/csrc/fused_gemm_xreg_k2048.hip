@@ -1,5 +1,6 @@
 // Fused Hadamard -> GEMM with the transformed operand held in registers, gfx950, 16-bit inputs,
-// K = 2048, with the K range split over pairs of wavefronts:
+// K = 2048 (and K = 4096 as two passes over 2048 k each, the second adding to what the first
+// stored), with the K range split over pairs of wavefronts:
 //     C[M,N] = W[M,K] * (scale * H_K * X[K,N]),  X given as Xt[N,K].
 //
 // A wavefront's 256 accumulation registers hold 32768 16-bit values.  With all of K = 2048 per
@@ -12,7 +13,8 @@
 // stages (64 rows x 128 k; a stage is four K steps); a wavefront reads the fragments of its own
 // stream only.  At the end of a row block each wavefront of a pair hands the partner the
 // accumulators of two of the four 16-row fragments through LDS and finishes (adds, stores) the
-// other two, always as (k < 1024) + (k >= 1024).
+// other two (a sum of two terms: the result does not depend on who adds); that meeting is hidden
+// behind the MFMAs of the next row block.
 // The prologue is shared inside a pair: in each of four rounds the pair transforms eight columns of
 // its set, all of K (four columns per wavefront), and writes both halves into the pair's LDS area;
 // after a barrier each wavefront reads its own half of the eight columns in operand order (the half

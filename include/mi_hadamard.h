@@ -93,8 +93,8 @@ int mi_fused_ht_gemv(const void* W, const void* X, void* Y, uint32_t M, uint32_t
  *   in_dtype  : MI_F32 (fp32 MFMA) or MI_BF16 / MI_F16 (16-bit MFMA, fp32 accumulate).
  *   out_dtype : MI_F32, or the same 16-bit type as in_dtype.
  *   K : power of two, 32 <= K <= 4096.   M, N >= 1 (edge tiles are masked).
- * MI_F32 with K = 4096 enqueues two kernels on `stream` (the second adds to what the first stored
- * in C); every other case is one kernel.
+ * K = 4096 enqueues two kernels on `stream` for every dtype (the second adds to what the first
+ * stored in C, so nothing else may touch C between them); every other case is one kernel.
  */
 int mi_fused_ht_gemm(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
                      int in_dtype, int out_dtype, float scale, void* stream);
