@@ -220,9 +220,11 @@ def main() -> int:
         return 0
 
     # ---- the same kernel at other sizes: larger N and M amortise the prologue, K = 512 halves the LDS
-    # traffic per flop (bf16, fused / vendor GEMM without transform / transform + vendor GEMM) ---------
+    # traffic per flop; K = 2048 and 4096 run the kernel that splits K over wavefront pairs (bf16,
+    # fused / vendor GEMM without transform / transform + vendor GEMM) --------------------------------
     if not only:
-        for (Kx, Mx, Nx) in ((1024, 8192, 8192), (512, 4096, 4096), (512, 8192, 8192)):
+        for (Kx, Mx, Nx) in ((1024, 8192, 8192), (512, 4096, 4096), (512, 8192, 8192),
+                             (2048, 2048, 2048), (2048, 4096, 4096), (4096, 2048, 2048), (4096, 4096, 4096)):
             Wx = torch.randn(Mx, Kx, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(dev)
             Xx = torch.randn(Nx, Kx, generator=torch.Generator().manual_seed(0)).to(torch.bfloat16).to(dev)
             fx = 2 * Mx * Nx * Kx
