@@ -93,6 +93,8 @@ int mi_fused_ht_gemv(const void* W, const void* X, void* Y, uint32_t M, uint32_t
  *   in_dtype  : MI_F32 (fp32 MFMA) or MI_BF16 / MI_F16 (16-bit MFMA, fp32 accumulate).
  *   out_dtype : MI_F32, or the same 16-bit type as in_dtype.
  *   K : power of two, 32 <= K <= 4096.   M, N >= 1 (edge tiles are masked).
+ *   The register-resident kernels (16-bit inputs with K >= 512, MI_F32 with K >= 256) address W
+ *   with 32-bit byte offsets: W larger than 4 GiB, or N >= 2^24, is MI_ERR_SHAPE.
  * K = 4096 enqueues two kernels on `stream` for every dtype (the second adds to what the first
  * stored in C, so nothing else may touch C between them); every other case is one kernel.
  */

@@ -58,6 +58,11 @@ def test_argument_validation_happens_before_any_launch(libmod):
     assert lib.mi_fused_ht_gemm(buf, buf, buf, 4, 4, 48, 1, 1, 1.0, None) == MI_ERR_SIZE
     assert lib.mi_fused_ht_gemm(buf, buf, buf, 4, 4, 64, 1, 2, 1.0, None) == MI_ERR_DTYPE
     assert lib.mi_fused_ht_gemm(buf, None, buf, 4, 4, 64, 1, 1, 1.0, None) == MI_ERR_NULL
+    # the register-resident kernels address W with 32-bit byte offsets: more than 4 GiB of W is refused
+    assert lib.mi_fused_ht_gemm(buf, buf, buf, 1 << 22, 64, 1024, 1, 1, 1.0, None) == MI_ERR_SHAPE
+    assert lib.mi_fused_ht_gemm(buf, buf, buf, 1 << 20, 64, 4096, 1, 1, 1.0, None) == MI_ERR_SHAPE
+    assert lib.mi_fused_ht_gemm(buf, buf, buf, 1 << 21, 64, 2048, 2, 0, 1.0, None) == MI_ERR_SHAPE
+    assert lib.mi_fused_ht_gemm(buf, buf, buf, 1 << 20, 64, 1024, 0, 0, 1.0, None) == MI_ERR_SHAPE
     assert lib.mi_rht_quant_fp8(buf, buf, buf, buf, None, 4, 24, 1.0, None) == MI_ERR_SIZE
     assert lib.mi_rht_quant_fp8(buf, buf, buf, None, None, 4, 64, 1.0, None) == MI_ERR_NULL
     assert lib.mi_fp8_gemm_rowscale(buf, buf, buf, buf, buf, 4, 4, 100, None) == MI_ERR_SHAPE
