@@ -48,10 +48,98 @@ PER_FILE_FLAGS = {
 # before each use - while the previous MFMA may still be reading that register, which silently
 # corrupts results.  The build therefore looks at the generated ISA of these files and fails when an
 # accumulation register is written anywhere after a kernel's first such MFMA.
+#
+# The compiler does not know either that the result of such an MFMA arrives when the instruction
+# retires: an ordinary instruction that touches the destination registers too soon (a register copy
+# the allocator puts on a loop edge, say) would see the old value, where for its own MFMAs the
+# compiler inserts the wait states.  The build fails when anything but another MFMA reads an
+# assembly MFMA's destination within kResultWaitStates issue slots on any path.
 ISA_CHECKED = {"fused_gemm_xreg.hip", "fused_gemm_xreg_f32.hip", "fused_gemm_xreg_k2048.hip"}
 _MFMA_B_IN_AGPR = re.compile(r"^\s*v_mfma_\S+\s+v\[[0-9:]+\], v\S+, a")
 _AGPR_WRITE = re.compile(r"^\s*v_accvgpr_(write|mov)")
 _LABEL = re.compile(r"^([A-Za-z_][\w$]*):")
+_ANY_LABEL = re.compile(r"^([.A-Za-z_][\w$.]*):")
+_VREG_RANGE = re.compile(r"\bv\[(\d+):(\d+)\]")
+_VREG = re.compile(r"\bv(\d+)\b")
+kResultWaitStates = 11  # an eight-pass MFMA (16x16x32 16-bit, 16x16x4 fp32): passes + 3
+
+
+def _vregs(text: str) -> set:
+    regs = set()
+    for m in _VREG_RANGE.finditer(text):
+        regs.update(range(int(m.group(1)), int(m.group(2)) + 1))
+    for m in _VREG.finditer(text):
+        regs.add(int(m.group(1)))
+    return regs
+
+
+_NO_DESTINATION = ("ds_write", "ds_store", "global_store", "global_atomic", "global_load_lds", "scratch_store",
+                   "buffer_store", "flat_store")
+
+
+def _source_operands(text: str) -> str:
+    """The operands an instruction reads: all but the first, or all for stores and their like."""
+    op, _, rest = text.partition(" ")
+    if op.startswith(_NO_DESTINATION):
+        return rest
+    return rest.partition(",")[2]
+
+
+def check_mfma_results_not_touched_early(asm_text: str, where: str) -> int:
+    """Raises if a non-MFMA instruction reads the destination of an assembly MFMA (one whose B
+    operand is an accumulation register) within kResultWaitStates issue slots, on any path the
+    branches allow; returns the number of MFMAs checked.  (Writes are left alone: branch conditions
+    are not evaluated, and on the impossible path from a block whose result awaits its stores into a
+    block variant that has none to do, the allocator rightly reuses those registers.)"""
+    checked = 0
+    lines = asm_text.splitlines()
+    i = 0
+    while i < len(lines):
+        label = _LABEL.match(lines[i])
+        if not label:
+            i += 1
+            continue
+        name = label.group(1)
+        # one function: instructions and the positions of its local labels
+        ins, labels = [], {}
+        i += 1
+        while i < len(lines) and not _LABEL.match(lines[i]):
+            text = lines[i].split(";")[0].strip()
+            local = _ANY_LABEL.match(text)
+            if local:
+                labels[local.group(1)] = len(ins)
+            elif text and not text.startswith("."):
+                ins.append(text)
+            i += 1
+        for at, text in enumerate(ins):
+            if not _MFMA_B_IN_AGPR.match(text):
+                continue
+            checked += 1
+            seen = set()
+            todo = [(at + 1, kResultWaitStates, frozenset(_vregs(text.split(",")[0])))]
+            while todo:
+                k, left, pending = todo.pop()
+                while left > 0 and pending and k < len(ins) and (k, left, pending) not in seen:
+                    seen.add((k, left, pending))
+                    t = ins[k]
+                    op = t.split()[0]
+                    if op == "s_endpgm":
+                        break
+                    if not op.startswith("v_mfma"):
+                        if _vregs(_source_operands(t)) & pending:
+                            raise RuntimeError(f"{where}: {name}: `{t}` reads the result of `{text}` "
+                                               f"{kResultWaitStates - left} issue slots after it")
+                        if not op.startswith(_NO_DESTINATION):  # a register written anew is no longer that result
+                            pending = pending - _vregs(t.partition(",")[0])
+                    if op == "s_branch":
+                        k = labels.get(t.split()[1], len(ins))
+                        left -= 1
+                        continue
+                    if op.startswith("s_cbranch"):
+                        todo.append((labels.get(t.split()[1], len(ins)), left - 1, pending))
+                    left -= int(t.split()[1], 0) + 1 if op == "s_nop" else 1
+                    k += 1
+    return checked
 
 
 def check_register_resident_isa(asm_text: str, where: str) -> int:
@@ -106,8 +194,8 @@ def _compile(src: str) -> str:
         if len(isa) != 1:
             raise RuntimeError(f"no device assembly found for {src}")
         with open(isa[0]) as f:
-            n = check_register_resident_isa(f.read(), base)
-        if n == 0:
+            text = f.read()
+        if check_register_resident_isa(text, base) == 0 or check_mfma_results_not_touched_early(text, base) == 0:
             raise RuntimeError(f"{base}: no register-resident MFMA loop found in the device assembly")
         for t in temps:
             os.remove(t)

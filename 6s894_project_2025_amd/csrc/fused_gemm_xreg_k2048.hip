@@ -384,13 +384,15 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
                 }
             }
         }
-        // the last MFMAs retire before anything else touches their accumulators
-        drain_mfma(acc[cur]);
+        // (Nothing here reads the accumulators: the next block's K step 0 hands them over behind its
+        // fourth MFMA at the earliest, long after the last MFMA above has retired.  The build checks
+        // the generated code for copies the register allocator might put on the loop edge.)
     };
     // the same meeting of the halves with nothing to hide it behind: the last block of a workgroup,
     // and blocks whose stores need bounds checks
     auto meet_now = [&](auto set_tag) __attribute__((always_inline)) {
         constexpr int cur = decltype(set_tag)::value;
+        drain_mfma(acc[cur]);  // the last MFMAs retire before their accumulators are read
 #pragma unroll
         for (int i = 0; i < 4; ++i) lds_write16(xb_mine, acc[cur][2 + (i >> 1)][i & 1], i * 1024);
         wait_lds();

@@ -194,3 +194,36 @@ _Zplain: ; @_Zplain
     with pytest.raises(RuntimeError, match="_Zkernel_a writes an accumulation register"):
         build.check_register_resident_isa(bad, "bad")
     assert set(build.ISA_CHECKED) <= {os.path.basename(s) for s in build.sources()}
+
+
+def test_build_rejects_early_reads_of_an_assembly_mfma_result():
+    """The compiler does not know that the result of an inline-assembly MFMA arrives when it retires:
+    the build follows every path from such an MFMA for a few issue slots and fails on an ordinary
+    instruction that reads its destination there (a copy on a loop edge, say)."""
+    import importlib
+    build = importlib.import_module("6s894_project_2025_amd.build")
+    head = "_Zk: ; @_Zk\n.LBB0_1:\n\tv_mfma_f32_16x16x32_bf16 v[32:35], v[96:99], a[124:127], v[32:35]\n"
+    tail = "\ts_endpgm\n"
+    filler = "\tv_add_u32_e32 v1, v2, v3\n"
+
+    def check(body):
+        return build.check_mfma_results_not_touched_early(head + body + tail, "t")
+
+    # far enough away, behind enough idle cycles, or another MFMA accumulating into it: fine
+    assert check(filler * build.kResultWaitStates + "\tv_mov_b32_e32 v100, v33\n") == 1
+    assert check("\ts_nop 15\n\tv_mov_b32_e32 v100, v33\n") == 1
+    assert check("\tv_mfma_f32_16x16x32_bf16 v[32:35], v[96:99], a[128:131], v[32:35]\n" + filler * 11) == 2
+    # a register written anew is no longer the result; stores and LDS writes have no destination
+    assert check("\tv_xor_b32 v32, 0x80, v180\n\tds_read_b128 v[64:67], v32 offset:0\n") == 1
+    with pytest.raises(RuntimeError, match="reads the result"):
+        check(filler * 3 + "\tv_mov_b64_e32 v[114:115], v[34:35]\n")
+    with pytest.raises(RuntimeError, match="reads the result"):
+        check("\tds_write_b128 v7, v[32:35] offset:1024\n")
+    with pytest.raises(RuntimeError, match="reads the result"):
+        check("\tglobal_store_dword v5, v33, s[2:3] nt\n")
+    # branches are followed both ways
+    with pytest.raises(RuntimeError, match="reads the result"):
+        check("\ts_cbranch_vccnz .LBB0_9\n" + filler * 20 + ".LBB0_9:\n\tv_cvt_pk_bf16_f32 v9, v32, v33\n")
+    with pytest.raises(RuntimeError, match="reads the result"):
+        check("\ts_branch .LBB0_9\n" + "\ts_endpgm\n" + ".LBB0_9:\n\tv_cvt_pk_bf16_f32 v9, v32, v33\n")
+    assert check("\ts_cbranch_vccnz .LBB0_9\n" + filler * 20 + ".LBB0_9:\n" + filler * 11 + "\tv_mov_b32_e32 v9, v32\n") == 1
