@@ -95,16 +95,19 @@ int launch_reg(const void* in, void* out, uint64_t total, uint64_t num_steps, ui
                OutputScale os, hipStream_t s)
 {
     if (num_steps == 0) return MI_OK;
-    // Up to four steps per wavefront once every compute unit has a full set of wavefronts: the
+    // Up to three steps per wavefront once the chip is filled one and a half times over: the
     // operand set-up is paid once and the next row's loads overlap the current row's arithmetic.
+    // (Exactly filled, with the same number of steps for everybody, all wavefronts load, compute
+    // and store in phase: 4096 wavefronts of four steps each measured 1 - 2 % slower at
+    // [16384, 4096] and [32768, 2048] than 6144 and 10923 wavefronts.)
     // Beyond the 256 MiB Infinity Cache the transform is DRAM-bound, and there one step per
     // (short-lived) wavefront measured 2 - 4 % faster (the sweep through memory stays in order)
     // and non-temporal loads and stores another 5 - 13 % (lines that are never touched again
     // stay out of the caches).
     const bool big = total * (uint64_t)IO::ESIZE > (256ull << 20);
     uint64_t waves = num_steps;
-    const uint64_t resident = 256u * 16u;
-    const uint64_t per_wave = big ? 1u : 4u;
+    const uint64_t resident = 256u * 24u;
+    const uint64_t per_wave = big ? 1u : 3u;
     if (waves > resident)
         waves = (num_steps + per_wave - 1u) / per_wave > resident ? (num_steps + per_wave - 1u) / per_wave
                                                                   : resident;
