@@ -306,7 +306,7 @@ def main() -> int:
         xa = xa.to(torch.bfloat16).to(dev)
         sign = (1 - 2 * torch.randint(0, 2, (nq,), generator=torch.Generator().manual_seed(2))
                 ).to(torch.int8).to(dev)
-        ms, _ = events_ms(lambda: hada.rht_quant_fp8(xa, sign), 50, 3)
+        ms, _ = steady_ms(lambda: hada.rht_quant_fp8(xa, sign), 50)
         qbytes = T * nq * 3 + T * 4
         others["rht_quant_fp8_8192x4096"] = {
             "us": round(ms * 1e3, 2), "algorithmic_bytes": qbytes,
