@@ -114,7 +114,7 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
     using E = typename T16::E;
     using V8 = typename T16::V8;
     typedef E V2 __attribute__((ext_vector_type(2)));
-    static_assert(KTOT == 2048 || (KTOT == 4096), "K = 2048, or one half of K = 4096");
+    static_assert(KTOT == 2048 || KTOT == 4096, "K = 2048, or one half of K = 4096");
     static_assert(KTOT == 4096 || !ACCUM, "a single pass stores");
     constexpr int K = KTOT, NBF = 2, NM = 8;  // K: row length of W and Xt
     constexpr int SPB = k2h::SPB, AHEAD = k2h::AHEAD, KSTEPS = k2h::KSTEPS;
@@ -315,6 +315,12 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
             } else {
                 XMfma<T16>::add_pair_to_memory(lane_off, __builtin_bit_cast(uint32_t, V2{(E)v0, (E)v1}), row_ptr);
             }
+        } else if (KTOT == 4096) {
+            // the second pass reads these lines back: no streaming hint (M = N = 8192: 510 -> 485 us)
+            if (OUT_F32)
+                cached_store8(lane_off, u32x2{__float_as_uint(v0), __float_as_uint(v1)}, row_ptr);
+            else
+                cached_store4(lane_off, __builtin_bit_cast(uint32_t, V2{(E)v0, (E)v1}), row_ptr);
         } else if (OUT_F32) {
             stream_store8(lane_off, u32x2{__float_as_uint(v0), __float_as_uint(v1)}, row_ptr);
         } else {

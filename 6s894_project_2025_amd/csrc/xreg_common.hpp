@@ -170,6 +170,15 @@ __device__ __forceinline__ void stream_store8(uint32_t lane_off, u32x2 v, void* 
 {
     asm volatile("global_store_dwordx2 %0, %1, %2 nt" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
 }
+// the same without the streaming hint, for results that are read again soon
+__device__ __forceinline__ void cached_store4(uint32_t lane_off, uint32_t v, void* base)
+{
+    asm volatile("global_store_dword %0, %1, %2" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
+}
+__device__ __forceinline__ void cached_store8(uint32_t lane_off, u32x2 v, void* base)
+{
+    asm volatile("global_store_dwordx2 %0, %1, %2" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
+}
 // (A store of more than 8 bytes still reads its data registers during the next cycles; the compiler
 // keeps ordinary code away from them for that long, but does not know what this statement is.)
 __device__ __forceinline__ void stream_store16(uint32_t lane_off, u32x4 v, void* base)
