@@ -482,12 +482,11 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
 }
 
 template <class T16, int K, bool OUT_F32>
-int launch_as(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, float scale,
-              uint32_t mpx, hipStream_t s)
+int launch_as(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, float scale, hipStream_t s)
 {
     const OutputScale os =
         split_output_scale((double)scale, tile_stage_shift<2>(ilog2((uint32_t)K), kNarrowRange<T16>));
-    const Plan p = plan(M, N, Geom<K>::COLS, mpx);
+    const Plan p = plan16(M, N, (uint32_t)K);
     auto kern = fused_ht_gemm_xreg_kernel<T16, K, OUT_F32>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess)
@@ -501,10 +500,10 @@ int launch_as(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, fl
 
 template <class T16, int K>
 int launch(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, int out_f32, float scale,
-           uint32_t mpx, hipStream_t s)
+           hipStream_t s)
 {
-    return out_f32 ? launch_as<T16, K, true>(W, Xt, C, M, N, scale, mpx, s)
-                   : launch_as<T16, K, false>(W, Xt, C, M, N, scale, mpx, s);
+    return out_f32 ? launch_as<T16, K, true>(W, Xt, C, M, N, scale, s)
+                   : launch_as<T16, K, false>(W, Xt, C, M, N, scale, s);
 }
 
 }  // namespace xreg
@@ -522,11 +521,11 @@ int fused_gemm16_xreg(const void* W, const void* Xt, void* C, uint32_t M, uint32
     if ((uint64_t)M * K * 2u > 0xffffffffull || (uint64_t)N * 4u * 64u > 0xffffffffull)
         return MI_ERR_SHAPE;
     if (K == 1024u) {
-        if (in_dtype == MI_BF16) return xreg::launch<BF16, 1024>(W, Xt, C, M, N, out_f32, scale, 8u, s);
-        if (in_dtype == MI_F16) return xreg::launch<F16, 1024>(W, Xt, C, M, N, out_f32, scale, 8u, s);
+        if (in_dtype == MI_BF16) return xreg::launch<BF16, 1024>(W, Xt, C, M, N, out_f32, scale, s);
+        if (in_dtype == MI_F16) return xreg::launch<F16, 1024>(W, Xt, C, M, N, out_f32, scale, s);
     } else if (K == 512u) {
-        if (in_dtype == MI_BF16) return xreg::launch<BF16, 512>(W, Xt, C, M, N, out_f32, scale, 8u, s);
-        if (in_dtype == MI_F16) return xreg::launch<F16, 512>(W, Xt, C, M, N, out_f32, scale, 8u, s);
+        if (in_dtype == MI_BF16) return xreg::launch<BF16, 512>(W, Xt, C, M, N, out_f32, scale, s);
+        if (in_dtype == MI_F16) return xreg::launch<F16, 512>(W, Xt, C, M, N, out_f32, scale, s);
     } else if (K == 2048u || K == 4096u) {
         return fused_gemm16_xreg_k2048(W, Xt, C, M, N, K, in_dtype, out_f32, scale, s);
     } else {
@@ -543,8 +542,8 @@ extern "C" int mi_debug_fused_gemm_tiling(uint32_t M, uint32_t N, uint32_t K, ui
     using namespace mi;
     if (!header) return MI_ERR_NULL;
     if (M == 0 || N == 0) return MI_ERR_SHAPE;
-    if (K != 512u && K != 1024u && K != 2048u) return MI_ERR_SIZE;
-    const xreg::Plan p = xreg::plan(M, N, 131072u / K, 8u);
+    if (K != 512u && K != 1024u && K != 2048u && K != 4096u) return MI_ERR_SIZE;
+    const xreg::Plan p = xreg::plan16(M, N, K);
     const uint32_t h[8] = {p.ngroups, p.msplit, p.m_per_block, p.mpx, p.cgx, p.nrect, p.grid, 0u};
     for (int i = 0; i < 8; ++i) header[i] = h[i];
     if (!tiles) return MI_OK;

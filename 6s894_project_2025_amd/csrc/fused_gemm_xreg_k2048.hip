@@ -489,9 +489,8 @@ int launch_ksplit16(const void* W, const void* Xt, void* C, uint32_t M, uint32_t
                     hipStream_t s)
 {
     const OutputScale os = split_output_scale((double)scale, tile_stage_shift<2>(11u, kNarrowRange<T16>));
-    if (K == 2048u) return launch_pass<T16, OUT_F32, 2048, false>(W, Xt, C, M, N, plan(M, N, 64u, 8u), os, s);
-    // K = 4096: a workgroup transforms twice as much per column as at K = 2048 for the same main loop
-    const Plan p = plan(M, N, 64u, 8u, 18u, 4u);
+    const Plan p = plan16(M, N, K);
+    if (K == 2048u) return launch_pass<T16, OUT_F32, 2048, false>(W, Xt, C, M, N, p, os, s);
     const int rc = launch_pass<T16, OUT_F32, 4096, false>(W, Xt, C, M, N, p, os, s);
     if (rc != MI_OK) return rc;
     return launch_pass<T16, OUT_F32, 4096, true>(W, Xt, C, M, N, p, os, s);

@@ -265,5 +265,13 @@ inline Plan plan(uint32_t M, uint32_t N, uint32_t cols, uint32_t mpx_max, uint32
     return p;
 }
 
+// The plan of the 16-bit kernels by K: 131072 / K columns per workgroup (64 at K = 4096, whose two
+// passes each transform twice as much per column as the K = 2048 kernel does for the same main loop).
+inline Plan plan16(uint32_t M, uint32_t N, uint32_t K)
+{
+    if (K == 4096u) return plan(M, N, 64u, 8u, 18u, 4u);
+    return plan(M, N, 131072u / K, 8u);
+}
+
 }  // namespace xreg
 }  // namespace mi

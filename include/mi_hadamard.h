@@ -173,12 +173,12 @@ int mi_debug_mfma_rate(int shape, int lds_reads, uint32_t waves_per_simd, uint32
                        const void* operands, uint64_t* cycles, void* stream);
 
 /*
- * Host-only: how mi_fused_ht_gemm cuts a 16-bit problem with K = 512, 1024 or 2048 into workgroups (no
+ * Host-only: how mi_fused_ht_gemm cuts a 16-bit problem with K = 512 ... 4096 into workgroups (no
  * GPU call; MI_ERR_SIZE for any other K).
  * The (column group, M slice) grid, the XCD rectangles and the map from workgroup id to tile are
  * what decides L2 reuse and the number of launch rounds; this hook lets a test check on the CPU
  * that every tile is handled by exactly one workgroup.  No counterpart in the reference.
- *   header[8] : ngroups (groups of 131072 / K columns), msplit (M slices), m_per_block (rows per slice),
+ *   header[8] : ngroups (groups of 131072 / K columns, 64 at K = 4096), msplit (M slices), m_per_block (rows per slice),
  *               mpx, cgx (rectangle extents in M slices and column groups), nrect, grid
  *               (workgroups launched), 0
  *   tiles     : NULL, or 2 * capacity uint32: for workgroup id i, tiles[2i] = column group and

@@ -124,9 +124,9 @@ def test_fused_gemm_tiling_covers_every_tile_exactly_once(libmod):
               (2048, 8192), (8192, 2048), (4096, 16384), (16384, 4096), (700, 4095), (130, 2000),
               (4096, 130), (100000, 128), (64, 100000), (9999, 7777), (8192, 8192), (3968, 31 * 128)]
     for M, N, K in [(m, n, 1024) for m, n in shapes] + [(m, n, 512) for m, n in shapes[:12]] + \
-            [(m, n, 2048) for m, n in shapes[:12]]:
+            [(m, n, 2048) for m, n in shapes[:12]] + [(m, n, 4096) for m, n in shapes[:12]]:
         p, tiles = _tiling(lib, M, N, K)
-        assert p["ngroups"] == -(-N // (131072 // K))
+        assert p["ngroups"] == -(-N // max(64, 131072 // K))
         assert p["m_per_block"] % 64 == 0 and p["msplit"] == -(-M // p["m_per_block"])
         assert (p["msplit"] - 1) * p["m_per_block"] < M          # no empty slice
         real = [t for t in tiles if t != (0xFFFFFFFF, 0xFFFFFFFF)]
@@ -163,7 +163,7 @@ def test_fused_gemm_tiling_avoids_a_nearly_empty_last_round(libmod):
     assert p["ngroups"] * p["msplit"] <= 256
     # other K: rejected before anything else
     import ctypes
-    assert lib.mi_debug_fused_gemm_tiling(64, 64, 4096, (ctypes.c_uint32 * 8)(), None, 0) != 0
+    assert lib.mi_debug_fused_gemm_tiling(64, 64, 256, (ctypes.c_uint32 * 8)(), None, 0) != 0
 
 
 def test_build_rejects_accumulation_register_writes_inside_an_mfma_loop():
