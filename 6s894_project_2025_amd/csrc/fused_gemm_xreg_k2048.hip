@@ -196,34 +196,22 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
                 // pass keeps, [quarter][4 h .. 4 h + 3]
                 f32x4 qv[4][2];
                 {
+                    // A, B: the 1024-point transforms of the two halves of the 2048 values this pass
+                    // keeps (K = 4096: of x[0:2048] +- x[2048:4096], H_2048 being linear)
                     f32x4 sa[2], da[2], sb[2], db[2];
-                    column_pair_f32<T16>(in[e][0], in[e][1], po, sa, da);
-                    column_pair_f32<T16>(in[e][2], in[e][3], po, sb, db);
+                    if constexpr (KTOT == 4096) {
+                        column_pair_combined_f32<T16, ACCUM>(in[e][0], in[e][1], in[e][4], in[e][5], po, sa, da);
+                        column_pair_combined_f32<T16, ACCUM>(in[e][2], in[e][3], in[e][6], in[e][7], po, sb, db);
+                    } else {
+                        column_pair_f32<T16>(in[e][0], in[e][1], po, sa, da);
+                        column_pair_f32<T16>(in[e][2], in[e][3], po, sb, db);
+                    }
 #pragma unroll
                     for (int h = 0; h < 2; ++h) {  // A_lo + B_lo, A_hi + B_hi, A_lo - B_lo, A_hi - B_hi
                         qv[0][h] = sa[h] + sb[h];
                         qv[1][h] = da[h] + db[h];
                         qv[2][h] = sa[h] - sb[h];
                         qv[3][h] = da[h] - db[h];
-                    }
-                }
-                if constexpr (KTOT == 4096) {  // the same of the column's second half, added or subtracted
-                    f32x4 sa[2], da[2], sb[2], db[2];
-                    column_pair_f32<T16>(in[e][4], in[e][5], po, sa, da);
-                    column_pair_f32<T16>(in[e][6], in[e][7], po, sb, db);
-#pragma unroll
-                    for (int h = 0; h < 2; ++h) {
-                        if (ACCUM) {
-                            qv[0][h] -= sa[h] + sb[h];
-                            qv[1][h] -= da[h] + db[h];
-                            qv[2][h] -= sa[h] - sb[h];
-                            qv[3][h] -= da[h] - db[h];
-                        } else {
-                            qv[0][h] += sa[h] + sb[h];
-                            qv[1][h] += da[h] + db[h];
-                            qv[2][h] += sa[h] - sb[h];
-                            qv[3][h] += da[h] - db[h];
-                        }
                     }
                 }
                 if (c + kAhead < 16) load_col(c + kAhead);

@@ -131,5 +131,35 @@ __device__ __forceinline__ void column_pair_f32(typename T16::V8 t0, typename T1
     }
 }
 
+// The same for the sum (NEGATE = false) or difference (true) of two 1024-element columns, formed in
+// the accumulators of stage 1 (which is linear), so that the 16-bit value between the stages is
+// rounded once and stage 2 runs once: s, d = halves of H_1024 (x +- y), x = [t0; t1], y = [u0; u1].
+template <class T16, bool NEGATE>
+__device__ __forceinline__ void column_pair_combined_f32(typename T16::V8 t0, typename T16::V8 t1,
+                                                         typename T16::V8 u0, typename T16::V8 u1,
+                                                         const PairOperands<T16>& po, f32x4 (&s)[2],
+                                                         f32x4 (&d)[2])
+{
+    using E = typename T16::E;
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        // (sign bits flipped: exact for either 16-bit type)
+        const u32x4 flip = {0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
+        const typename T16::V8 g1y =
+            NEGATE ? __builtin_bit_cast(typename T16::V8, __builtin_bit_cast(u32x4, po.g1[h]) ^ flip) : po.g1[h];
+        const f32x4 d0 = T16::mfma32(u0, g1y, T16::mfma32(t0, po.g1[h], zero));
+        const f32x4 d1 = T16::mfma32(u1, g1y, T16::mfma32(t1, po.g1[h], zero));
+        typename T16::V8 a2;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            a2[r] = (E)d0[r];
+            a2[4 + r] = (E)d1[r];
+        }
+        s[h] = T16::mfma32(a2, po.g2s, zero);
+        d[h] = T16::mfma32(a2, po.g2d, zero);
+    }
+}
+
 }  // namespace xreg
 }  // namespace mi

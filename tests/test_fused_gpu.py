@@ -148,7 +148,11 @@ def test_gemm_k1024_every_output_written_once(pkg, oracle, K):
             C = pkg.fused_ht_gemm(Wd, Xd, s2, out_dtype=od)
         torch.cuda.synchronize()
         err = (C.float() - ref).abs().max().item() / scale
-        assert err <= (8e-3 if od == torch.bfloat16 else 2e-3), (od, err)
+        # K = 4096 forms x[0:2048] +- x[2048:4096] inside the first matrix-core stage, so its 16-bit
+        # operand is rounded at other places than the stand-alone transform's (as close to the
+        # exact product, which the oracle checks measure, but not the same bits)
+        tol32 = 4e-3 if K == 4096 else 2e-3
+        assert err <= (8e-3 if od == torch.bfloat16 else tol32), (od, err)
 
 
 # Shapes whose launch plan differs from the benchmark's: rectangles that do not fill all eight XCDs
