@@ -540,48 +540,61 @@ fused_ht_gemm_xreg_f32_ksplit_kernel(const float* __restrict__ W, const float* _
             };
 #pragma unroll
             for (int i = 0; i < 2 * NQ; ++i) load_tile(0, i);
-            // Quarters (pairs of tiles) software-pipelined by hand, as in the kernel above: while
-            // the MFMA chains of one quarter run, the vector unit splits the next one.
+            // K = 4096: the transform is linear, so the two quarters this phase keeps are
+            //   Y_{2 ph} = T(u) + T(v),  Y_{2 ph + 1} = T(u) - T(v),
+            //   u = x_0 + sigma x_2,  v = x_1 + sigma x_3,  sigma = (-1)^ph,
+            // x_i the quarters of the column: two 1024-point transforms per column and phase instead of
+            // four (the sums are fp32 additions of the inputs: one more rounding of 2^-24).
+            // K = 2048: u = x_0, v = x_1.  `half` = tile j (0 .. 3) of (u, v).
+            auto split_half = [&](int j, SplitTileF32& o) __attribute__((always_inline)) {
+                if constexpr (NQ == 4) {
+                    float t[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) t[e] = in[j][e] + sigma * in[j + 4][e];
+                    split_tile_f32(t, o);
+                } else {
+                    split_tile_f32(in[j], o);
+                }
+            };
+            // Halves (pairs of tiles) software-pipelined by hand, as in the kernel above: while the
+            // MFMA chains of one half run, the vector unit splits the next one.
             SplitTileF32 cur[2], nxt[2];
-            split_tile_f32(in[0], cur[0]);
-            split_tile_f32(in[1], cur[1]);
+            split_half(0, cur[0]);
+            split_half(1, cur[1]);
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
-                // Y[h][g][t]: elements 512 g + 256 t + 4 lane + e of quarter h of this phase, summed
-                // over the quarters i of the input as their transforms arrive:
-                //   K = 2048: Y_0 = T_0 + T_1, Y_1 = T_0 - T_1
-                //   K = 4096: Y_{2 ph} = T_0 + T_1 + sigma (T_2 + T_3),
-                //             Y_{2 ph + 1} = T_0 - T_1 + sigma (T_2 - T_3),  sigma = (-1)^ph
+                // Y[h][g][t]: elements 512 g + 256 t + 4 lane + e of quarter h of this phase:
+                //   Y[0] = T(u) + T(v),  Y[1] = T(u) - T(v)
                 f32x4 Y[2][2][2];
 #pragma unroll
-                for (int i = 0; i < NQ; ++i) {
-                    if (r + 1 < 8) {  // tiles 2 i, 2 i + 1 are split already: refill them for the next round
+                for (int i = 0; i < 2; ++i) {
+                    if (r + 1 < 8) {  // tiles 2 i, 2 i + 1 (and their partners) are split already: refill them
                         load_tile(r + 1, 2 * i);
                         load_tile(r + 1, 2 * i + 1);
+                        if (NQ == 4) {
+                            load_tile(r + 1, 2 * i + 4);
+                            load_tile(r + 1, 2 * i + 5);
+                        }
                     }
                     // (the loads stay here, a round ahead of their use: left alone, the scheduler
                     // sinks them to the use and the wavefront waits out every one)
                     __builtin_amdgcn_sched_barrier(0);
-                    if (!(r == 7 && i == NQ - 1)) {
-                        split_tile_f32(in[(2 * i + 2) % (2 * NQ)], nxt[0]);
-                        split_tile_f32(in[(2 * i + 3) % (2 * NQ)], nxt[1]);
+                    if (!(r == 7 && i == 1)) {
+                        split_half((2 * i + 2) % 4, nxt[0]);
+                        split_half((2 * i + 3) % 4, nxt[1]);
                     }
                     f32x4 a[2][2];
                     tile_pair_mfma_f32(cur, ops, a);
     #pragma unroll
                     for (int t = 0; t < 2; ++t) {
-                        f32x4 u = a[0][t] + a[1][t], v = a[0][t] - a[1][t];  // the two halves of T_i
-                        if (i >= 2) {
-                            u = u * sigma;
-                            v = v * sigma;
-                        }
+                        const f32x4 u = a[0][t] + a[1][t], v = a[0][t] - a[1][t];  // the two halves of T
                         if (i == 0) {
                             Y[0][0][t] = u, Y[0][1][t] = v, Y[1][0][t] = u, Y[1][1][t] = v;
                         } else {
                             Y[0][0][t] = Y[0][0][t] + u;
                             Y[0][1][t] = Y[0][1][t] + v;
-                            Y[1][0][t] = (i & 1) ? Y[1][0][t] - u : Y[1][0][t] + u;
-                            Y[1][1][t] = (i & 1) ? Y[1][1][t] - v : Y[1][1][t] + v;
+                            Y[1][0][t] = Y[1][0][t] - u;
+                            Y[1][1][t] = Y[1][1][t] - v;
                         }
                     }
                     cur[0] = nxt[0];
