@@ -7,6 +7,7 @@ torch is used for device memory and streams only; all arithmetic happens in HIP 
 """
 from __future__ import annotations
 
+import contextlib
 import math
 
 import torch
@@ -24,8 +25,24 @@ def _is_pow2(n: int) -> bool:
     return n > 0 and (n & (n - 1)) == 0
 
 
+_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_SAME_DEVICE = contextlib.nullcontext()
+
+
 def _stream(t: torch.Tensor) -> int:
+    """The current stream of ``t``'s device as a raw handle (the direct query when this torch has
+    it: a fraction of the cost of building a ``torch.cuda.Stream`` object on every call)."""
+    if _RAW_STREAM is not None and t.device.index is not None:
+        return _RAW_STREAM(t.device.index)
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _on_device_of(t: torch.Tensor):
+    """Context that makes ``t``'s device current for the launch; nothing to do (and nothing to
+    pay) when it already is, the usual case."""
+    if t.device.index is None or t.device.index == torch.cuda.current_device():
+        return _SAME_DEVICE
+    return torch.cuda.device(t.device)
 
 
 def _require_cuda(t: torch.Tensor, name: str) -> None:
@@ -71,7 +88,7 @@ def hadamard_transform(x: torch.Tensor, scale: float | None = None, *, inplace: 
     else:
         dst = torch.empty(x.shape, dtype=x.dtype, device=x.device)
     lib = _lib.load()
-    with torch.cuda.device(x.device):
+    with _on_device_of(x):
         st = lib.mi_fwht(src.data_ptr(), dst.data_ptr(), rows, n, _DTYPE_CODE[x.dtype], s,
                          _stream(x))
     _lib.check(st, "hadamard_transform")
@@ -105,7 +122,7 @@ def fused_ht_gemv(W: torch.Tensor, X: torch.Tensor, scale: float | None = None) 
         return Y
     Wc, Xc = _dense16(W), _dense16(X)
     lib = _lib.load()
-    with torch.cuda.device(W.device):
+    with _on_device_of(W):
         st = lib.mi_fused_ht_gemv(Wc.data_ptr(), Xc.data_ptr(), Y.data_ptr(), M, N, B,
                                   _lib.MI_F32, s, _stream(W))
     _lib.check(st, "fused_ht_gemv")
@@ -147,7 +164,7 @@ def fused_ht_gemm(W: torch.Tensor, Xt: torch.Tensor, scale: float | None = None,
         return C
     Wc, Xc = _dense16(W), _dense16(Xt)
     lib = _lib.load()
-    with torch.cuda.device(W.device):
+    with _on_device_of(W):
         st = lib.mi_fused_ht_gemm(Wc.data_ptr(), Xc.data_ptr(), C.data_ptr(), M, N, K,
                                   _DTYPE_CODE[W.dtype], _DTYPE_CODE[od], s, _stream(W))
     _lib.check(st, "fused_ht_gemm")
@@ -179,7 +196,7 @@ def rht_quant_fp8(x: torch.Tensor, sign: torch.Tensor, scale: float | None = Non
     y = torch.empty((T, n), dtype=torch.bfloat16, device=x.device) if return_prequant else None
     if T:
         lib = _lib.load()
-        with torch.cuda.device(x.device):
+        with _on_device_of(x):
             st = lib.mi_rht_quant_fp8(xc.data_ptr(), sg.data_ptr(), q.data_ptr(), rs.data_ptr(),
                                       y.data_ptr() if y is not None else None, T, n, s, _stream(x))
         _lib.check(st, "rht_quant_fp8")
@@ -214,7 +231,7 @@ def fp8_gemm_rowscale(qa: torch.Tensor, sa: torch.Tensor, qb: torch.Tensor, sb: 
     sa = sa.to(device=qa.device, dtype=torch.float32).contiguous().view(-1)
     sb = sb.to(device=qa.device, dtype=torch.float32).contiguous().view(-1)
     lib = _lib.load()
-    with torch.cuda.device(qa.device):
+    with _on_device_of(qa):
         st = lib.mi_fp8_gemm_rowscale(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(),
                                       out.data_ptr(), T, N, K, _stream(qa))
     _lib.check(st, "fp8_gemm_rowscale")
