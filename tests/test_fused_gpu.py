@@ -48,7 +48,9 @@ def test_gemv_reference_self_check(pkg, oracle, M, N, B):
 # Launch paths that only larger problems reach: the 64-row workgroup variant (column groups x
 # 64-row blocks >= 256; the benchmark's M=N=1024 with B=256 and B=512, the shapes of
 # fused_ht/fwht_gemv_fusion.cu:643-653) and a workgroup that walks several row blocks with one
-# transformed tile (more row blocks than workgroup rows in the grid).
+# transformed tile (more row blocks than workgroup rows in the grid).  (The 32-row variant runs
+# between 128 and 255 such groups: (1024, 1024, 128) here and (256, 256, 512) above; everything
+# smaller runs 16-row workgroups.)
 @pytest.mark.parametrize("M,N,B", [(1024, 1024, 256), (1024, 1024, 512), (1024, 1024, 128),
                                    (4096, 256, 4096), (2000, 64, 1000), (4100, 2048, 130)])
 def test_gemv_large_launch_paths(pkg, oracle, M, N, B):
