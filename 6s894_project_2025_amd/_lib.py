@@ -1,4 +1,5 @@
-"""ctypes binding of ``libmi_hadamard.so`` (declarations: ``include/mi_hadamard.h``)."""
+"""ctypes binding of ``libmi_hadamard.so`` (declarations: ``include/mi_hadamard.h``) and of the
+benchmark harness's ``libmi_probe.so`` (``include/mi_probe.h``)."""
 from __future__ import annotations
 
 import ctypes
@@ -23,11 +24,16 @@ SIGNATURES = {
     "mi_debug_mfma_16x16": (_i, [_i, _vp, _vp, _vp, _vp]),
     "mi_debug_convert": (_i, [_i, _vp, _vp, _u64, _vp]),
     "mi_debug_device_fwht": (_i, [_vp, _vp, _u64, _u32, _i, _f, _vp]),
-    "mi_debug_mfma_rate": (_i, [_i, _i, _u32, _u32, _vp, _vp, _vp]),
     "mi_debug_fused_gemm_tiling": (_i, [_u32, _u32, _u32, _vp, _vp, _u32]),
 }
 
+PROBE_LIB_PATH = os.path.join(HERE, "libmi_probe.so")
+PROBE_SIGNATURES = {
+    "mi_probe_mfma_rate": (_i, [_i, _i, _u32, _u32, _vp, _vp, _vp]),
+}
+
 _lib = None
+_probe = None
 
 
 def load() -> ctypes.CDLL:
@@ -49,6 +55,23 @@ def load() -> ctypes.CDLL:
         fn.restype = res
         fn.argtypes = args
     _lib = lib
+    return lib
+
+
+def load_probe() -> ctypes.CDLL:
+    """Load the matrix-core rate probe (benchmark harness only; no op of the package uses it)."""
+    global _probe
+    if _probe is not None:
+        return _probe
+    load()
+    if not os.path.exists(PROBE_LIB_PATH):
+        raise RuntimeError(f"{PROBE_LIB_PATH} is missing: build it with `python 6s894_project_2025_amd/build.py`")
+    lib = ctypes.CDLL(PROBE_LIB_PATH)
+    for name, (res, args) in PROBE_SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _probe = lib
     return lib
 
 

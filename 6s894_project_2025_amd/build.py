@@ -1,4 +1,5 @@
-"""Builds ``libmi_hadamard.so`` (the C-ABI library) in-tree with hipcc for gfx950.
+"""Builds ``libmi_hadamard.so`` (the C-ABI library) and ``libmi_probe.so`` (the benchmark
+harness's matrix-core rate probe, kept out of the product library) in-tree with hipcc for gfx950.
 
 Run as ``python 6s894_project_2025_amd/build.py`` or through ``__graft_entry__.build()``.
 hipcc cross-compiles without a GPU, so this works on a CPU-only machine.
@@ -18,6 +19,8 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "libmi_hadamard.so")
+PROBE_SRC = os.path.join(HERE, "probe")
+PROBE_LIB_PATH = os.path.join(HERE, "libmi_probe.so")
 
 ARCH = "gfx950"
 # Packed-fp32 VALU forms are switched off for every device translation unit.
@@ -165,6 +168,26 @@ def check_register_resident_isa(asm_text: str, where: str) -> int:
     return kernels
 
 
+_M0_USE = re.compile(r"\bm0\b")
+_M0_SET_BY_TRANSFER = re.compile(r"^\s*s_add_i32 m0, ")
+
+
+def check_m0_is_the_transfers_alone(asm_text: str, where: str) -> int:
+    """The direct global -> LDS transfers take their LDS base from M0, written by an opaque statement
+    one instruction earlier.  Raises if any other instruction of the file names M0 (a compiler use
+    between the two would redirect a transfer); returns the number of M0 writes seen."""
+    writes = 0
+    for line in asm_text.splitlines():
+        text = line.split(";")[0]
+        if not _M0_USE.search(text) or text.lstrip().startswith("."):
+            continue
+        if _M0_SET_BY_TRANSFER.match(text):
+            writes += 1
+        else:
+            raise RuntimeError(f"{where}: `{text.strip()}` uses M0, which belongs to the global -> LDS transfers")
+    return writes
+
+
 def sources() -> list[str]:
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
@@ -197,25 +220,37 @@ def _compile(src: str) -> str:
             text = f.read()
         if check_register_resident_isa(text, base) == 0 or check_mfma_results_not_touched_early(text, base) == 0:
             raise RuntimeError(f"{base}: no register-resident MFMA loop found in the device assembly")
+        if check_m0_is_the_transfers_alone(text, base) == 0:
+            raise RuntimeError(f"{base}: no global -> LDS transfer found in the device assembly")
         for t in temps:
             os.remove(t)
     return obj
 
 
-def build(verbose: bool = True, jobs: int = 4) -> str:
-    """Compile every ``csrc/*.hip`` and link the shared library.  Always recompiles."""
-    os.makedirs(OBJ_DIR, exist_ok=True)
-    srcs = sources()
-    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(_compile, srcs))
-    tmp = LIB_PATH + ".tmp"
+def probe_sources() -> list[str]:
+    return sorted(os.path.join(PROBE_SRC, f) for f in os.listdir(PROBE_SRC) if f.endswith(".hip"))
+
+
+def _link(objs: list[str], lib_path: str) -> None:
+    tmp = lib_path + ".tmp"
     cmd = [_hipcc(), "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", tmp]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stderr}")
-    os.replace(tmp, LIB_PATH)
+    os.replace(tmp, lib_path)
+
+
+def build(verbose: bool = True, jobs: int = 4) -> str:
+    """Compile every ``csrc/*.hip`` into the product library and every ``probe/*.hip`` into the
+    probe library.  Always recompiles."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    srcs, probes = sources(), probe_sources()
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(_compile, srcs + probes))
+    _link(objs[:len(srcs)], LIB_PATH)
+    _link(objs[len(srcs):], PROBE_LIB_PATH)
     if verbose:
-        print(f"built {LIB_PATH} from {len(srcs)} sources")
+        print(f"built {LIB_PATH} from {len(srcs)} sources, {PROBE_LIB_PATH} from {len(probes)}")
     return LIB_PATH
 
 

@@ -97,19 +97,13 @@ __device__ __forceinline__ void drain_mfma(f32x4 (&acc)[4][4])
 }
 
 __device__ __forceinline__ void wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-// at most N vector memory operations of this wavefront still outstanding (they complete in order)
-// (`n` folds to a constant once the loops around the call are unrolled)
+// at most n vector memory loads of this wavefront still outstanding (they complete in order); a
+// negative n means there is nothing to wait for.  `n` must fold to a constant once the loops around
+// the call are unrolled: it is an immediate of the instruction, so a count that does not fold, or
+// one the counter's six bits cannot hold, fails to build instead of silently dropping the wait.
 __device__ __forceinline__ void wait_vm(int n)
 {
-    switch (n) {
-        case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-        case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
-        case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
-        case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
-        case 16: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
-        case 20: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
-        default: break;  // nothing to wait for
-    }
+    if (n >= 0) asm volatile("s_waitcnt vmcnt(%0)" ::"i"(n) : "memory");
 }
 
 // A wavefront that has its SIMD to itself issues one instruction every four cycles, whatever the
@@ -124,7 +118,9 @@ __device__ __forceinline__ void wait_vm(int n)
 // must fold to a constant (an immediate of the scalar add: a transfer then needs no scalar
 // register of its own).  The instruction's own offset field is left at zero: the hardware adds
 // it to the LDS address as well as to the global one.
-// (M0 carries the LDS base of the transfer; nothing else in these kernels uses it.)
+// (M0 carries the LDS base of the transfer.  It is a reserved register that cannot be named as a
+// clobber, so the build reads the generated ISA instead and fails if anything but these statements
+// touches M0 in a kernel that uses them: build.py, check_m0_is_the_transfers_alone.)
 __device__ __forceinline__ void lds_transfer_target(uint32_t lds_wave_base, int lds_imm)
 {
     asm volatile("s_add_i32 m0, %0, %1" :: "s"(lds_wave_base), "i"(lds_imm) : "memory", "scc");

@@ -98,7 +98,8 @@ class TestConfig:
 def _check_case(name: str, case: Case, full: torch.Tensor) -> None:
     """Runs the case on the *full-size* buffer (so the launch path that gets timed is the one that
     gets checked) and compares bounded row slices of the result with the truth path, which costs
-    O(rows * n^2) and is therefore evaluated on slices only.  Restores the buffer afterwards."""
+    O(rows * n^2) and is therefore evaluated on slices only.  Only those slices are put back to
+    their input values; the caller resets the whole buffer between cases."""
     rows, n = full.shape
     take = min(rows, max(1, (1 << 21) // n))
     starts = sorted({0, max(0, rows // 2 - take // 2), rows - take})
@@ -254,18 +255,18 @@ def run_gemv(configs=None, warmup: int = 10, iters: int = 100, out_prefix: str |
 
 def mfma_probe(shape: int, lds_reads: int, waves_per_simd: int, operands: torch.Tensor,
                steps: int = 4096, repeats: int = 20, warm_ms: float = 30.0) -> dict[str, Any]:
-    """One configuration of ``mi_debug_mfma_rate``: nothing but back-to-back bf16 MFMAs on every
+    """One configuration of ``mi_probe_mfma_rate`` (``libmi_probe.so``): nothing but back-to-back bf16 MFMAs on every
     SIMD (plus ``lds_reads`` fragment reads per step), timed past the clock ramp.  ``ghz`` is loop
     cycles (shader clock counter, slowest wavefront) over the event-timed duration of the whole
     launch, so it is a slight underestimate."""
     from . import _lib
 
-    lib = _lib.load()
+    lib = _lib.load_probe()
     stream = torch.cuda.current_stream().cuda_stream
     cycles = torch.zeros(512, dtype=torch.int64, device=operands.device)
 
     def call():
-        _lib.check(lib.mi_debug_mfma_rate(shape, lds_reads, waves_per_simd, steps, operands.data_ptr(),
+        _lib.check(lib.mi_probe_mfma_rate(shape, lds_reads, waves_per_simd, steps, operands.data_ptr(),
                                           cycles.data_ptr(), stream), "mfma probe")
     ms, _ = steady_window_ms(call, repeats, warm_ms)
     flops = 256 * 4 * waves_per_simd * steps * 131072

@@ -1,4 +1,5 @@
-// Matrix-core throughput probe (mi_debug_mfma_rate), gfx950.
+// Matrix-core throughput probe (mi_probe_mfma_rate), gfx950.  Built into libmi_probe.so, a
+// measurement aid beside the product library: nothing in libmi_hadamard.so depends on it.
 //
 // What a kernel can get out of the matrix cores depends on more than the instruction's issue
 // rate: the clock the chip sustains under the load (which depends on the operand data: random
@@ -12,6 +13,7 @@
 //
 // No counterpart in the reference (it has no matrix-core kernels in its fused path).
 #include "common.hpp"
+#include "mi_probe.h"
 
 namespace mi {
 namespace {
@@ -107,7 +109,7 @@ int launch_probe(const void* operands, uint64_t* cycles, uint32_t waves_per_simd
 }  // namespace
 }  // namespace mi
 
-extern "C" int mi_debug_mfma_rate(int shape, int lds_reads, uint32_t waves_per_simd, uint32_t steps,
+extern "C" int mi_probe_mfma_rate(int shape, int lds_reads, uint32_t waves_per_simd, uint32_t steps,
                                   const void* operands, uint64_t* cycles, void* stream)
 {
     using namespace mi;

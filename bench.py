@@ -19,8 +19,10 @@ JSON line:
 Timing protocol (the reference's, bench/bench.py:112-127): warm-up launches, then K back-to-back
 launches inside one event window on the launch stream, inputs resident in HBM.  The matrix-core
 bound kernels are warmed for at least 60 ms first (clock ramp).  `others` carries the remaining
-configurations (fp32 fused GEMM, HT+GEMV with its unfused comparator, RHT+FP8 quantize, FP8 GEMM),
-and with --sweep the n = 2^4..2^15 transform sweep.
+configurations (the 15 (K, N, M) shapes of the reference's sweep, fused_ht/benchmark_sweep.py:20-45,
+in bf16 and in fp32, each beside transform + vendor GEMM; HT+GEMV with its unfused comparator;
+RHT+FP8 quantize; FP8 GEMM).  `fwht.sweep_128MiB` is the bf16 n = 2^4..2^15 sweep of configs[1];
+--sweep adds fp16 and fp32.
 """
 from __future__ import annotations
 
@@ -40,6 +42,7 @@ if ROOT not in sys.path:
 PKG = "6s894_project_2025_amd"
 HBM_PEAK_GBS = 8000.0
 PEAK_TFLOPS = {"bf16": 2516.6, "f16": 2516.6, "f32": 157.3, "fp8": 5033.2}
+RAMP_MS = 60.0  # untimed device time before a matrix-core-bound kernel is timed (clock ramp)
 BASELINE_METRIC = "fused HT+GEMM TFLOP/s (K=1024,M=N=4096) + standalone FWHT HBM GB/s vs peak"
 
 
@@ -75,6 +78,23 @@ def roofline(bound, achieved, peak, unit, traffic, **extra):
          "frac": round(achieved / peak, 4), "traffic": traffic}
     r.update(extra)
     return r
+
+
+def fwht_sweep(hada, events_ms, torch, dev, dtypes, calls=50):
+    """In-place transform of a 128 MiB tensor for every n = 2^4 .. 2^15: 3 warm-up launches, then
+    `calls` back-to-back launches in one event window; bytes = one read + one write."""
+    sweep = {}
+    for dname, dt, es in dtypes:
+        for p in range(4, 16):
+            nn = 1 << p
+            numel = (128 << 20) // es
+            t = torch.randn(numel // nn, nn, device=dev).to(dt)
+            ms, _ = events_ms(lambda: hada.hadamard_transform(t, inplace=True), calls, 3)
+            gbs = 2 * numel * es / ms / 1e6
+            sweep[f"{dname}_n{nn}"] = {"us": round(ms * 1e3, 2), "GB/s": round(gbs, 1),
+                                       "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+            del t
+    return sweep
 
 
 def main() -> int:
@@ -124,13 +144,13 @@ def main() -> int:
         err = ((C.float() - ref).abs().max() / ref.abs().max()).item()
         del ref
         gsteps = max(10, steps)
-        steady_ms(lambda: hada.fused_ht_gemm(W, Xt), 4)  # clock ramp, untimed
+        steady_ms(lambda: hada.fused_ht_gemm(W, Xt), 4, RAMP_MS)  # clock ramp, untimed
         ms, wall_ms = events_ms(lambda: hada.fused_ht_gemm(W, Xt), gsteps, warmup)
         tf = flops / ms / 1e9
-        mm_ms, _ = steady_ms(lambda: torch.matmul(W, Xt.t()), gsteps)
+        mm_ms, _ = steady_ms(lambda: torch.matmul(W, Xt.t()), gsteps, RAMP_MS)
         # the reference's "Baseline (Unfused)" (fusion_pipelined.cu:640-656): transform kernel, H(X)
         # through HBM, then the GEMM (here the vendor library's)
-        un_ms, _ = steady_ms(lambda: torch.matmul(W, hada.hadamard_transform(Xt).t()), gsteps)
+        un_ms, _ = steady_ms(lambda: torch.matmul(W, hada.hadamard_transform(Xt).t()), gsteps, RAMP_MS)
         # what this box sustains with nothing but MFMAs (random bf16 operands, one wavefront per
         # SIMD with four LDS fragment reads per step, the regime of the fused kernel), and the
         # launch-to-launch time of a kernel that does next to nothing
@@ -140,6 +160,13 @@ def main() -> int:
         result.update({
             "metric": BASELINE_METRIC,
             "value": round(tf, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": gsteps, "warmup": warmup,
+            "warmup_protocol": {
+                "clock_ramp_ms": RAMP_MS, "calls_after_ramp": warmup,
+                "note": "every matrix-core-bound timing (this one, the vendor GEMM, the unfused path, the "
+                        "`others` GEMM rows) is preceded by at least clock_ramp_ms of untimed back-to-back "
+                        "launches of the same call (the clocks keep settling for ~30 ms of sustained load); "
+                        "the headline then runs `warmup` more untimed calls before the timed window, the "
+                        "comparators go straight into theirs; `others` rows ramp for 30 ms"},
             "ms_per_step": round(ms, 6), "wall_ms_per_step": round(wall_ms, 6),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16", "data": "synthetic",
@@ -158,7 +185,7 @@ def main() -> int:
                 "sustained_tflops": round(probe["tflops"], 1), "shader_ghz": round(probe["ghz"], 3),
                 "frac_of_peak": round(probe["tflops"] / PEAK_TFLOPS["bf16"], 4),
                 "note": "back-to-back v_mfma_f32_16x16x32_bf16 on every SIMD from registers, random bf16 "
-                        "operands (mi_debug_mfma_rate): the rate this box sustains under full matrix-core "
+                        "operands (mi_probe_mfma_rate, libmi_probe.so): the rate this box sustains under full matrix-core "
                         "load; value / sustained_tflops = " + str(round(tf / probe["tflops"], 3))},
             "launch_floor_us": round(floor["us_per_launch"], 2),
         })
@@ -211,6 +238,10 @@ def main() -> int:
                                      add_one_proxy_gbs=round(bb / ams / 1e6, 1))}
             del big
         fw["dram_bound"] = dram
+        # configs[1]'s sweep: last dim 2^4 .. 2^15, row count chosen so that each tensor is 128 MiB
+        # (bench/bench.py:133,138 of the reference sweeps the same sizes); bf16 here, --sweep adds
+        # fp16 and fp32
+        fw["sweep_128MiB"] = fwht_sweep(hada, events_ms, torch, dev, (("bf16", torch.bfloat16, 2),))
         if result:
             result["fwht"] = fw
         else:
@@ -223,8 +254,11 @@ def main() -> int:
     # traffic per flop; K = 2048 and 4096 run the kernel that splits K over wavefront pairs (bf16,
     # fused / vendor GEMM without transform / transform + vendor GEMM) --------------------------------
     if not only:
-        for (Kx, Mx, Nx) in ((1024, 8192, 8192), (512, 4096, 4096), (512, 8192, 8192),
-                             (2048, 2048, 2048), (2048, 4096, 4096), (4096, 2048, 2048), (4096, 4096, 4096)):
+        # the reference's 15 sweep shapes (fused_ht/benchmark_sweep.py:20-45) but the headline one,
+        # which is the top-level record, and two larger ones
+        shapes = [(k, sz, sz) for k in (256, 512, 1024, 2048, 4096) for sz in (1024, 2048, 4096)
+                  if (k, sz) != (K, M)] + [(1024, 8192, 8192), (512, 8192, 8192)]
+        for (Kx, Mx, Nx) in shapes:
             Wx = torch.randn(Mx, Kx, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(dev)
             Xx = torch.randn(Nx, Kx, generator=torch.Generator().manual_seed(0)).to(torch.bfloat16).to(dev)
             fx = 2 * Mx * Nx * Kx
@@ -233,7 +267,8 @@ def main() -> int:
             u_ms, _ = steady_ms(lambda: torch.matmul(Wx, hada.hadamard_transform(Xx).t()), 30, 30.0)
             others[f"fused_ht_gemm_bf16_K{Kx}_M{Mx}_N{Nx}"] = {
                 "us": round(f_ms * 1e3, 2), "algorithmic_flops": fx,
-                "roofline": roofline("mfma", fx / f_ms / 1e9, PEAK_TFLOPS["bf16"], "TFLOP/s", None),
+                "roofline": roofline("mfma", fx / f_ms / 1e9, PEAK_TFLOPS["bf16"], "TFLOP/s",
+                                     traffic.get(f"fused_ht_gemm_bf16_K{Kx}_M{Mx}_N{Nx}")),
                 "library_gemm_without_transform_us": round(v_ms * 1e3, 2),
                 "unfused_transform_then_library_gemm_us": round(u_ms * 1e3, 2),
                 "fused_over_unfused_speedup": round(u_ms / f_ms, 3)}
@@ -258,13 +293,14 @@ def main() -> int:
         del W, Xt
         # the other K of the reference's sweep at the same M = N (fp32 is the reference's precision)
         if not only:
-            for Kx in (256, 512, 2048, 4096):
-                Wx = torch.randn(M, Kx, generator=torch.Generator().manual_seed(1)).to(dev)
-                Xx = torch.randn(N, Kx, generator=torch.Generator().manual_seed(0)).to(dev)
-                fx = 2 * M * N * Kx
+            for Kx, Sx in [(k, sz) for k in (256, 512, 1024, 2048, 4096) for sz in (1024, 2048, 4096)
+                           if (k, sz) != (K, M)]:
+                Wx = torch.randn(Sx, Kx, generator=torch.Generator().manual_seed(1)).to(dev)
+                Xx = torch.randn(Sx, Kx, generator=torch.Generator().manual_seed(0)).to(dev)
+                fx = 2 * Sx * Sx * Kx
                 f_ms, _ = steady_ms(lambda: hada.fused_ht_gemm(Wx, Xx), 10, 30.0)
                 u_ms, _ = steady_ms(lambda: torch.matmul(Wx, hada.hadamard_transform(Xx).t()), 10, 30.0)
-                others[f"fused_ht_gemm_f32_K{Kx}_M{M}_N{N}"] = {
+                others[f"fused_ht_gemm_f32_K{Kx}_M{Sx}_N{Sx}"] = {
                     "us": round(f_ms * 1e3, 2), "algorithmic_flops": fx,
                     "roofline": roofline("mfma", fx / f_ms / 1e9, PEAK_TFLOPS["f32"], "TFLOP/s", None),
                     "unfused_transform_then_library_gemm_us": round(u_ms * 1e3, 2),
@@ -273,8 +309,10 @@ def main() -> int:
 
     # ---- fused HT+GEMV and its unfused comparator (fwht_gemv_fusion.cu:323-363) ----------------------
     if want("gemv"):
+        # config 3 (M = N = 256, B = 512; M = N = 1024, B = 8 .. 512) and the two large shapes of the
+        # reference's own benchmark list (fwht_gemv_fusion.cu:643-653)
         for (m, nn, b) in ((256, 256, 512), (1024, 1024, 8), (1024, 1024, 64), (1024, 1024, 256),
-                           (1024, 1024, 512)):
+                           (1024, 1024, 512), (1024, 1024, 2048), (2048, 2048, 512)):
             Wg = torch.randn(m, nn, device=dev) / math.sqrt(nn)
             X = torch.randn(nn, b, device=dev)
             Xcols = X.t().contiguous()  # untimed layout change for the unfused leg's transform
@@ -334,17 +372,8 @@ def main() -> int:
         return 0
 
     if args.sweep:
-        sweep = {}
-        for dname, dt, es in (("bf16", torch.bfloat16, 2), ("f16", torch.float16, 2), ("f32", torch.float32, 4)):
-            for p in range(4, 16):
-                nn = 1 << p
-                numel = (128 << 20) // es
-                t = torch.randn(numel // nn, nn, device=dev).to(dt)
-                ms, _ = events_ms(lambda: hada.hadamard_transform(t, inplace=True), 50, 3)
-                sweep[f"{dname}_n{nn}"] = {"us": round(ms * 1e3, 2),
-                                           "GB/s": round(2 * numel * es / ms / 1e6, 1)}
-                del t
-        others["fwht_sweep_128MiB"] = sweep
+        others["fwht_sweep_128MiB"] = fwht_sweep(hada, events_ms, torch, dev,
+                                                 (("f16", torch.float16, 2), ("f32", torch.float32, 4)))
     result["others"] = others
 
     # ---- CPU baselines: the reference's truth path on the host cores ----------------------------------

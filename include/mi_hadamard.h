@@ -157,22 +157,6 @@ int mi_debug_device_fwht(const void* in, void* out, uint64_t rows, uint32_t n, i
                          float scale, void* stream);
 
 /*
- * Matrix-core throughput probe: 256 workgroups (one per compute unit) of 256 * waves_per_simd
- * threads each run `steps` K steps of eight independent v_mfma_f32_16x16x32_bf16 (shape 16) or
- * four v_mfma_f32_32x32x16_bf16 (shape 32; the same 131072 flops per wavefront and step), with
- * lds_reads (0 or 4) 16-byte-per-lane LDS fragment reads per step beside them, on operands copied
- * from `operands`; cycles[w] receives the shader clock cycles workgroup w spent in the loop.  Used
- * to measure the clock and the matrix-core rate the chip sustains for a given operand pattern.
- * No counterpart in the reference.
- *   operands : device, 16-byte aligned, at least 64 KiB (any bit pattern; bf16 operands)
- *   cycles   : device, 512 x uint64: [0, 256) cycles per workgroup, [256, 512) a checksum of each
- *              workgroup's accumulators (an output whose only purpose is to keep the arithmetic alive)
- *   waves_per_simd in {1, 2, 4};  steps a positive multiple of 4.
- */
-int mi_debug_mfma_rate(int shape, int lds_reads, uint32_t waves_per_simd, uint32_t steps,
-                       const void* operands, uint64_t* cycles, void* stream);
-
-/*
  * Host-only: how mi_fused_ht_gemm cuts a 16-bit problem with K = 512 ... 4096 into workgroups (no
  * GPU call; MI_ERR_SIZE for any other K).
  * The (column group, M slice) grid, the XCD rectangles and the map from workgroup id to tile are

@@ -1,0 +1,34 @@
+/*
+ * mi_probe.h -- C ABI of libmi_probe.so, the measurement aid that ships beside libmi_hadamard.so
+ * (benchmark harness only; the product library neither links nor loads it).
+ * Status codes are mi_status values (mi_hadamard.h).
+ */
+#ifndef MI_PROBE_H
+#define MI_PROBE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/*
+ * Matrix-core throughput probe: 256 workgroups (one per compute unit) of 256 * waves_per_simd
+ * threads each run `steps` K steps of eight independent v_mfma_f32_16x16x32_bf16 (shape 16) or
+ * four v_mfma_f32_32x32x16_bf16 (shape 32; the same 131072 flops per wavefront and step), with
+ * lds_reads (0 or 4) 16-byte-per-lane LDS fragment reads per step beside them, on operands copied
+ * from `operands`; cycles[w] receives the shader clock cycles workgroup w spent in the loop.  Used
+ * to measure the clock and the matrix-core rate the chip sustains for a given operand pattern.
+ * No counterpart in the reference.
+ *   operands : device, 16-byte aligned, at least 64 KiB (any bit pattern; bf16 operands)
+ *   cycles   : device, 512 x uint64: [0, 256) cycles per workgroup, [256, 512) a checksum of each
+ *              workgroup's accumulators (an output whose only purpose is to keep the arithmetic alive)
+ *   waves_per_simd in {1, 2, 4};  steps a positive multiple of 4.
+ */
+int mi_probe_mfma_rate(int shape, int lds_reads, uint32_t waves_per_simd, uint32_t steps,
+                       const void* operands, uint64_t* cycles, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI_PROBE_H */

@@ -12,8 +12,11 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "mi_hadamard.h")
 
 
-def _declared_symbols():
-    text = open(HEADER).read()
+PROBE_HEADER = os.path.join(ROOT, "include", "mi_probe.h")
+
+
+def _declared_symbols(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(mi_[a-z0-9_]+)\s*\(", text)))
 
@@ -30,6 +33,17 @@ def test_library_exports_every_declared_symbol(libmod):
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/mi_hadamard.h but not exported"
     assert sorted(libmod.SIGNATURES) == declared
+
+
+def test_probe_library_is_separate_from_the_product_library(libmod):
+    # the matrix-core rate probe is a measurement aid: its own header, its own library, and the
+    # product library exports nothing of it
+    declared = _declared_symbols(PROBE_HEADER)
+    assert declared == sorted(libmod.PROBE_SIGNATURES) == ["mi_probe_mfma_rate"]
+    probe = libmod.load_probe()
+    for name in declared:
+        assert hasattr(probe, name)
+        assert not hasattr(libmod.load(), name)
 
 
 def test_version_and_status_text(libmod):
@@ -227,3 +241,16 @@ def test_build_rejects_early_reads_of_an_assembly_mfma_result():
     with pytest.raises(RuntimeError, match="reads the result"):
         check("\ts_branch .LBB0_9\n" + "\ts_endpgm\n" + ".LBB0_9:\n\tv_cvt_pk_bf16_f32 v9, v32, v33\n")
     assert check("\ts_cbranch_vccnz .LBB0_9\n" + filler * 20 + ".LBB0_9:\n" + filler * 11 + "\tv_mov_b32_e32 v9, v32\n") == 1
+
+
+def test_build_rejects_other_uses_of_m0():
+    """The global -> LDS transfers take their LDS base from M0, set by an opaque statement; the
+    build fails if anything else in such a file names M0."""
+    import importlib
+    build = importlib.import_module("6s894_project_2025_amd.build")
+    good = ("_Zk: ; @_Zk\n\ts_add_i32 m0, s5, 0x8000\n\tv_mfma_f32_16x16x32_bf16 v[32:35], v[96:99], a[124:127], v[32:35]\n"
+            "\tglobal_load_lds_dwordx4 v7, s[2:3]\n\ts_add_i32 m0, s5, 0x8400 ; comment mentioning m0\n\ts_endpgm\n")
+    assert build.check_m0_is_the_transfers_alone(good, "good") == 2
+    for other in ("\ts_mov_b32 m0, s9\n", "\ts_mov_b32 s9, m0\n", "\tv_readlane_b32 s4, v3, m0\n"):
+        with pytest.raises(RuntimeError, match="uses M0"):
+            build.check_m0_is_the_transfers_alone(good.replace("\ts_endpgm\n", other + "\ts_endpgm\n"), "bad")
