@@ -134,95 +134,229 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
 
     // ---- prologue: Y fragments of this wavefront's columns ---------------------------------------
     // Column of fragment nb, fragment column j (= MFMA B column = lane lo): n0 + CPW w + NBF j + nb,
-    // so that a lane ends up with NBF adjacent output columns.  One round = the 16 columns of one
-    // fragment index; the tiles of the next round are requested as this round's are consumed, and
-    // the first AHEAD stages of W behind the last X tile (vector memory operations complete in
-    // order, so anything issued earlier would hold the tiles back), two pieces per column of the
-    // last round, while its tiles arrive.
+    // so that a lane ends up with NBF adjacent output columns.  Columns are taken in the order
+    // c = 16 nb + j as one software pipeline in which four things run side by side:
+    //   - the fetch of X: column c + 16 is requested when column c has been consumed, so sixteen
+    //     columns (32 KB per wavefront) are in flight all the time, enough to keep the path from the
+    //     L2 busy across its latency;
+    //   - the transform of column c on the matrix cores (its conversions in the MFMAs' shadow);
+    //   - the layout change through LDS: a transformed column is written as it is produced (lane l
+    //     owns 8 consecutive k), and the sixteen columns of a round are read back in operand order
+    //     (lane (hi, lo): 8 consecutive k of column lo) during the first four columns of the next
+    //     round, whose own results wait in registers until those reads have been issued (LDS
+    //     operations of one wavefront complete in order: no barrier between its writes and reads);
+    //   - stage 0 of W, requested behind the X columns of the first round.
+    // Only the last round's reads are left over at the end.  The wavefront's LDS area is 32 KB (a
+    // whole round at K = 1024, two rounds taking turns at K = 512), laid over its own rows of stage
+    // buffers 1 .. 3 and of the 32 KB behind the ring: once its last reads have returned, the
+    // wavefront requests its pieces of stages 1 .. AHEAD - 1 without waiting for anybody else.
     V8 yf[NBF][KSTEPS];
     {
-        unsigned char* area = lds + kAreaBase + wave * kAreaBytes;
-        auto prefetch_w = [&](int nb, int j) __attribute__((always_inline)) {
-            if (nb == NBF - 1 && j >= 2 && j < 2 + 4 * AHEAD) {
-                const int p = 2 * (j - 2);
-                w_issue(p >> 3, p >> 3, p & 7);
-                w_issue((p + 1) >> 3, (p + 1) >> 3, (p + 1) & 7);
+        constexpr int NH = K / 512;       // 512-element halves of a column
+        constexpr int TOTAL = 16 * NBF;   // columns of this wavefront
+        constexpr int RPR = KSTEPS;       // reads per round: one per K step
+        // half/buffer b, column j -> byte offset inside the workgroup's LDS, before the chunk term
+        auto area_at = [&](int b, uint32_t j) __attribute__((always_inline)) -> uint32_t {
+            return area_piece_offset(wave, (uint32_t)b + 2u * (j >> 3)) + (j & 7u) * 1024u;
+        };
+        constexpr int LA = K == 1024 ? 12 : 16;   // columns in flight (what the register file leaves room for)
+        V8 in[LA][NH];
+        // X is addressed as a uniform base (the wavefront's first column, clamped into the matrix)
+        // plus a 32-bit lane offset: column (clamped to the last one) and the lane's 16 bytes
+        const uint32_t col_first = min(n0 + CPW * wave, N - 1u);
+        const unsigned char* const xb = reinterpret_cast<const unsigned char*>(Xt) + (uint64_t)col_first * (K * 2u);
+        const uint32_t last_rel = (N - 1u - col_first) * (K * 2u), lane16 = lane << 4;
+        auto column_offset = [&](int c) __attribute__((always_inline)) -> uint32_t {
+            return min((uint32_t)(NBF * (c & 15) + (c >> 4)) * (K * 2u), last_rel) + lane16;
+        };
+        auto load_col = [&](int c) __attribute__((always_inline)) {
+            const uint32_t off = column_offset(c);
+#pragma unroll
+            for (int t = 0; t < NH; ++t)
+                in[c % LA][t] = *reinterpret_cast<const V8*>(xb + off + 1024u * t);
+        };
+#pragma unroll
+        for (int c = 0; c < LA; ++c) load_col(c);
+        PairOperands<T16> po;
+        TileOperands<T16> ops;
+        if constexpr (K == 1024)
+            make_pair_operands<T16>(po, exp2);
+        else
+            make_tile_operands<T16, 2>(9, ops, exp2);
+        V8 held[4][NH];
+        // the reads of round nb, eight (K = 1024) or four (K = 512) at a time
+        auto read_back = [&](int nb, int first, int count) __attribute__((always_inline)) {
+#pragma unroll
+            for (int r = first; r < first + count; ++r) {
+                const int b = NH == 2 ? r / 16 : (nb & 1), s16 = r % 16;
+                yf[nb][r] = *reinterpret_cast<const V8*>(lds + area_at(b, lo) + (((4u * s16 + hi) ^ lo) << 4));
+            }
+        };
+        auto write_col = [&](int nb, int j, const V8 (&out)[NH]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int t = 0; t < NH; ++t) {
+                const int b = NH == 2 ? t : (nb & 1);
+                *reinterpret_cast<V8*>(lds + area_at(b, (uint32_t)j) + ((lane ^ (uint32_t)j) << 4)) = out[t];
             }
         };
         if constexpr (K == 1024) {
-            PairOperands<T16> po;
-            make_pair_operands<T16>(po, exp2);
-            V8 in[16][2];
-            auto load_col = [&](int nb, int j) {
-                const uint32_t col = min(n0 + CPW * wave + (uint32_t)(NBF * j + nb), N - 1u);
-#pragma unroll
-                for (int t = 0; t < 2; ++t)
-                    in[j][t] = *reinterpret_cast<const V8*>(Xt + ((uint64_t)col * K + 512u * t + 8u * lane));
+            // Columns go through in pairs (A = column 2p, B = column 2p + 1), sixteen MFMA slots per
+            // pair: stage 1 of A, stage 1 of B, stage 2 of A, stage 2 of B, four MFMAs each.  The
+            // thirty-two conversions, four LDS writes and four loads of a pair are placed between
+            // them by hand, every one at least three slots behind the MFMA whose result it reads, so
+            // that no instruction waits for a result (the compiler's own order finishes one column
+            // before it starts the next).  Slot k of pair p therefore also carries work of pair p - 1.
+            // What bounds the loop is instruction issue: a lone wavefront issues about one
+            // instruction every eight cycles (measured: an MFMA plus one vector or scalar
+            // instruction per 16-cycle MFMA slot is free, every further one adds eight cycles), and a
+            // column is eight MFMAs and some twenty-two other instructions.
+            struct Col {
+                f32x4 d0[2], d1[2];   // stage 1: tile 0 / tile 1, output half h
+                u32x4 a2[2];          // the same rounded to 16 bits: operand of stage 2
+                f32x4 s[2], d[2];     // stage 2: first / second half of the column
+                u32x4 o[2];           // rounded: what goes to LDS
             };
+            Col st[2][2];             // [pair parity][A, B]
+            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+            auto pack = [](float a, float b) __attribute__((always_inline)) -> uint32_t {
+                return __builtin_bit_cast(uint32_t, V2{(E)a, (E)b});
+            };
+            auto S1 = [&](Col& c, int col, int i) __attribute__((always_inline)) {
+                const int h = i >> 1;
+                if (i & 1)
+                    c.d1[h] = T16::mfma32(in[col % LA][1], po.g1[h], zero);
+                else
+                    c.d0[h] = T16::mfma32(in[col % LA][0], po.g1[h], zero);
+            };
+            auto C1 = [&](Col& c, int i) __attribute__((always_inline)) {
+                const int h = i >> 2, q = i & 3;
+                c.a2[h][q] = q < 2 ? pack(c.d0[h][2 * q], c.d0[h][2 * q + 1])
+                                   : pack(c.d1[h][2 * q - 4], c.d1[h][2 * q - 3]);
+            };
+            auto S2 = [&](Col& c, int i) __attribute__((always_inline)) {
+                const int h = i >> 1;
+                if (i & 1)
+                    c.d[h] = T16::mfma32(__builtin_bit_cast(V8, c.a2[h]), po.g2d, zero);
+                else
+                    c.s[h] = T16::mfma32(__builtin_bit_cast(V8, c.a2[h]), po.g2s, zero);
+            };
+            auto C2 = [&](Col& c, int i) __attribute__((always_inline)) {
+                const int h = i >> 2, q = i & 3;
+                if (q < 2)
+                    c.o[0][2 * h + q] = pack(c.s[h][2 * q], c.s[h][2 * q + 1]);
+                else
+                    c.o[1][2 * h + q - 2] = pack(c.d[h][2 * q - 4], c.d[h][2 * q - 3]);
+            };
+            // column `col` is complete: to LDS, or into `held` while the previous round is read back
+            auto WR = [&](Col& c, int col, int t) __attribute__((always_inline)) {
+                const int nb = col >> 4, j = col & 15;
+                const V8 v = __builtin_bit_cast(V8, c.o[t]);
+                if (nb > 0 && j < 4)
+                    held[j][t] = v;
+                else
+                    *reinterpret_cast<V8*>(lds + area_at(t, (uint32_t)j) + ((lane ^ (uint32_t)j) << 4)) = v;
+            };
+            auto LD = [&](int col, int t) __attribute__((always_inline)) {
+                if (col >= TOTAL) return;
+                in[col % LA][t] = *reinterpret_cast<const V8*>(xb + column_offset(col) + 1024u * t);
+            };
+            constexpr int PAIRS = TOTAL / 2;
 #pragma unroll
-            for (int j = 0; j < 16; ++j) load_col(0, j);
+            for (int p = 0; p <= PAIRS; ++p) {
+                const int a = 2 * p, b = 2 * p + 1;        // this pair's columns
+                Col& A = st[p & 1][0];
+                Col& B = st[p & 1][1];
+                Col& PA = st[(p + 1) & 1][0];              // the pair before
+                Col& PB = st[(p + 1) & 1][1];
+                const bool cur = p < PAIRS, prev = p > 0;
+                // The previous round is read back one read per slot, from the slot after its last
+                // column was written (slot 5 of the round's first pair) on: 32 slots.  The four
+                // columns that get finished meanwhile wait in `held` and are written in the second
+                // half of the round's third pair.
+                const int nbr = a >> 4, slot0 = 16 * (p - 8 * nbr);   // round, first slot of the pair in it
 #pragma unroll
-            for (int nb = 0; nb < NBF; ++nb) {
-                V8 hold[16];  // second halves (k >= 512) wait here while the first go through LDS
-#pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    V8 first_half;
-                    column_transform<T16>(in[j][0], in[j][1], po, first_half, hold[j]);
-                    if (nb + 1 < NBF) load_col(nb + 1, j);
-                    prefetch_w(nb, j);
-                    // area: [16 columns][64 chunks of 16 B], chunk q of column j stored at q ^ j
-                    *reinterpret_cast<V8*>(area + area_offset(j, lane)) = first_half;
+                for (int k = 0; k < 16; ++k) {
+                    if (cur) {
+                        if (k < 4) S1(A, a, k);
+                        else if (k < 8) S1(B, b, k - 4);
+                        else if (k < 12) S2(A, k - 8);
+                        else S2(B, k - 12);
+                    }
+                    // work of the pair before: the rest of its conversions and its LDS writes
+                    if (prev) {
+                        if (k == 0) { C2(PA, 4); C2(PA, 5); C2(PA, 6); }
+                        if (k == 1) { C2(PA, 7); WR(PA, a - 2, 0); WR(PA, a - 2, 1); }
+                        if (k == 2) { C2(PB, 0); C2(PB, 1); C2(PB, 2); }
+                        if (k == 3) { C2(PB, 3); C2(PB, 4); C2(PB, 5); }
+                        if (k == 4) { C2(PB, 6); C2(PB, 7); }
+                        if (k == 5) { WR(PB, b - 2, 0); WR(PB, b - 2, 1); }
+                    }
+                    if (cur) {
+                        if (k == 4) LD(a + LA, 0);
+                        if (k == 5) LD(a + LA, 1);
+                        if (k == 6) { C1(A, 0); C1(A, 1); C1(A, 2); }
+                        if (k == 7) { C1(A, 3); C1(A, 4); C1(A, 5); }
+                        if (k == 8) { C1(A, 6); C1(A, 7); LD(b + LA, 0); }
+                        if (k == 9) { LD(b + LA, 1); C1(B, 0); C1(B, 1); }
+                        if (k == 10) { C1(B, 2); C1(B, 3); C1(B, 4); }
+                        if (k == 11) { C1(B, 5); C1(B, 6); C1(B, 7); }
+                        if (k == 12) { C2(A, 0); C2(A, 1); C2(A, 2); }
+                        if (k == 13) C2(A, 3);
+                        // stage 0 of W behind the first round's columns: one piece per pair
+                        if (k == 14 && p >= 4 && p < 12) w_issue(0, 0, p - 4);
+                        const int at = slot0 + k;
+                        if (nbr > 0 && at >= 6 && at < 6 + RPR) read_back(nbr - 1, at - 6, 1);
+                        if (nbr > 0 && at >= 40 && at < 48) {
+                            const int jj = (at - 40) >> 1, t = (at - 40) & 1;
+                            *reinterpret_cast<V8*>(lds + area_at(t, (uint32_t)jj) + ((lane ^ (uint32_t)jj) << 4)) = held[jj][t];
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-                // LDS operations of one wavefront complete in order: no barrier between its own
-                // writes and reads
-#pragma unroll
-                for (int s = 0; s < KSTEPS / 2; ++s)
-                    yf[nb][s] = *reinterpret_cast<const V8*>(area + area_offset(lo, 4u * s + hi));
-#pragma unroll
-                for (int j = 0; j < 16; ++j)
-                    *reinterpret_cast<V8*>(area + area_offset(j, lane)) = hold[j];
-#pragma unroll
-                for (int s = 0; s < KSTEPS / 2; ++s)
-                    yf[nb][KSTEPS / 2 + s] =
-                        *reinterpret_cast<const V8*>(area + area_offset(lo, 4u * s + hi));
             }
-        } else {  // K = 512: a column is one tile
-            TileOperands<T16> ops;
-            make_tile_operands<T16, 2>(9, ops, exp2);
-            V8 in[16];
-            auto load_col = [&](int nb, int j) {
-                const uint32_t col = min(n0 + CPW * wave + (uint32_t)(NBF * j + nb), N - 1u);
-                in[j] = *reinterpret_cast<const V8*>(Xt + ((uint64_t)col * K + 8u * lane));
-            };
-#pragma unroll
-            for (int j = 0; j < 16; ++j) load_col(0, j);
-#pragma unroll
-            for (int nb = 0; nb < NBF; ++nb) {
-#pragma unroll
-                for (int j = 0; j < 16; ++j) {
+        } else {
+    #pragma unroll
+            for (int c = 0; c < TOTAL; ++c) {
+                const int nb = c >> 4, j = c & 15;
+                V8 out[NH];
+                if constexpr (K == 1024) {
+                    column_transform<T16>(in[j][0], in[j][1], po, out[0], out[1]);
+                } else {
                     f32x4 t2[2];
-                    tile_transform<T16>(in[j], ops, t2);
-                    V8 o;
-#pragma unroll
+                    tile_transform<T16>(in[j][0], ops, t2);
+    #pragma unroll
                     for (int t = 0; t < 2; ++t)
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) o[4 * t + r] = (E)t2[t][r];
-                    if (nb + 1 < NBF) load_col(nb + 1, j);
-                    prefetch_w(nb, j);
-                    *reinterpret_cast<V8*>(area + area_offset(j, lane)) = o;
+    #pragma unroll
+                        for (int r = 0; r < 4; ++r) out[0][4 * t + r] = (E)t2[t][r];
                 }
-#pragma unroll
-                for (int s = 0; s < KSTEPS; ++s)
-                    yf[nb][s] = *reinterpret_cast<const V8*>(area + area_offset(lo, 4u * s + hi));
+                if (c + 16 < TOTAL) load_col(c + 16);
+                if (c >= 8 && c < 16) w_issue(0, 0, c - 8);  // stage 0, behind the first round's columns
+                if (nb > 0 && j < 4) {
+                    read_back(nb - 1, j * (RPR / 4), RPR / 4);
+    #pragma unroll
+                    for (int t = 0; t < NH; ++t) held[j][t] = out[t];
+                    if (j == 3) {
+    #pragma unroll
+                        for (int jj = 0; jj < 4; ++jj) write_col(nb, jj, held[jj]);
+                    }
+                } else {
+                    write_col(nb, j, out);
+                }
             }
         }
+        read_back(NBF - 1, 0, RPR);
+        // This wavefront's reads have returned: its rows of stage buffers 1 .. 3 are free, and it
+        // requests its pieces of the stages the main loop expects to be in flight.
+        wait_lds();
+#pragma unroll
+        for (int g = 1; g < AHEAD; ++g)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) w_issue(g, g, i);
     }
 
-    // Every wavefront has finished with its area (stage buffer 3 may be filled from now on), and
-    // its pieces of stage 0 have landed (those of the AHEAD - 1 stages behind it may still be in
-    // flight).
+    // Stage 0 has landed (the 8 (AHEAD - 1) pieces behind it may still be in flight) and every
+    // wavefront has finished with its area.
     wait_vm(8 * (AHEAD - 1));
-    wait_lds();
     __builtin_amdgcn_s_barrier();
 
     // Fragment of row block mb, K step ks of a stage: row 16 mb + lo, chunk 4 ks + hi.  In the
@@ -252,58 +386,68 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     }
 
     // ---- output addressing ------------------------------------------------------------------------
-    // lane (hi, lo) of a row block owns rows 16 mb + 4 hi + r and the NBF adjacent columns
-    // NBF lo .. NBF lo + NBF - 1 of its wavefront's columns
+    // The transformed operand is the MFMA's A operand and W its B operand, so a lane's accumulator
+    // of fragment (mb, nb) is C[row 16 mb + lo][fragment column 4 hi + r]: over the NBF fragments
+    // lane (hi, lo) owns the 4 NBF adjacent columns CPL hi .. CPL hi + CPL - 1 of its wavefront's
+    // columns in row 16 mb + lo, element NBF r + nb from acc[mb][nb][r] - whole 16-byte stores.
     constexpr uint32_t esize = OUT_F32 ? 4u : 2u;
-    const uint32_t col = n0 + CPW * wave + (uint32_t)NBF * lo;
-    const uint32_t lane_off = (4u * hi * N + col) * esize;  // inside the row block, < 2^32
+    constexpr int CPL = 4 * NBF;                          // adjacent columns per lane
+    constexpr int EPS = 16 / (int)esize;                  // elements per 16-byte store
+    constexpr int PPF = CPL / EPS;                        // stores per 16-row fragment
+    constexpr int NPIECES = 4 * PPF;                      // stores per row block and lane
+    const uint32_t col = n0 + CPW * wave + (uint32_t)CPL * hi;
+    const uint32_t lane_off = (lo * N + col) * esize;     // inside a 16-row fragment, < 2^32
     unsigned char* const Cb = static_cast<unsigned char*>(C);
     // `mult` is the part of the scale that is not a power of two (1 for K = 1024 and the usual
     // n^-1/2, sqrt(2)-ish for K = 512); it is applied to the fp32 result at the store.  Row blocks
-    // of full column groups take the vector store path.
-    const bool cols_full = n0 + kCols <= N && (N % (uint32_t)NBF) == 0;
+    // of full column groups whose rows start on 16-byte boundaries take the vector store path.
+    const bool cols_full = n0 + kCols <= N && ((N * esize) & 15u) == 0;
 
-    // one store of the interleaved epilogue: rows 16 mb + 4 hi + r of a full row block
-    auto store_pair = [&](const f32x4 (&acc)[4][NBF], uint64_t block_base, int mb, int r)
-        __attribute__((always_inline)) {
+    // Store p of a full row block (fragment mb = p / PPF, 16-byte part q = p % PPF of the lane's
+    // columns), in steps so that its conversions can be spread over several K steps of the next
+    // block: `prepare(half)` rounds half of the part's values into `staged`, `commit` stores it.
+    u32x4 staged;
+    auto piece_value = [&](const f32x4 (&acc)[4][NBF], int p, int i) __attribute__((always_inline)) -> float {
+        const int e = (p % PPF) * EPS + i;                // element of the lane's CPL columns
+        return acc[p / PPF][e % NBF][e / NBF] * mult;
+    };
+    auto piece_prepare = [&](const f32x4 (&acc)[4][NBF], int p, int half) __attribute__((always_inline)) {
+        if constexpr (OUT_F32) {
+#pragma unroll
+            for (int i = 2 * half; i < 2 * half + 2; ++i)
+                staged[i] = __builtin_bit_cast(uint32_t, piece_value(acc, p, i));
+        } else {
+#pragma unroll
+            for (int i = 2 * half; i < 2 * half + 2; ++i)
+                staged[i] = __builtin_bit_cast(uint32_t, V2{(E)piece_value(acc, p, 2 * i), (E)piece_value(acc, p, 2 * i + 1)});
+        }
+    };
+    auto piece_commit = [&](uint64_t block_base, int p) __attribute__((always_inline)) {
         // streaming stores: C is not read again, and keeping it out of the L2 leaves the cache to
         // the operands
-        unsigned char* row_ptr = Cb + (block_base + (uint64_t)((16u * mb + r) * N) * esize);  // scalar
-        if constexpr (NBF == 2) {
-            const float v0 = acc[mb][0][r] * mult, v1 = acc[mb][1][r] * mult;
-            if (OUT_F32)
-                stream_store8(lane_off, u32x2{__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1)}, row_ptr);
-            else
-                stream_store4(lane_off, __builtin_bit_cast(uint32_t, V2{(E)v0, (E)v1}), row_ptr);
-        } else {
-            const float v0 = acc[mb][0][r] * mult, v1 = acc[mb][1][r] * mult, v2 = acc[mb][2][r] * mult,
-                        v3 = acc[mb][3][r] * mult;
-            if (OUT_F32)
-                stream_store16(lane_off, u32x4{__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1),
-                                               __builtin_bit_cast(uint32_t, v2), __builtin_bit_cast(uint32_t, v3)}, row_ptr);
-            else
-                stream_store8(lane_off, __builtin_bit_cast(u32x2, V4{(E)v0, (E)v1, (E)v2, (E)v3}), row_ptr);
-        }
+        unsigned char* frag_ptr = Cb + (block_base + (uint64_t)(16u * (uint32_t)(p / PPF) * N) * esize);  // scalar
+        stream_store16(lane_off, staged, frag_ptr, (p % PPF) * 16);
     };
     // the same for a row block at the edge of the matrix (masked, element by element)
     auto store_edge = [&](const f32x4 (&acc)[4][NBF], uint32_t row_base) __attribute__((always_inline)) {
 #pragma unroll
-        for (int mb = 0; mb < 4; ++mb)
+        for (int mb = 0; mb < 4; ++mb) {
+            const uint32_t row = row_base + 16u * mb + lo;
+            if (row >= m_end) continue;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const uint32_t row = row_base + 16u * mb + 4u * hi + r;
-                if (row >= m_end) continue;
+            for (int r = 0; r < 4; ++r)
 #pragma unroll
                 for (int nb = 0; nb < NBF; ++nb) {
-                    if (col + nb >= N) continue;
+                    const uint32_t c = col + (uint32_t)(NBF * r + nb);
+                    if (c >= N) continue;
                     const float v = acc[mb][nb][r] * mult;
-                    const uint64_t at = (uint64_t)row * N + col + nb;
+                    const uint64_t at = (uint64_t)row * N + c;
                     if (OUT_F32)
                         static_cast<float*>(C)[at] = v;
                     else
                         static_cast<E*>(C)[at] = (E)v;
                 }
-            }
+        }
     };
 
     // ---- one row block: KSTEPS K steps into `acc`, while `prev` (the previous row block's result,
@@ -356,18 +500,27 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
                         w_target(fill_slot, pi);
                     }
                     if (kk == 0)
-                        XMfma<T16>::first(acc[mb][nb], fr[ks & 3][mb], yf[nb][0]);
+                        XMfma<T16>::first_resident_a(acc[mb][nb], yf[nb][0], fr[ks & 3][mb]);
                     else
-                        XMfma<T16>::next(acc[mb][nb], fr[ks & 3][mb], yf[nb][kk]);
+                        XMfma<T16>::next_resident_a(acc[mb][nb], yf[nb][kk], fr[ks & 3][mb]);
                     // memory instructions in the shadow of the MFMA
                     if (m < 4) frag_read(fr[(ks + 2) & 3][m], fa, read_slot, m);
                     if (transfer) w_go(fill_kq, pi);
-                    // the previous block's sixteen stores, one per K step behind its last MFMA,
-                    // from the K step after the first stage's barrier on (a store costs the MFMA
-                    // stream about 16 cycles; two in a row cost more than twice that)
+                    // the previous block's stores, spread over the sixteen K steps that follow the
+                    // first stage's barrier, each behind the last MFMA of its K step (a store costs
+                    // the MFMA stream about 16 cycles; two in a row cost more than twice that): per
+                    // store one K step for each half of its conversions and one for the store
                     if (prev_full && kk >= 6 && kk < 22 && m == NM - 1) {
-                        const int e = kk - 6;
-                        store_pair(prev, prev_base, e >> 2, e & 3);
+                        constexpr int SPP = 16 / NPIECES;     // K steps per store: 4 (16-bit) or 2 (fp32)
+                        const int p = (kk - 6) / SPP, phase = (kk - 6) % SPP;
+                        if constexpr (SPP >= 4) {
+                            if (phase == 0) piece_prepare(prev, p, 0);
+                            if (phase == 1) piece_prepare(prev, p, 1);
+                            if (phase == 2) piece_commit(prev_base, p);
+                        } else {
+                            if (phase == 0) { piece_prepare(prev, p, 0); piece_prepare(prev, p, 1); }
+                            if (phase == 1) piece_commit(prev_base, p);
+                        }
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -397,9 +550,11 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     auto store_block = [&](f32x4 (&acc)[4][NBF], uint64_t base) __attribute__((always_inline)) {
         drain_mfma(acc);
 #pragma unroll
-        for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) store_pair(acc, base, mb, r);
+        for (int p = 0; p < NPIECES; ++p) {
+            piece_prepare(acc, p, 0);
+            piece_prepare(acc, p, 1);
+            piece_commit(base, p);
+        }
     };
     auto block_place = [&](uint32_t rbi, bool& full, uint64_t& base, uint32_t& row_base)
         __attribute__((always_inline)) {
@@ -409,7 +564,7 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     };
     if constexpr (NBF <= 2) {
         // Two accumulator sets take turns: a finished full block is stored during the next one.
-        static_assert(KSTEPS >= 22, "the sixteen stores take K steps 6 .. 21 of the next block");
+        static_assert(KSTEPS >= 22 && NPIECES <= 8, "the stores take K steps 6 .. 21 of the next block");
         f32x4 accA[4][NBF], accB[4][NBF];
         bool pend = false;        // accB holds a finished full row block that is not stored yet
         uint64_t pend_base = 0;

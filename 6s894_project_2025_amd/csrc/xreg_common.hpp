@@ -63,6 +63,37 @@ constexpr bool lds_patterns_conflict_free()
 }
 static_assert(lds_patterns_conflict_free(), "an LDS access pattern of the fused GEMM would serialise");
 
+// The 16-bit kernels' prologue area: 32 KB per wavefront in four 8 KB pieces, piece p of wavefront w
+// being the wavefront's own rows (16 w .. 16 w + 15) of stage buffer 1 + p for p < 3 and 8 KB of the
+// 32 KB behind the ring for p = 3.  A piece holds eight transformed columns of 512 k, column j' at
+// 1 KB j' with its 16-byte chunk q stored at q ^ j (j = the column's number in its round of 16).
+// Half (K = 1024) or round parity (K = 512) b, columns 8 h .. 8 h + 7 use piece b + 2 h, so the two
+// halves of a column are 32 KB apart: one address register and an immediate serve both.
+__host__ __device__ constexpr uint32_t area_piece_offset(uint32_t w, uint32_t p)
+{
+    return (p < 3u ? (1u + p) * (uint32_t)kStageBytes : (uint32_t)(kSlots * kStageBytes)) + w * 8192u;
+}
+static_assert(kSlots * kStageBytes + 4 * 8192 == kLdsBytes, "the fourth pieces fill the 32 KB behind the ring");
+constexpr bool area16_patterns_conflict_free()
+{
+    for (uint32_t b = 0; b < 2; ++b) {
+        // write: every lane stores chunk `lane` of column j; read: lane (hi, lo) takes chunk 4 s + hi of column lo
+        for (uint32_t j = 0; j < 16; ++j)
+            if (!lds::conflict_free_b128([=](uint32_t lane) {
+                    return area_piece_offset(0, b + 2u * (j >> 3)) + (j & 7u) * 1024u + ((lane ^ j) << 4);
+                }))
+                return false;
+        for (uint32_t s = 0; s < 16; ++s)
+            if (!lds::conflict_free_b128([=](uint32_t lane) {
+                    const uint32_t lo = lane & 15u, hi = lane >> 4;
+                    return area_piece_offset(0, b + 2u * (lo >> 3)) + (lo & 7u) * 1024u + (((4u * s + hi) ^ lo) << 4);
+                }))
+                return false;
+    }
+    return true;
+}
+static_assert(area16_patterns_conflict_free(), "an LDS access pattern of the 16-bit prologue would serialise");
+
 // Waits out the matrix-core pipeline before `acc` is read by anything but an MFMA.  Two statements:
 // the delay itself, which names no register (naming them lets the compiler set the operands up
 // with register copies *in front of* the statement, i.e. reads of the accumulators right behind
@@ -106,10 +137,12 @@ __device__ __forceinline__ void wait_vm(int n)
     if (n >= 0) asm volatile("s_waitcnt vmcnt(%0)" ::"i"(n) : "memory");
 }
 
-// A wavefront that has its SIMD to itself issues one instruction every four cycles, whatever the
-// instruction: between two 16-cycle MFMAs there is room for three others, waits and no-ops
-// included.  The statements below are therefore as few instructions as they can be, and are
-// placed by hand.
+// A wavefront that has its SIMD to itself issues roughly one instruction every eight cycles
+// (measured on loops of one v_mfma_f32_16x16x32 plus n independent instructions: 19 cycles for n = 0,
+// 20 for n = 1, 24 / 32 / 39 for n = 2 / 3 / 4, the same for vector and scalar arithmetic; one
+// ds_read_b128 per MFMA: 27 cycles; s_nop and satisfied waits cost next to nothing).  Between two
+// 16-cycle MFMAs one other instruction is free and every further one costs the MFMA stream eight
+// cycles, so the statements below are as few instructions as they can be, and are placed by hand.
 //
 // 16 bytes per lane from global memory straight into LDS, in two statements so that an MFMA can
 // stand between them (M0 must be written one instruction before the transfer that uses it):
@@ -177,9 +210,9 @@ __device__ __forceinline__ void cached_store8(uint32_t lane_off, u32x2 v, void* 
 }
 // (A store of more than 8 bytes still reads its data registers during the next cycles; the compiler
 // keeps ordinary code away from them for that long, but does not know what this statement is.)
-__device__ __forceinline__ void stream_store16(uint32_t lane_off, u32x4 v, void* base)
+__device__ __forceinline__ void stream_store16(uint32_t lane_off, u32x4 v, void* base, int offset = 0)
 {
-    asm volatile("global_store_dwordx4 %0, %1, %2 nt\n\ts_nop 1" :: "v"(lane_off), "v"(v), "s"(base) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, %2 offset:%3 nt\n\ts_nop 1" :: "v"(lane_off), "v"(v), "s"(base), "i"(offset) : "memory");
 }
 
 // Workgroup id -> (column group, M slice); false for an id past the last rectangle.
