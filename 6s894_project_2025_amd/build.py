@@ -58,7 +58,7 @@ PER_FILE_FLAGS = {
 # compiler inserts the wait states.  The build fails when anything but another MFMA reads an
 # assembly MFMA's destination within kResultWaitStates issue slots on any path.
 ISA_CHECKED = {"fused_gemm_xreg.hip", "fused_gemm_xreg_f32.hip", "fused_gemm_xreg_k2048.hip"}
-_MFMA_B_IN_AGPR = re.compile(r"^\s*v_mfma_\S+\s+v\[[0-9:]+\], (v\S+, a|a\S+, v)")  # A or B resident
+_MFMA_B_IN_AGPR = re.compile(r"^\s*v_mfma_\S+\s+v\[[0-9:]+\], v\S+, a")
 _AGPR_WRITE = re.compile(r"^\s*v_accvgpr_(write|mov)")
 _LABEL = re.compile(r"^([A-Za-z_][\w$]*):")
 _ANY_LABEL = re.compile(r"^([.A-Za-z_][\w$.]*):")

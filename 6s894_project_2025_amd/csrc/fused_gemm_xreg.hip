@@ -386,68 +386,58 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     }
 
     // ---- output addressing ------------------------------------------------------------------------
-    // The transformed operand is the MFMA's A operand and W its B operand, so a lane's accumulator
-    // of fragment (mb, nb) is C[row 16 mb + lo][fragment column 4 hi + r]: over the NBF fragments
-    // lane (hi, lo) owns the 4 NBF adjacent columns CPL hi .. CPL hi + CPL - 1 of its wavefront's
-    // columns in row 16 mb + lo, element NBF r + nb from acc[mb][nb][r] - whole 16-byte stores.
+    // lane (hi, lo) of a row block owns rows 16 mb + 4 hi + r and the NBF adjacent columns
+    // NBF lo .. NBF lo + NBF - 1 of its wavefront's columns
     constexpr uint32_t esize = OUT_F32 ? 4u : 2u;
-    constexpr int CPL = 4 * NBF;                          // adjacent columns per lane
-    constexpr int EPS = 16 / (int)esize;                  // elements per 16-byte store
-    constexpr int PPF = CPL / EPS;                        // stores per 16-row fragment
-    constexpr int NPIECES = 4 * PPF;                      // stores per row block and lane
-    const uint32_t col = n0 + CPW * wave + (uint32_t)CPL * hi;
-    const uint32_t lane_off = (lo * N + col) * esize;     // inside a 16-row fragment, < 2^32
+    const uint32_t col = n0 + CPW * wave + (uint32_t)NBF * lo;
+    const uint32_t lane_off = (4u * hi * N + col) * esize;  // inside the row block, < 2^32
     unsigned char* const Cb = static_cast<unsigned char*>(C);
     // `mult` is the part of the scale that is not a power of two (1 for K = 1024 and the usual
     // n^-1/2, sqrt(2)-ish for K = 512); it is applied to the fp32 result at the store.  Row blocks
-    // of full column groups whose rows start on 16-byte boundaries take the vector store path.
-    const bool cols_full = n0 + kCols <= N && ((N * esize) & 15u) == 0;
+    // of full column groups take the vector store path.
+    const bool cols_full = n0 + kCols <= N && (N % (uint32_t)NBF) == 0;
 
-    // Store p of a full row block (fragment mb = p / PPF, 16-byte part q = p % PPF of the lane's
-    // columns), in steps so that its conversions can be spread over several K steps of the next
-    // block: `prepare(half)` rounds half of the part's values into `staged`, `commit` stores it.
-    u32x4 staged;
-    auto piece_value = [&](const f32x4 (&acc)[4][NBF], int p, int i) __attribute__((always_inline)) -> float {
-        const int e = (p % PPF) * EPS + i;                // element of the lane's CPL columns
-        return acc[p / PPF][e % NBF][e / NBF] * mult;
-    };
-    auto piece_prepare = [&](const f32x4 (&acc)[4][NBF], int p, int half) __attribute__((always_inline)) {
-        if constexpr (OUT_F32) {
-#pragma unroll
-            for (int i = 2 * half; i < 2 * half + 2; ++i)
-                staged[i] = __builtin_bit_cast(uint32_t, piece_value(acc, p, i));
-        } else {
-#pragma unroll
-            for (int i = 2 * half; i < 2 * half + 2; ++i)
-                staged[i] = __builtin_bit_cast(uint32_t, V2{(E)piece_value(acc, p, 2 * i), (E)piece_value(acc, p, 2 * i + 1)});
-        }
-    };
-    auto piece_commit = [&](uint64_t block_base, int p) __attribute__((always_inline)) {
+    // one store of the interleaved epilogue: rows 16 mb + 4 hi + r of a full row block
+    auto store_pair = [&](const f32x4 (&acc)[4][NBF], uint64_t block_base, int mb, int r)
+        __attribute__((always_inline)) {
         // streaming stores: C is not read again, and keeping it out of the L2 leaves the cache to
         // the operands
-        unsigned char* frag_ptr = Cb + (block_base + (uint64_t)(16u * (uint32_t)(p / PPF) * N) * esize);  // scalar
-        stream_store16(lane_off, staged, frag_ptr, (p % PPF) * 16);
+        unsigned char* row_ptr = Cb + (block_base + (uint64_t)((16u * mb + r) * N) * esize);  // scalar
+        if constexpr (NBF == 2) {
+            const float v0 = acc[mb][0][r] * mult, v1 = acc[mb][1][r] * mult;
+            if (OUT_F32)
+                stream_store8(lane_off, u32x2{__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1)}, row_ptr);
+            else
+                stream_store4(lane_off, __builtin_bit_cast(uint32_t, V2{(E)v0, (E)v1}), row_ptr);
+        } else {
+            const float v0 = acc[mb][0][r] * mult, v1 = acc[mb][1][r] * mult, v2 = acc[mb][2][r] * mult,
+                        v3 = acc[mb][3][r] * mult;
+            if (OUT_F32)
+                stream_store16(lane_off, u32x4{__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1),
+                                               __builtin_bit_cast(uint32_t, v2), __builtin_bit_cast(uint32_t, v3)}, row_ptr);
+            else
+                stream_store8(lane_off, __builtin_bit_cast(u32x2, V4{(E)v0, (E)v1, (E)v2, (E)v3}), row_ptr);
+        }
     };
     // the same for a row block at the edge of the matrix (masked, element by element)
     auto store_edge = [&](const f32x4 (&acc)[4][NBF], uint32_t row_base) __attribute__((always_inline)) {
 #pragma unroll
-        for (int mb = 0; mb < 4; ++mb) {
-            const uint32_t row = row_base + 16u * mb + lo;
-            if (row >= m_end) continue;
+        for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t row = row_base + 16u * mb + 4u * hi + r;
+                if (row >= m_end) continue;
 #pragma unroll
                 for (int nb = 0; nb < NBF; ++nb) {
-                    const uint32_t c = col + (uint32_t)(NBF * r + nb);
-                    if (c >= N) continue;
+                    if (col + nb >= N) continue;
                     const float v = acc[mb][nb][r] * mult;
-                    const uint64_t at = (uint64_t)row * N + c;
+                    const uint64_t at = (uint64_t)row * N + col + nb;
                     if (OUT_F32)
                         static_cast<float*>(C)[at] = v;
                     else
                         static_cast<E*>(C)[at] = (E)v;
                 }
-        }
+            }
     };
 
     // ---- one row block: KSTEPS K steps into `acc`, while `prev` (the previous row block's result,
@@ -500,27 +490,18 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
                         w_target(fill_slot, pi);
                     }
                     if (kk == 0)
-                        XMfma<T16>::first_resident_a(acc[mb][nb], yf[nb][0], fr[ks & 3][mb]);
+                        XMfma<T16>::first(acc[mb][nb], fr[ks & 3][mb], yf[nb][0]);
                     else
-                        XMfma<T16>::next_resident_a(acc[mb][nb], yf[nb][kk], fr[ks & 3][mb]);
+                        XMfma<T16>::next(acc[mb][nb], fr[ks & 3][mb], yf[nb][kk]);
                     // memory instructions in the shadow of the MFMA
                     if (m < 4) frag_read(fr[(ks + 2) & 3][m], fa, read_slot, m);
                     if (transfer) w_go(fill_kq, pi);
-                    // the previous block's stores, spread over the sixteen K steps that follow the
-                    // first stage's barrier, each behind the last MFMA of its K step (a store costs
-                    // the MFMA stream about 16 cycles; two in a row cost more than twice that): per
-                    // store one K step for each half of its conversions and one for the store
+                    // the previous block's sixteen stores, one per K step behind its last MFMA,
+                    // from the K step after the first stage's barrier on (a store costs the MFMA
+                    // stream about 16 cycles; two in a row cost more than twice that)
                     if (prev_full && kk >= 6 && kk < 22 && m == NM - 1) {
-                        constexpr int SPP = 16 / NPIECES;     // K steps per store: 4 (16-bit) or 2 (fp32)
-                        const int p = (kk - 6) / SPP, phase = (kk - 6) % SPP;
-                        if constexpr (SPP >= 4) {
-                            if (phase == 0) piece_prepare(prev, p, 0);
-                            if (phase == 1) piece_prepare(prev, p, 1);
-                            if (phase == 2) piece_commit(prev_base, p);
-                        } else {
-                            if (phase == 0) { piece_prepare(prev, p, 0); piece_prepare(prev, p, 1); }
-                            if (phase == 1) piece_commit(prev_base, p);
-                        }
+                        const int e = kk - 6;
+                        store_pair(prev, prev_base, e >> 2, e & 3);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -550,11 +531,9 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     auto store_block = [&](f32x4 (&acc)[4][NBF], uint64_t base) __attribute__((always_inline)) {
         drain_mfma(acc);
 #pragma unroll
-        for (int p = 0; p < NPIECES; ++p) {
-            piece_prepare(acc, p, 0);
-            piece_prepare(acc, p, 1);
-            piece_commit(base, p);
-        }
+        for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) store_pair(acc, base, mb, r);
     };
     auto block_place = [&](uint32_t rbi, bool& full, uint64_t& base, uint32_t& row_base)
         __attribute__((always_inline)) {
@@ -564,7 +543,7 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
     };
     if constexpr (NBF <= 2) {
         // Two accumulator sets take turns: a finished full block is stored during the next one.
-        static_assert(KSTEPS >= 22 && NPIECES <= 8, "the stores take K steps 6 .. 21 of the next block");
+        static_assert(KSTEPS >= 22, "the sixteen stores take K steps 6 .. 21 of the next block");
         f32x4 accA[4][NBF], accB[4][NBF];
         bool pend = false;        // accB holds a finished full row block that is not stored yet
         uint64_t pend_base = 0;

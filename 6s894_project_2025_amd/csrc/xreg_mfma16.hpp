@@ -26,16 +26,6 @@ struct XMfma<BF16> {
     {
         asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
     }
-    // the same with the register-file-resident operand as A: c (+)= A_resident(16 x 32) * B(32 x 16),
-    // i.e. the transpose of the product above for the same two register operands
-    static __device__ __forceinline__ void first_resident_a(f32x4& c, bf16x8 a, bf16x8 b)
-    {
-        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=v"(c) : "a"(a), "v"(b));
-    }
-    static __device__ __forceinline__ void next_resident_a(f32x4& c, bf16x8 a, bf16x8 b)
-    {
-        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "a"(a), "v"(b));
-    }
     // adds a pair of adjacent 16-bit values to memory (performed in the L2, nothing returned)
     static __device__ __forceinline__ void add_pair_to_memory(uint32_t lane_off, uint32_t v, void* base)
     {
@@ -51,14 +41,6 @@ struct XMfma<F16> {
     static __device__ __forceinline__ void next(f32x4& c, f16x8 a, f16x8 b)
     {
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
-    }
-    static __device__ __forceinline__ void first_resident_a(f32x4& c, f16x8 a, f16x8 b)
-    {
-        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=v"(c) : "a"(a), "v"(b));
-    }
-    static __device__ __forceinline__ void next_resident_a(f32x4& c, f16x8 a, f16x8 b)
-    {
-        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "a"(a), "v"(b));
     }
     static __device__ __forceinline__ void add_pair_to_memory(uint32_t lane_off, uint32_t v, void* base)
     {
