@@ -1,14 +1,21 @@
 // Randomized Hadamard + FP8 (OCP E4M3FN) quantize epilogue (mi_rht_quant_fp8), gfx950.  The
 // reference has no FP8 path; the arithmetic convention is the one stated in include/mi_hadamard.h.
 //
-// Quantize kernel: same skeleton as the stand-alone transform (one 16-byte load per 8 elements,
-// two MFMA stages per 512-element tile, fp32 butterflies across tiles), with
-//   - the +-1 diagonal folded into the load as a sign-bit XOR (exact),
-//   - the result rounded to bf16 exactly as mi_fwht would store it (so the codes equal
-//     quantising mi_fwht's output), the row amax taken over those bf16 values by a lane
-//     reduction over the lanes that share a row,
+// Quantize kernel: the stand-alone transform's tiles (one 16-byte load per 8 elements, two MFMA
+// stages per 512-element tile) with
+//   - the +-1 diagonal folded into the load as a sign-bit XOR (exact), its masks kept in LDS (they
+//     are the same for every row),
+//   - for n > 512 the butterflies between a row's tiles folded into the second MFMA stage: output
+//     tile o is the sum over tile pairs of [a(2i); a(2i+1)] contracted with [+-G2; +-G2], the signs
+//     (-1)^popcount(o & tile), accumulated on the matrix cores (no vector add/sub at all),
+//   - the result rounded to bf16 as mi_fwht would store it, the row amax taken on the fp32 values
+//     by a lane reduction over the lanes that share a row,
 //   - v_cvt_pk_fp8_f32 for the narrowing (hardware RNE to E4M3FN), 8 codes = one 8-byte store.
-// Bandwidth-bound: 2 bytes in, 1 byte (+ 4 bytes per row) out per element.
+// The kernel is bound by vector-instruction issue, not by memory (the same loads and stores without
+// arithmetic take a third of the time at [8192, 4096]): it is kept at four wavefronts per SIMD
+// (at most 128 registers: simple two-operand instructions then issue every 2.2 cycles per SIMD,
+// conversions and three-operand ones every 4.3; with three wavefronts 2.7 and 5.2) and at as few
+// vector instructions per element as the arithmetic allows.
 #include <type_traits>
 
 #include "fwht_device.hpp"
@@ -60,27 +67,42 @@ rht_quant_fp8_kernel(const __bf16* __restrict__ x, const int8_t* __restrict__ si
 {
     const uint64_t first = (uint64_t)blockIdx.x * 4u + (threadIdx.x >> 6);
     const uint64_t stride = (uint64_t)gridDim.x * 4u;
-    if (first >= num_steps) return;
+    __shared__ u32x4 flip_lds[NT][64];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t n = 1u << p;
 
     TileOperands<BF16> ops;
     make_tile_operands<BF16, 2>(p, ops, exp2);
 
-    // sign-bit masks of this lane's 8 columns in each tile of a step; the column pattern repeats
-    // from step to step (a step covers a whole number of rows)
-    u32x4 flip[NT];
+    // stage-2 operands that also fold the tile index bits: [s G2; s' G2] for the sign pairs
+    // (+,+), (+,-), (-,-), (-,+)
+    bf16x8 gfold[4];
 #pragma unroll
-    for (int c = 0; c < NT; ++c) {
-        const uint32_t col = (uint32_t)((first * NT + c) * 512u + 8u * lane) & (n - 1u);
-        const u32x2 sg = *reinterpret_cast<const u32x2*>(sign + col);  // 8 int8, +1 / -1
+    for (int j = 0; j < 4; ++j) {
+        gfold[0][j] = ops.g2[j]; gfold[0][4 + j] = ops.g2[j];
+        gfold[1][j] = ops.g2[j]; gfold[1][4 + j] = -ops.g2[j];
+        gfold[2][j] = -ops.g2[j]; gfold[2][4 + j] = -ops.g2[j];
+        gfold[3][j] = -ops.g2[j]; gfold[3][4 + j] = ops.g2[j];
+    }
+    // sign-bit masks of a lane's 8 columns in each tile of a step: the column pattern is the same
+    // for every step (a step covers a whole number of rows), so the first wavefront leaves them in
+    // LDS for all four
+    if (threadIdx.x < 64u) {
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const uint32_t s2 = (w < 2 ? sg[0] : sg[1]) >> (16 * (w & 1));
-            // byte 0 -> element 2w, byte 1 -> element 2w+1; -1 = 0xff has bit 7 set
-            flip[c][w] = ((s2 & 0x80u) << 8) | ((s2 & 0x8000u) << 16);
+        for (int c = 0; c < NT; ++c) {
+            const uint32_t col = (uint32_t)((first * NT + c) * 512u + 8u * lane) & (n - 1u);
+            const u32x2 sg = *reinterpret_cast<const u32x2*>(sign + col);  // 8 int8, +1 / -1
+            u32x4 f;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t s2 = (w < 2 ? sg[0] : sg[1]) >> (16 * (w & 1));
+                f[w] = ((s2 & 0x80u) << 8) | ((s2 & 0x8000u) << 16);
+            }
+            flip_lds[c][lane] = f;
         }
     }
+    __syncthreads();
+    if (first >= num_steps) return;
     // lanes that share a row: lane bit i carries element bit 3 + i, so the low min(6, p - 3)
     // lane bits index inside a row
     const uint32_t row_lane_bits = p >= 9u ? 6u : p - 3u;
@@ -93,33 +115,59 @@ rht_quant_fp8_kernel(const __bf16* __restrict__ x, const int8_t* __restrict__ si
             const uint64_t off = (step * NT + c) * 512u + 8u * lane;
             u32x4 bits = {0u, 0u, 0u, 0u};
             if (XB > 0 || off + 8u <= total) bits = *reinterpret_cast<const u32x4*>(x + off);
-            in[c] = __builtin_bit_cast(bf16x8, bits ^ flip[c]);
+            in[c] = __builtin_bit_cast(bf16x8, bits ^ flip_lds[c][lane]);
         }
         __builtin_amdgcn_sched_barrier(0);
 
-        f32x4 acc[NT][2];
-#pragma unroll
-        for (int c = 0; c < NT; ++c) tile_transform<BF16>(in[c], ops, acc[c]);
-        cross_tile_butterflies<NT, XB>(acc);
-
-        // round to bf16 (the pre-quant values).  Rounding is monotonic, so the row maximum of the
-        // rounded magnitudes is the rounded maximum of the fp32 magnitudes: one v_max3 per two
-        // values, one rounding per row.
         bf16x8 y[NT];
         float amax[NT];
+        if constexpr (XB > 0) {
+            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+            bf16x4 a2[NT][2];
 #pragma unroll
-        for (int c = 0; c < NT; ++c) {
-            float m = 0.0f;
+            for (int c = 0; c < NT; ++c)
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                f32x4 v = acc[c][t];
-                if (MUL) v = v * mult;
+                for (int t = 0; t < 2; ++t) a2[c][t] = narrow4<BF16>(BF16::mfma32(in[c], ops.g1[t], zero));
 #pragma unroll
-                for (int r = 0; r < 4; ++r) y[c][4 * t + r] = (__bf16)v[r];
-                m = fmaxf(fmaxf(__builtin_fabsf(v[0]), __builtin_fabsf(v[1])), m);
-                m = fmaxf(fmaxf(__builtin_fabsf(v[2]), __builtin_fabsf(v[3])), m);
+            for (int o = 0; o < NT; ++o) {
+                float m = 0.0f;
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    f32x4 d = zero;
+#pragma unroll
+                    for (int pr = 0; pr < NT / 2; ++pr) {
+                        bf16x8 A;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) { A[i] = a2[2 * pr][t][i]; A[4 + i] = a2[2 * pr + 1][t][i]; }
+                        const bool m0 = __builtin_popcount(o & (2 * pr)) & 1, m1 = __builtin_popcount(o & (2 * pr + 1)) & 1;
+                        d = BF16::mfma32(A, gfold[(m0 ? 2 : 0) + (m1 != m0 ? 1 : 0)], d);
+                    }
+                    if (MUL) d = d * mult;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) y[o][4 * t + r] = (__bf16)d[r];
+                    m = fmaxf(fmaxf(__builtin_fabsf(d[0]), __builtin_fabsf(d[1])), m);
+                    m = fmaxf(fmaxf(__builtin_fabsf(d[2]), __builtin_fabsf(d[3])), m);
+                }
+                amax[o] = m;
             }
-            amax[c] = m;
+        } else {
+            f32x4 acc[NT][2];
+#pragma unroll
+            for (int c = 0; c < NT; ++c) tile_transform<BF16>(in[c], ops, acc[c]);
+#pragma unroll
+            for (int c = 0; c < NT; ++c) {
+                float m = 0.0f;
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    f32x4 v = acc[c][t];
+                    if (MUL) v = v * mult;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) y[c][4 * t + r] = (__bf16)v[r];
+                    m = fmaxf(fmaxf(__builtin_fabsf(v[0]), __builtin_fabsf(v[1])), m);
+                    m = fmaxf(fmaxf(__builtin_fabsf(v[2]), __builtin_fabsf(v[3])), m);
+                }
+                amax[c] = m;
+            }
         }
         if (XB > 0) {  // one row spans all NT tiles: fold the tiles, then one lane reduction
             float m = amax[0];
@@ -158,28 +206,10 @@ rht_quant_fp8_kernel(const __bf16* __restrict__ x, const int8_t* __restrict__ si
                 pk = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], pk, true);
                 codes[c][w] = (uint32_t)pk;
             }
-            if (XB == 0) __builtin_nontemporal_store(codes[c], reinterpret_cast<u32x2*>(q + off));
+            // streaming stores: the codes are not read again here (an exchange between neighbouring
+            // lanes would make them 16-byte stores, but costs more vector instructions than it saves)
+            __builtin_nontemporal_store(codes[c], reinterpret_cast<u32x2*>(q + off));
             if (y_out) *reinterpret_cast<bf16x8*>(y_out + off) = y[c];
-        }
-        if constexpr (XB > 0) {
-            // Whole rows: neighbouring lanes trade 8 codes so that the even lane stores 16
-            // consecutive bytes of tile c and the odd lane 16 of tile c+1: half as many store
-            // instructions, each covering two 512-byte runs.  (Streaming stores: the codes are
-            // not read again here.)
-            const bool odd = lane & 1u;
-#pragma unroll
-            for (int c = 0; c < NT; c += 2) {
-                u32x2 give, got;
-#pragma unroll
-                for (int w = 0; w < 2; ++w) {
-                    give[w] = odd ? codes[c][w] : codes[c + 1][w];
-                    got[w] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)give[w], 0xB1, 0xf, 0xf, false);
-                }
-                const u32x4 out = odd ? u32x4{got[0], got[1], codes[c + 1][0], codes[c + 1][1]}
-                                      : u32x4{codes[c][0], codes[c][1], got[0], got[1]};
-                const uint64_t at = (step * NT + c + (odd ? 1u : 0u)) * 512u + 16u * (lane >> 1);
-                __builtin_nontemporal_store(out, reinterpret_cast<u32x4*>(q + at));
-            }
         }
     }
 }
@@ -190,13 +220,13 @@ int launch_quant(const void* x, const int8_t* sign, void* q, float* rs, void* y_
 {
     // a wavefront's steps must all see the same column pattern: with NT tiles per step a step
     // covers NT * 512 elements, a whole number of rows for every n <= NT * 512 (true here)
-    // Grid: one step per wavefront up to one and a half times what the chip holds at once, four steps
-    // per wavefront for large inputs, that many wavefronts in between.  (With 4096 wavefronts of
-    // exactly two steps each, everybody loads, computes and stores in phase: [8192, 4096] took
-    // 19.6 us instead of 18.5.)
+    // Grid: the kernel keeps four wavefronts per SIMD (at most 128 registers), 4096 on the chip; one
+    // step per wavefront up to that many, and exactly that many wavefronts, each walking its share of
+    // the steps, beyond (for [8192, 4096]: two rows per wavefront on every SIMD alike; workgroups
+    // that only start when others have finished cost about 1.5 us each at this size).
     uint64_t waves = num_steps;
-    const uint64_t resident = 256u * 24u;
-    if (waves > resident) waves = (num_steps + 3u) / 4u > resident ? (num_steps + 3u) / 4u : resident;
+    const uint64_t resident = 256u * 16u;
+    if (waves > resident) waves = resident;
     const uint64_t blocks = (waves + 3u) / 4u;
     if (blocks > 0x7fffffffull) return MI_ERR_SHAPE;
     if (os.mult == 1.0f)
