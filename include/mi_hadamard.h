@@ -97,6 +97,16 @@ int mi_fused_ht_gemv(const void* W, const void* X, void* Y, uint32_t M, uint32_t
  *   with 32-bit byte offsets: W larger than 4 GiB, or N >= 2^24, is MI_ERR_SHAPE.
  * K = 4096 enqueues two kernels on `stream` for every dtype (the second adds to what the first
  * stored in C, so nothing else may touch C between them); every other case is one kernel.
+ * Precision at K = 4096: each kernel accumulates its half of the K range in fp32.  With MI_F32
+ * output the halves meet in fp32 (one more fp32 rounding than a single pass).  With 16-bit output
+ * the first kernel stores its half-K sum P0 rounded to the 16-bit type and the second adds its own
+ * half P1, rounded to 16 bits, in 16-bit arithmetic (a packed add performed by the L2; masked edge
+ * blocks add in fp32 and round once), so the result carries up to three 16-bit roundings instead of
+ * the single one of K <= 2048:
+ *     |C - exact| <= ulp16(P0) + ulp16(P1) + ulp16(C),   ulp16(v) = the 16-bit type's spacing at |v|,
+ * which is a larger *relative* error than usual when P0 and P1 nearly cancel, and for MI_F16 a half-K
+ * sum beyond 65504 becomes infinite even if the total is representable.  Callers that need the
+ * single rounding ask for MI_F32 output.
  */
 int mi_fused_ht_gemm(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
                      int in_dtype, int out_dtype, float scale, void* stream);

@@ -405,3 +405,54 @@ def test_gemm_register_resident_kernels_are_deterministic(pkg, oracle, dt, K):
                 bad = (_bits(again) != _bits(first)).nonzero()
                 pytest.fail(f"launch {i} differs from launch 0 in {len(bad)} elements, first at {bad[0].tolist()} "
                             f"({dt}, K={K}, out {od})")
+
+
+def slack_of(Wd, Y, eps16):
+    # The kernel rounds the transformed operand H(x) to 16 bits (relative error eps16 per element,
+    # independent between elements): the sum over K of |w y| eps16 would be the worst case, its
+    # root-mean-square size is smaller by sqrt(K); six times that is never reached in practice.
+    K = Wd.shape[1]
+    return 6.0 * eps16 * (Wd.double().abs() @ Y.abs().t()) / K ** 0.5
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_gemm16_k4096_sixteen_bit_output_contract(pkg, oracle, dt):
+    # K = 4096 with 16-bit output runs two passes that meet in C in 16-bit arithmetic: the stated bound
+    # is ulp16(P0) + ulp16(P1) + ulp16(C) around the exact result, with P0, P1 the half-K sums.  Checked
+    # against the fp32-output result (both halves in fp32) on ordinary data and on data whose halves
+    # nearly cancel: W[:, 2048:] = -W[:, :2048] + small, and columns of X whose second half is zero, so
+    # that H(x)[2048:] = H(x)[:2048] and P1 = -P0 + small.
+    K, M, N = 4096, 300, 200                       # edge blocks (fp32 add) and full blocks (16-bit add)
+    eps16 = 2.0 ** (-8 if dt == torch.bfloat16 else -11)   # half the relative spacing of the type
+
+    def ulp(v):                                     # spacing of the 16-bit type at |v| (normal range)
+        return torch.pow(2.0, torch.floor(torch.log2(v.abs().clamp_min(1e-30)))) * (2.0 * eps16)
+
+    g = torch.Generator().manual_seed(11)
+    for case in ("random", "cancelling"):
+        W = torch.randn(M, K, generator=g)
+        Xt = torch.randn(N, K, generator=g)
+        if case == "cancelling":
+            W[:, 2048:] = -W[:, :2048] + 0.01 * torch.randn(M, 2048, generator=g)
+            Xt[:, 2048:] = 0.0
+        Wd, Xd = W.to(dt).cuda(), Xt.to(dt).cuda()
+        C32 = pkg.fused_ht_gemm(Wd, Xd, out_dtype=torch.float32)
+        C16 = pkg.fused_ht_gemm(Wd, Xd, out_dtype=dt)
+        torch.cuda.synchronize()
+        assert torch.isfinite(C16.float()).all()
+        # the halves, from the library's own transform (fp64 products on the device)
+        Y = pkg.hadamard_transform(Xd.float(), 1.0 / 64.0).double()
+        P0 = Wd[:, :2048].double() @ Y[:, :2048].t()
+        P1 = Wd[:, 2048:].double() @ Y[:, 2048:].t()
+        exact = P0 + P1
+        # fp32 output: both halves meet in fp32; what is left is the 16-bit rounding of the operand
+        assert ((C32.double() - exact).abs() <= slack_of(Wd, Y, eps16) + 1e-5 * exact.abs()).all()
+        bound = ulp(P0) + ulp(P1) + ulp(exact)
+        # (the operand H(x) itself is rounded to 16 bits inside the kernel: allow for that too, one
+        # part in 2^8 or 2^11 of the typical magnitude of a half-K sum's terms)
+        slack = slack_of(Wd, Y, eps16)
+        worst = ((C16.double() - exact).abs() - bound - slack).max().item()
+        assert worst <= 0.0, (case, worst)
+        if case == "cancelling":
+            # the point of the case: the partial sums dwarf the result
+            assert (P0.abs().median() > 20 * exact.abs().median()).item()
