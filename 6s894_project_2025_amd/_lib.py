@@ -30,6 +30,7 @@ SIGNATURES = {
 PROBE_LIB_PATH = os.path.join(HERE, "libmi_probe.so")
 PROBE_SIGNATURES = {
     "mi_probe_mfma_rate": (_i, [_i, _i, _u32, _u32, _vp, _vp, _vp]),
+    "mi_probe_issue_rate": (_i, [_i, _i, _i, _u32, _u32, _vp, _vp, _vp, _vp]),
 }
 
 _lib = None

@@ -7,6 +7,8 @@ Sub-commands (run from the repository root)::
     python -m 6s894_project_2025_amd.harness plot P.csv [--out-dir plots]
     python -m 6s894_project_2025_amd.harness gemv  [--iters 100] [--out-prefix P]
     python -m 6s894_project_2025_amd.harness mfma  [--steps 4096]
+    python -m 6s894_project_2025_amd.harness issue
+    python -m 6s894_project_2025_amd.harness power [--seconds 1.5]
 
 ``fwht`` follows the protocol of the reference's bench/bench.py: a registry of in-place cases
 (add-one roofline proxies around the transform, :96-103), a correctness pass of every case with
@@ -27,6 +29,11 @@ between the two reported like :694-703.
 ``gemv`` is the benchmark half of fused_ht/fwht_gemv_fusion.cu's main() (:643-653): its seven
 (M, N, B) shapes, fused HT+GEMV against transform-then-GEMM, with its FLOP count and its
 memory-traffic model (:576-588).
+
+``mfma``, ``issue`` and ``power`` are measurement aids with no counterpart in the reference: the
+matrix-core rate and clock the chip sustains, what a SIMD can issue beside its MFMAs and per vector
+instruction kind, and package power and shader clock while each kernel runs (read from the amdgpu
+sysfs files).
 """
 from __future__ import annotations
 
@@ -36,6 +43,7 @@ import functools
 import json
 import math
 import sys
+import time
 from dataclasses import dataclass, field
 from datetime import datetime
 from typing import Any, Callable
@@ -297,6 +305,137 @@ def run_mfma_probe(steps: int = 4096, repeats: int = 20) -> list[dict[str, Any]]
     return rows
 
 
+ISSUE_KINDS = {"v_add_f32": 0, "v_cvt_pk_bf16_f32": 1, "s_add_u32": 2, "ds_read_b128": 3,
+               "v_cvt_pk_fp8_f32": 4, "v_max3_f32": 5, "v_lshlrev_b32": 6}
+
+
+def run_issue_probe(reps: int = 1000) -> list[dict[str, Any]]:
+    """What a SIMD issues per cycle (``mi_probe_issue_rate``): the cost of a group of one MFMA plus n
+    other instructions on a lone wavefront (the regime of the register-resident GEMM kernels), and
+    the cycles per vector instruction and SIMD at one to four wavefronts per SIMD (the regime of the
+    streaming kernels)."""
+    from . import _lib
+
+    lib = _lib.load_probe()
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    src = torch.rand(256 * 8, device=dev) + 0.5
+    out = torch.zeros(1024, device=dev)
+    cycles = torch.zeros(16, dtype=torch.int64, device=dev)
+    rows = []
+
+    def run(mode, kind, n, wps):
+        for _ in range(2):
+            _lib.check(lib.mi_probe_issue_rate(mode, ISSUE_KINDS[kind], n, wps, reps, src.data_ptr(),
+                                               out.data_ptr(), cycles.data_ptr(), stream), "issue probe")
+        torch.cuda.synchronize()
+        return cycles[:4 * wps].max().item()
+
+    for kind in ("v_add_f32", "v_cvt_pk_bf16_f32", "s_add_u32", "ds_read_b128"):
+        for n in range(0, 5):
+            c = run(0, kind, n, 1) / (8.0 * reps)
+            rows.append({"mode": "mfma_plus_n", "kind": kind, "n": n, "cycles_per_group": c})
+            print(f"lone wavefront, [1 MFMA 16x16x32 + {n} x {kind}]: {c:6.2f} cycles per group")
+    for kind in ("v_add_f32", "v_cvt_pk_bf16_f32", "v_max3_f32", "v_lshlrev_b32", "v_cvt_pk_fp8_f32"):
+        for wps in (1, 2, 3, 4):
+            c = run(1, kind, 8, wps) / (64.0 * reps * wps)
+            rows.append({"mode": "stream", "kind": kind, "waves_per_simd": wps, "cycles_per_instruction_per_simd": c})
+            print(f"{wps} wavefront(s) per SIMD, {kind} back to back: {c:5.2f} cycles per instruction per SIMD")
+    return rows
+
+
+def _read_power_and_clock() -> dict[str, Any]:
+    """Package power (W) and the current shader clock level from the amdgpu sysfs files, which an
+    ordinary user may read; empty where the files are absent."""
+    import glob
+
+    out: dict[str, Any] = {}
+    for path in glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input"):
+        try:
+            with open(path) as f:
+                out["watts"] = int(f.read()) / 1e6
+            with open(path.replace("power1_input", "power1_cap")) as f:
+                out["cap_watts"] = int(f.read()) / 1e6
+        except (OSError, ValueError):
+            pass
+    for path in glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"):
+        try:
+            with open(path) as f:
+                cur = [line for line in f.read().splitlines() if "*" in line]
+            if cur:
+                out["sclk_mhz"] = int("".join(ch for ch in cur[0].split(":")[1] if ch.isdigit()))
+        except (OSError, ValueError, IndexError):
+            pass
+    return out
+
+
+def run_power(seconds: float = 1.5) -> list[dict[str, Any]]:
+    """Package power and shader clock while each kernel runs back to back for ``seconds``, next to
+    its launch-to-launch time: a matrix-core kernel that sits at the power cap runs at whatever
+    clock the cap allows, so its rate is set by the energy a launch needs, not by its cycle count."""
+    import threading
+
+    from . import fp8_gemm_rowscale, fused_ht_gemm, rht_quant_fp8
+
+    dev = torch.device("cuda:0")
+
+    def watch(name, fn):
+        samples: list[dict[str, Any]] = []
+        stop = threading.Event()
+
+        def sampler():
+            while not stop.is_set():
+                samples.append(_read_power_and_clock())
+                time.sleep(0.05)
+        th = threading.Thread(target=sampler)
+        th.start()
+        t0 = time.time()
+        while time.time() - t0 < seconds:
+            for _ in range(50):
+                fn()
+            torch.cuda.synchronize()
+        stop.set()
+        th.join()
+        ms, _ = steady_window_ms(fn, 30, 20.0)   # timed after the sampler has stopped
+        tail = [x for x in samples[len(samples) // 2:] if "watts" in x]
+        row = {"kernel": name, "us_per_launch": ms * 1e3}
+        if tail:
+            row.update({"watts": sum(x["watts"] for x in tail) / len(tail), "cap_watts": tail[-1].get("cap_watts"),
+                        "sclk_mhz": sum(x.get("sclk_mhz", 0) for x in tail) / len(tail)})
+        print(f"{name:48s} {row['us_per_launch']:9.2f} us  {row.get('watts', float('nan')):7.0f} W of "
+              f"{row.get('cap_watts', float('nan')):.0f}  {row.get('sclk_mhz', float('nan')):6.0f} MHz")
+        return row
+
+    rows = [dict(kernel="idle", **_read_power_and_clock())]
+    print("idle:", rows[0])
+    g = torch.Generator(device=dev).manual_seed(0)
+    W = torch.randn(4096, 1024, device=dev, generator=g)
+    X = torch.randn(4096, 1024, device=dev, generator=g)
+    Wb, Xb = W.to(torch.bfloat16), X.to(torch.bfloat16)
+    rows.append(watch("fused HT->GEMM bf16 K=1024 M=N=4096", lambda: fused_ht_gemm(Wb, Xb)))
+    rows.append(watch("vendor GEMM bf16 K=1024 M=N=4096 (no transform)", lambda: torch.matmul(Wb, Xb.t())))
+    rows.append(watch("fused HT->GEMM fp32 K=1024 M=N=4096", lambda: fused_ht_gemm(W, X)))
+    W4 = torch.randn(4096, 4096, device=dev, generator=g).to(torch.bfloat16)
+    X4 = torch.randn(4096, 4096, device=dev, generator=g).to(torch.bfloat16)
+    rows.append(watch("fused HT->GEMM bf16 K=4096 M=N=4096", lambda: fused_ht_gemm(W4, X4)))
+    rows.append(watch("vendor GEMM bf16 K=4096 M=N=4096 (no transform)", lambda: torch.matmul(W4, X4.t())))
+    xb = torch.randn(16384, 4096, device=dev, generator=g).to(torch.bfloat16)
+    rows.append(watch("FWHT bf16 [16384, 4096] in place", lambda: hadamard_transform(xb, inplace=True)))
+    xa = torch.randn(8192, 4096, device=dev, generator=g).to(torch.bfloat16)
+    sign = (1 - 2 * torch.randint(0, 2, (4096,))).to(torch.int8).to(dev)
+    wq = (torch.randn(14336, 4096, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    qx, sx = rht_quant_fp8(xa, sign)
+    qw, sw = rht_quant_fp8(wq, sign)
+    rows.append(watch("RHT + FP8 quantize [8192, 4096]", lambda: rht_quant_fp8(xa, sign)))
+    rows.append(watch("FP8 GEMM [8192, 4096] x [14336, 4096]^T", lambda: fp8_gemm_rowscale(qx, sx, qw, sw)))
+    try:
+        rows.append(watch("vendor row-scaled FP8 GEMM, same operands", lambda: torch._scaled_mm(
+            qx, qw.t(), scale_a=sx.view(-1, 1), scale_b=sw.view(1, -1), out_dtype=torch.bfloat16)))
+    except Exception as ex:  # not every torch build exposes it
+        print("vendor row-scaled FP8 GEMM unavailable:", str(ex)[:80])
+    return rows
+
+
 def plot_fused(csv_path: str, out_dir: str = "plots") -> list[str]:
     """Figures and a table from the sweep CSV, the counterpart of the five outputs of
     fused_ht/plot_results.py (speed-up by dimension :23-68, rate / time comparison :72-125, speed-up
@@ -412,6 +551,9 @@ def main(argv=None) -> int:
     p5.add_argument("--out-prefix", default=None)
     p4 = sub.add_parser("mfma")
     p4.add_argument("--steps", type=int, default=4096)
+    sub.add_parser("issue")
+    p6 = sub.add_parser("power")
+    p6.add_argument("--seconds", type=float, default=1.5)
     p3 = sub.add_parser("plot")
     p3.add_argument("csv")
     p3.add_argument("--out-dir", default="plots")
@@ -425,6 +567,12 @@ def main(argv=None) -> int:
         return 2
     if args.cmd == "mfma":
         run_mfma_probe(args.steps)
+        return 0
+    if args.cmd == "issue":
+        run_issue_probe()
+        return 0
+    if args.cmd == "power":
+        run_power(args.seconds)
         return 0
     if args.cmd == "gemv":
         run_gemv(iters=args.iters, out_prefix=args.out_prefix)

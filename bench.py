@@ -46,31 +46,49 @@ RAMP_MS = 60.0  # untimed device time before a matrix-core-bound kernel is timed
 BASELINE_METRIC = "fused HT+GEMM TFLOP/s (K=1024,M=N=4096) + standalone FWHT HBM GB/s vs peak"
 
 
-def kernel_sources_digest() -> str:
-    """sha256 over the HIP sources the timed kernels are built from (names and contents)."""
+_SHARED_HEADERS = ("common.hpp", "fwht_device.hpp")
+_XREG_HEADERS = _SHARED_HEADERS + ("xreg_common.hpp", "lds_layout.hpp")
+# which HIP sources each measured kernel is built from: a traffic figure is reported only while
+# these are what they were when it was measured
+TRAFFIC_SOURCES = {
+    "fused_ht_gemm_bf16": _XREG_HEADERS + ("xreg_mfma16.hpp", "fused_gemm_xreg.hip"),
+    "fused_ht_gemm_bf16_K2048_M4096_N4096": _XREG_HEADERS + ("xreg_mfma16.hpp", "fused_gemm_xreg_k2048.hip"),
+    "fused_ht_gemm_bf16_K4096_M4096_N4096": _XREG_HEADERS + ("xreg_mfma16.hpp", "fused_gemm_xreg_k2048.hip"),
+    "fused_ht_gemm_f32": _XREG_HEADERS + ("fused_gemm_xreg_f32.hip",),
+    "fwht_bf16_16384x4096": _SHARED_HEADERS + ("hadamard_device.hpp", "fwht.hip"),
+    "fwht_bf16_2^30_n4096": _SHARED_HEADERS + ("hadamard_device.hpp", "fwht.hip"),
+    "fwht_bf16_2^30_n32768": _SHARED_HEADERS + ("hadamard_device.hpp", "fwht.hip"),
+    "rht_quant_fp8_8192x4096": _SHARED_HEADERS + ("rht_fp8.hip",),
+    "fp8_gemm_8192x14336x4096_l2_fill_plus_write": ("common.hpp", "fp8_gemm.hip"),
+}
+
+
+def kernel_sources_digest(names) -> str:
+    """sha256 over the named HIP sources (names and contents)."""
     h = hashlib.sha256()
     csrc = os.path.join(ROOT, PKG, "csrc")
-    for name in sorted(os.listdir(csrc)):
-        if name.endswith((".hip", ".hpp")):
-            h.update(name.encode())
-            with open(os.path.join(csrc, name), "rb") as f:
-                h.update(f.read())
+    for name in sorted(names):
+        h.update(name.encode())
+        with open(os.path.join(csrc, name), "rb") as f:
+            h.update(f.read())
     return h.hexdigest()
 
 
 def load_traffic() -> dict:
     """HBM bytes per launch recorded from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs
-    (profiles/hbm_traffic.json, figures taken from the summaries beside it).  The file names the
-    digest of the kernel sources it was measured on; when the sources have changed since, every
-    figure is reported as null rather than as a stale number."""
+    (profiles/hbm_traffic.json, figures taken from the summaries beside it).  Every entry names the
+    digest of the kernel sources it was measured on (TRAFFIC_SOURCES); an entry whose sources have
+    changed since is dropped, i.e. reported as null rather than as a stale number."""
     p = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if not os.path.exists(p):
         return {}
     with open(p) as f:
         rec = json.load(f)
-    if rec.get("kernel_sources_sha256") != kernel_sources_digest():
-        return {}
-    return rec.get("bytes_per_launch", {})
+    out = {}
+    for key, entry in rec.get("entries", {}).items():
+        if key in TRAFFIC_SOURCES and entry.get("sources_sha256") == kernel_sources_digest(TRAFFIC_SOURCES[key]):
+            out[key] = entry.get("bytes_per_launch")
+    return out
 
 
 def roofline(bound, achieved, peak, unit, traffic, **extra):
@@ -104,6 +122,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--sweep", action="store_true", help="also time n = 2^4..2^15 (128 MiB each)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--only-gemm-large-k", action="store_true",
+                    help="fused bf16 GEMM at K = 2048 and 4096, M = N = 4096, nothing else (profiling)")
     for flag, what in (("fwht", "stand-alone transform"), ("gemm", "fused bf16 GEMM"),
                        ("gemm-f32", "fused fp32 GEMM"), ("gemv", "fused HT+GEMV"),
                        ("rht", "RHT + FP8 quantize and FP8 GEMM")):
@@ -130,6 +150,16 @@ def main() -> int:
 
     result: dict = {}
     others: dict = {}
+
+    if args.only_gemm_large_k:
+        out = {}
+        for Kx in (2048, 4096):
+            Wx = torch.randn(4096, Kx, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(dev)
+            Xx = torch.randn(4096, Kx, generator=torch.Generator().manual_seed(0)).to(torch.bfloat16).to(dev)
+            f_ms, _ = steady_ms(lambda: hada.fused_ht_gemm(Wx, Xx), max(10, min(steps, 50)), 30.0)
+            out[f"fused_ht_gemm_bf16_K{Kx}_M4096_N4096"] = {"us": round(f_ms * 1e3, 2)}
+        print(json.dumps(out))
+        return 0
 
     # ---- fused HT -> GEMM, bf16 (config 4): the first half of the metric -----------------------------
     M = N = 4096

@@ -28,6 +28,21 @@ extern "C" {
 int mi_probe_mfma_rate(int shape, int lds_reads, uint32_t waves_per_simd, uint32_t steps,
                        const void* operands, uint64_t* cycles, void* stream);
 
+/*
+ * Instruction-issue probe, one compute unit (a single workgroup).  No counterpart in the reference.
+ *   mode 0: one wavefront per SIMD runs reps x 8 groups of [one v_mfma_f32_16x16x32_bf16 + n (0..4)
+ *           independent instructions of `kind`]; cycles[w] = shader clock cycles of wavefront w, so
+ *           cycles / (8 reps) is the cost of a group.  kind: 0 v_add_f32, 1 v_cvt_pk_bf16_f32,
+ *           2 s_add_u32, 3 ds_read_b128.  waves_per_simd must be 1.
+ *   mode 1: no MFMA: waves_per_simd (1..4) wavefronts per SIMD each run reps x 64 independent
+ *           instructions of `kind` (0 v_add_f32, 1 v_cvt_pk_bf16_f32, 4 v_cvt_pk_fp8_f32, 5 v_max3_f32,
+ *           6 v_lshlrev_b32); max(cycles) / (64 reps waves_per_simd) = cycles per instruction and SIMD.
+ *   in     : device, 256 x 8 fp32 (any finite values)      out : device, 1024 fp32 (keeps the work alive)
+ *   cycles : device, 16 x uint64
+ */
+int mi_probe_issue_rate(int mode, int kind, int n, uint32_t waves_per_simd, uint32_t reps,
+                        const float* in, float* out, uint64_t* cycles, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
