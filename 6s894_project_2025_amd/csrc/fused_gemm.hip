@@ -2,10 +2,9 @@
 // X given as Xt[N,K].  The transformed operand lives only in LDS.
 //
 // This file: the dispatcher and the LDS-resident variant, used for K = 32 .. 256 (64 columns per
-// workgroup, a column at most one tile; the kernel is written for any BN and for columns of several
-// tiles, which larger K used before the register-resident kernels took them over).  K >= 512 goes to
-// the register-resident variants in fused_gemm_xreg.hip and fused_gemm_xreg_k2048.hip, which hold
-// more columns per compute unit.
+// workgroup, a column at most half a 512-element tile).  K >= 512 goes to the register-resident
+// variants in fused_gemm_xreg.hip and fused_gemm_xreg_k2048.hip, which hold more columns per
+// compute unit.
 //
 // Structure ("X-stationary"): a workgroup owns BN columns of X for the whole K extent.
 //   prologue : its wavefronts transform those BN rows of Xt on the matrix cores (tile_transform,
@@ -99,17 +98,12 @@ static_assert(lds::conflict_free_b128(stage_write_offset) && lds::conflict_free_
 static_assert(y_patterns_conflict_free<0>() && y_patterns_conflict_free<1>() && y_patterns_conflict_free<2>(),
               "an access pattern of the transformed tile would serialise");
 
-// XB = log2(max(K,512)/512): tiles per column that need cross-tile butterflies.
-// KFIX: K when it is known at compile time (lets the K loop be scheduled without run-time guards),
-// 0 for the generic instantiation.
-template <class T16, int BN, int XB, int KFIX>
+template <class T16, int BN>
 __global__ void __launch_bounds__(kGemmThreads)
 fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16::E* __restrict__ Xt,
-                       void* __restrict__ C, uint32_t M, uint32_t N, uint32_t K_rt, uint32_t logK_rt,
+                       void* __restrict__ C, uint32_t M, uint32_t N, uint32_t K, uint32_t logK,
                        uint32_t m_per_block, uint32_t msplit, int out_f32, float fscale)
 {
-    const uint32_t K = KFIX ? (uint32_t)KFIX : K_rt;
-    const uint32_t logK = KFIX ? (uint32_t)__builtin_ctz(KFIX ? KFIX : 1) : logK_rt;
     using E = typename T16::E;
     using V8 = typename T16::V8;
     constexpr int NB = BN / 16;  // 16-column fragments of Y (A-operand blocks)
@@ -164,9 +158,7 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
     {
         TileOperands<T16> ops;
         make_tile_operands<T16, 2>(logK, ops);
-        constexpr int NT = 1 << XB;                       // tiles per column (or 1)
         constexpr int BATCH = 16;                         // tiles in flight per wavefront
-        static_assert(BATCH % NT == 0, "batch must hold whole columns");
         const uint32_t block_tiles = (BN * K) >> 9;       // 512-element tiles in this block
         const uint64_t total = (uint64_t)N * K;           // elements in Xt
         const uint64_t tile_base = ((uint64_t)n0 * K) >> 9;
@@ -188,24 +180,18 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
                     }
                 }
 #pragma unroll
-                for (int g = 0; g < BATCH / NT; ++g) {
-                    f32x4 acc[NT][2];
+                for (int g = 0; g < BATCH; ++g) {   // a tile holds 512 / K whole columns
+                    if (GUARD && t0 + g >= block_tiles) continue;
+                    f32x4 acc[2];
+                    tile_transform<T16>(in[g], ops, acc);
+                    V8 o;
 #pragma unroll
-                    for (int c = 0; c < NT; ++c) tile_transform<T16>(in[g * NT + c], ops, acc[c]);
-                    cross_tile_butterflies<NT, XB>(acc);
+                    for (int t = 0; t < 2; ++t)
 #pragma unroll
-                    for (int c = 0; c < NT; ++c) {
-                        if (GUARD && t0 + g * NT + c >= block_tiles) continue;
-                        V8 o;
-#pragma unroll
-                        for (int t = 0; t < 2; ++t)
-#pragma unroll
-                            for (int r = 0; r < 4; ++r) o[4 * t + r] = (E)(acc[c][t][r] * fscale);
-                        const uint32_t e = (t0 + g * NT + c) * 512u + 8u * lane;  // offset in the block
-                        const uint32_t n = e >> logK, q = (e & (K - 1u)) >> 3;
-                        *reinterpret_cast<V8*>(ylds + y_chunk_offset<LOG_NB>(n, q, K * 2u, swz_mask)) =
-                            o;
-                    }
+                        for (int r = 0; r < 4; ++r) o[4 * t + r] = (E)(acc[t][r] * fscale);
+                    const uint32_t e = (t0 + g) * 512u + 8u * lane;  // offset in the block
+                    const uint32_t n = e >> logK, q = (e & (K - 1u)) >> 3;
+                    *reinterpret_cast<V8*>(ylds + y_chunk_offset<LOG_NB>(n, q, K * 2u, swz_mask)) = o;
                 }
             }
         };
@@ -418,7 +404,7 @@ fused_ht_gemm16_kernel(const typename T16::E* __restrict__ W, const typename T16
     }
 }
 
-template <class T16, int BN, int XB, int KFIX>
+template <class T16, int BN>
 int launch_gemm16(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N, uint32_t K,
                   int out_f32, float scale, hipStream_t s)
 {
@@ -435,7 +421,7 @@ int launch_gemm16(const void* W, const void* Xt, void* C, uint32_t M, uint32_t N
     const uint32_t m_per_block = ((row_blocks + msplit - 1u) / msplit) * 512u;
     msplit = (M + m_per_block - 1u) / m_per_block;
     const size_t lds = (size_t)BN * K * 2u + (size_t)kGemmWaves * kStageBytes;
-    auto kern = fused_ht_gemm16_kernel<T16, BN, XB, KFIX>;
+    auto kern = fused_ht_gemm16_kernel<T16, BN>;
     if (lds > 64u * 1024u) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -456,7 +442,7 @@ int dispatch_gemm16(const void* W, const void* Xt, void* C, uint32_t M, uint32_t
         case 32:
         case 64:
         case 128:
-        case 256: return launch_gemm16<T16, 64, 0, 0>(W, Xt, C, M, N, K, out_f32, scale, s);
+        case 256: return launch_gemm16<T16, 64>(W, Xt, C, M, N, K, out_f32, scale, s);
         case 512:
         case 1024:
         case 2048:
