@@ -1,28 +1,54 @@
 // Fused Hadamard + GEMV-batch (mi_fused_ht_gemv), fp32, gfx950:
 //     Y[M,B] = W[M,N] * (scale * H_N * X[N,B]),  transform down dimension 0 of X.
 //
-// A workgroup owns 16 columns of X and 16, 32 or 64 rows of W.
-//   prologue : the 16 columns are brought into LDS as T[N][16] (a row is 64 bytes, so the 16
+// A workgroup owns 16 or 32 columns of X and 16, 32 or 64 rows of W at a time; it keeps its
+// transformed columns in LDS for several row blocks when there are more row blocks than compute
+// units to spread them over.
+//   prologue, N >= 512: the columns are brought into LDS column by column (TT[NC][N + 4]: a
+//              thread reads 16 contiguous bytes of a row of X and scatters them over four
+//              columns), transformed there by the exact fp32 tile transform on the matrix cores
+//              (fwht_device.hpp: 512-element tiles read and written back with 16-byte LDS accesses,
+//              taken in pairs whose MFMA chains interleave, the tiles of a column joined by fp32
+//              butterflies in registers; wavefront w takes columns (NC/4) w ..), and read by the
+//              product as 16-byte B fragments.  N = 1024 measured 10.4 us per workgroup for the
+//              register-butterfly prologue below (every LDS access 4 bytes, 128 of them per thread
+//              and pass) against 4 us of loading and 6 us of transform for twice the columns here.
+//   prologue, N < 512: the 16 columns are brought into LDS as T[N][16] (a row is 64 bytes, so the 16
 //              column-lanes of a wavefront read global memory contiguously) while radix-16
 //              register butterflies run: each thread owns one column and 16 rows per step, so
 //              log2(N) stages cost ceil(log2(N)/4) passes over LDS, the first one straight from
 //              global memory.  Row positions are XOR-swizzled so every access pattern below
 //              touches four different 64-byte bank groups per wavefront.
-//   product  : v_mfma_f32_16x16x4_f32 with W as the A operand (one 16-byte load per lane gives
-//              four consecutive k for four MFMAs) and T as the B operand; each W element is read
-//              once per workgroup instead of once per column.  The four wavefronts each take a
-//              quarter of the K range with four K steps of loads in flight (the loop is
-//              latency-bound otherwise), and their partial sums are added through LDS.
+//   product  : v_mfma_f32_16x16x4_f32 (32 cycles each) with W as the A operand (one 16-byte load
+//              per lane gives four consecutive k for four MFMAs) and T as the B operand; each W
+//              element is read once per workgroup instead of once per column.  The four wavefronts
+//              each take a quarter of the K steps with four steps of loads in flight, the B
+//              fragments of a step read one step early, and their partial sums are added through
+//              LDS.  With 32 columns (N = 512 and 1024, once that still gives every compute unit a
+//              workgroup) the K loop runs at 0.88 of the matrix cores' rate (18.5 thousand cycles
+//              for 512 MFMAs per wavefront); with 16 columns it is bound by the stream of W from
+//              the L2, which is why 32 are taken where the LDS holds them.
+//   placement: workgroups are numbered so that the column groups sharing a slice of W run on one
+//              XCD (one L2).
 //
 // Behaviour replaced: fused_hadamard_gemv_kernel(_vec), fused_ht/fwht_gemv_fusion.cu:98-244, where
 // every column's block re-reads all of W and reduces with warp shuffles.
-#include "common.hpp"
+#include <type_traits>
+
+#include "fwht_device.hpp"
 
 namespace mi {
 namespace {
 
 constexpr int kCols = 16;
 constexpr int kThreads = 256;
+constexpr uint32_t kXcds = 8;
+
+// N >= 512: column c of the transformed tile lives at TT + c * (N + kPad) floats.  With a row
+// stride of 16 bytes modulo 128 the 16-byte accesses of eight adjacent lanes (eight columns, the
+// same k) fall into eight different 16-byte columns of the LDS row, as do those of eight lanes on
+// consecutive k of one column.
+constexpr uint32_t kPad = 4;
 
 // physical row of logical row r in the LDS tile: low two bits mixed with bits 2-3 and 4-5
 __device__ __forceinline__ uint32_t prow(uint32_t r)
@@ -108,45 +134,176 @@ __device__ __forceinline__ void pass_w(int wbits, const float* __restrict__ X, f
 // MI = 16-row blocks of W per workgroup (16, 32 or 64 rows).  The four wavefronts split the K range
 // of the product between them (every wavefront covers all MI row blocks over a quarter of N), so
 // each one streams a short, deeply prefetched run of W, and the partial sums meet in LDS.
-template <int MI>
+template <int MI, bool TILED, int NC, int PF>
 __global__ void __launch_bounds__(kThreads)
 fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
                      float* __restrict__ Y, uint32_t M, uint32_t N, uint32_t B, uint32_t logN,
-                     float scale, uint32_t rows_per_group)
+                     float scale, uint32_t rows_per_group, uint32_t col_groups, uint32_t row_groups,
+                     uint32_t per_xcd)
 {
+    static_assert(NC == kCols || (TILED && NC == 2 * kCols), "wider tiles only in the column-major form");
+    constexpr int NF = NC / 16;  // 16-column fragments of the product per workgroup
     extern __shared__ __attribute__((aligned(16))) float tile[];  // [N][16] rows swizzled, then sums
-    const uint32_t b0 = blockIdx.x * kCols;
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    // Workgroups are handed to the eight XCDs in turn, each with an L2 of its own.  Position
+    // (XCD, slot) takes place XCD * per_xcd + slot of the row-group-major order of the tiles, so
+    // that the column groups which share a slice of W run side by side on one XCD and read it
+    // from that L2 (W is read once per column group, X once per row group).
+    const uint32_t place = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
+    if (place >= col_groups * row_groups) return;
+    const uint32_t b0 = (place % col_groups) * NC;
+    // the wavefront's index as a scalar: everything derived from it (its K range above all) then
+    // steers branches instead of lane masks
+    const uint32_t lane = threadIdx.x & 63u, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t lo = lane & 15u, hi = lane >> 4;
     // this workgroup's rows: [m_first, m_last), a multiple of 16 * MI except at the end of W
-    const uint32_t m_first = blockIdx.y * rows_per_group;
+    const uint32_t m_first = (place / col_groups) * rows_per_group;
     const uint32_t m_last = min(M, m_first + rows_per_group);
 
-    constexpr int PF = 4;  // K steps (of 16) in flight per wavefront
+    // PF = K steps (of 16) in flight per wavefront: four, and eight for N = 2048, where a compute
+    // unit holds one workgroup (four wavefronts) whose 64 KB on the way at the latency of the L2
+    // left the K loop at half the rate of the matrix cores.  (The 32-column workgroups are bound by
+    // the matrix cores with four; eight measured slower, 40.7 -> 44.2 us for four row blocks.)
     const uint32_t total = N >> 4;
     const uint32_t quarter = (total + 3u) / 4u;
     const uint32_t k_begin = min(wave * quarter, total), k_end = min(k_begin + quarter, total);
+    // The wavefront's i-th K step.  TILED (N >= 512, so the steps divide evenly): steps 2p and
+    // 2p+1 of a wavefront are the two 64-byte halves of one 128-byte line of each row of W, asked
+    // for together, and the four wavefronts take adjacent lines.  (With a quarter of the K range
+    // each, the halves of a line were asked for a step apart, with 256 other lines of rows a
+    // multiple of 4 KB apart in between.  Measured: N = 2048, 33.6 -> 31.4 thousand cycles per
+    // row block; N = 1024, no change.)
+    auto kof = [&](uint32_t i) { return TILED ? ((i >> 1) << 3) + 2u * wave + (i & 1u) : k_begin + i; };
     const float* wrow[MI];
     f32x4 a[PF][MI];
-    auto start_block = [&](uint32_t mb) {
+    auto rows_of = [&](uint32_t mb, const float* (&rows)[MI]) {
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) {
             const uint32_t m = min(mb + 16u * mi + lo, M - 1u);
-            wrow[mi] = W + (uint64_t)m * N + 4u * hi;
+            rows[mi] = W + (uint64_t)m * N + 4u * hi;
         }
+    };
+    auto start_block = [&](uint32_t mb) {
+        rows_of(mb, wrow);
+        if constexpr (TILED) {
 #pragma unroll
-        for (int j = 0; j < PF; ++j)
-            if (k_begin + j < k_end) {
+            for (int j = 0; j < PF; j += 2)
 #pragma unroll
-                for (int mi = 0; mi < MI; ++mi)
-                    a[j][mi] = *reinterpret_cast<const f32x4*>(wrow[mi] + 16u * (k_begin + j));
-            }
+                for (int mi = 0; mi < MI; ++mi) {
+                    a[j][mi] = *reinterpret_cast<const f32x4*>(wrow[mi] + 16u * kof(j));
+                    a[j + 1][mi] = *reinterpret_cast<const f32x4*>(wrow[mi] + 16u * kof(j + 1));
+                }
+        } else {
+#pragma unroll
+            for (int j = 0; j < PF; ++j)
+                if (k_begin + j < k_end) {
+#pragma unroll
+                    for (int mi = 0; mi < MI; ++mi)
+                        a[j][mi] = *reinterpret_cast<const f32x4*>(wrow[mi] + 16u * kof(j));
+                }
+        }
     };
     // The first W fragments do not depend on the transform: start them before the prologue.
     start_block(m_first);
 
     // ---- prologue: T = scale * H_N * X[:, b0:b0+16] --------------------------------------------
-    {
+    const uint32_t cstride = N + kPad;  // TILED: floats per column of TT
+    if constexpr (TILED) {
+        // X[:, b0 .. b0+NC-1] -> TT: a thread reads four adjacent columns of a row.  A wavefront
+        // covers 16 rows by 16 columns, so that its four-byte LDS writes (bank = 16 * (column / 4) +
+        // row modulo 64) never meet in a bank.
+        {
+            constexpr uint32_t WQ = NC / 16;        // wavefronts side by side along a row
+            constexpr uint32_t RP = 16u * 4u / WQ;  // rows per pass of the workgroup
+            const uint32_t q4 = (lane & 3u) + 4u * (wave % WQ), r0 = (lane >> 2) + 16u * (wave / WQ);
+            const bool vec_ok = b0 + NC <= B && (B & 3u) == 0;
+            // DEPTH rows in flight per thread (DEPTH * RP divides 512): the tile is NC * 4 bytes of
+            // each of N rows, from the L2
+            constexpr int DEPTH = NC == kCols ? 8 : 16;
+            for (uint32_t rb = r0; rb < N; rb += (uint32_t)DEPTH * RP) {
+                f32x4 v[DEPTH];
+#pragma unroll
+                for (int u = 0; u < DEPTH; ++u) {
+                    const uint32_t r = rb + (uint32_t)u * RP;
+                    v[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+                    const uint64_t at = (uint64_t)r * B + b0 + 4u * q4;
+                    if (vec_ok) {
+                        v[u] = *reinterpret_cast<const f32x4*>(X + at);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (b0 + 4u * q4 + e < B) v[u][e] = X[at + e];
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < DEPTH; ++u) {
+                    const uint32_t r = rb + (uint32_t)u * RP;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) tile[(4u * q4 + e) * cstride + r] = v[u][e];
+                }
+            }
+        }
+        __syncthreads();
+        // Wavefront w transforms columns (NC/4) w .. (NC/4) (w+1) - 1: its tiles (N / 512 per
+        // column) are taken in pairs whose MFMA chains interleave, the next pair's LDS reads and
+        // three-way splits sitting in the shadow of this pair's MFMAs (one wavefront per SIMD may
+        // be all there is); the tiles of a column are then joined by fp32 butterflies in registers.
+        TileOperands<BF16> ops;
+        make_tile_operands<BF16, 4>(9, ops);
+        auto transform_columns = [&](auto nt_tag) __attribute__((always_inline)) {
+            constexpr int NT = decltype(nt_tag)::value;  // tiles per column
+            constexpr int XB = NT == 4 ? 2 : (NT == 2 ? 1 : 0);
+            constexpr int CW = NC / 4;                   // columns per wavefront
+            constexpr int PAIRS = CW * NT / 2;
+            constexpr int HOLD = NT > 2 ? NT : 2;        // tiles held until their column is whole
+            float* const first = tile + (uint32_t)CW * wave * cstride;
+            auto at = [&](int t) { return first + (uint32_t)(t / NT) * cstride + 512u * (uint32_t)(t % NT); };
+            auto fetch = [&](int t, SplitTileF32& o) __attribute__((always_inline)) {
+                float in[8];
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const f32x4 q = *reinterpret_cast<const f32x4*>(at(t) + 256u * h + 4u * lane);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) in[4 * h + r] = q[r];
+                }
+                split_tile_f32(in, o);
+            };
+            SplitTileF32 cur[2], nxt[2];
+            fetch(0, cur[0]);
+            fetch(1, cur[1]);
+            f32x4 held[HOLD][2];
+#pragma unroll
+            for (int p = 0; p < PAIRS; ++p) {
+                if (p + 1 < PAIRS) {
+                    fetch(2 * p + 2, nxt[0]);
+                    fetch(2 * p + 3, nxt[1]);
+                }
+                f32x4 a[2][2];
+                tile_pair_mfma_f32(cur, ops, a);
+#pragma unroll
+                for (int c = 0; c < 2; ++c)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) held[(2 * p + c) % HOLD][h] = a[c][h];
+                if ((2 * p + 2) % HOLD == 0) {
+                    if constexpr (NT > 1) cross_tile_butterflies<NT, XB>(held);
+#pragma unroll
+                    for (int i = 0; i < HOLD; ++i)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h)
+                            *reinterpret_cast<f32x4*>(at(2 * p + 2 - HOLD + i) + 256u * h + 4u * lane) =
+                                held[i][h] * scale;
+                }
+                cur[0] = nxt[0];
+                cur[1] = nxt[1];
+            }
+        };
+        if (N == 512u)
+            transform_columns(std::integral_constant<int, 1>{});
+        else if (N == 1024u)
+            transform_columns(std::integral_constant<int, 2>{});
+        else
+            transform_columns(std::integral_constant<int, 4>{});
+        __syncthreads();
+    } else {
         uint32_t done = 0;
         bool first = true;
         uint32_t passes_left = (logN + 4u) / 5u;  // fewest radix-32 passes, bits spread evenly
@@ -163,40 +320,91 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
             __syncthreads();
         }
     }
-    f32x4* red = reinterpret_cast<f32x4*>(tile + (size_t)N * kCols);  // [4 wavefronts][MI][64 lanes]
+    // [MI * NF fragments][3 other wavefronts][64 lanes]
+    f32x4* red = reinterpret_cast<f32x4*>(tile + (size_t)(TILED ? cstride : N) * NC);
 
     for (uint32_t mb = m_first; mb < m_last; mb += 16u * MI) {
-        if (mb != m_first) start_block(mb);
+        // TILED: the previous block's last steps have already started this block's first loads
+        const bool has_next = mb + 16u * MI < m_last;
+        const float* wnext[MI];
+        if constexpr (TILED) {
+            if (has_next) rows_of(mb + 16u * MI, wnext);
+        } else {
+            if (mb != m_first) start_block(mb);
+        }
         // ---- product ------------------------------------------------------------------------------
-        f32x4 acc[MI];
+        f32x4 acc[MI * NF];  // fragment g = mi * NF + f: rows 16 mi .., columns 16 f ..
 #pragma unroll
-        for (int mi = 0; mi < MI; ++mi) acc[mi] = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (N >= 16u) {
-            for (uint32_t kk = k_begin; kk < k_end; kk += PF) {
+        for (int g = 0; g < MI * NF; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+        // One K step (16 columns of W) for all fragments.  refill: start the W loads PF steps ahead;
+        // more (TILED): read the next step's B fragments now, a step before their MFMAs.
+        f32x4 bq[2][NF];
+        auto read_b = [&](uint32_t k, f32x4 (&o)[NF]) __attribute__((always_inline)) {
+            if constexpr (TILED) {
+                const f32x4* const tile4 = reinterpret_cast<const f32x4*>(tile);
 #pragma unroll
-                for (int j = 0; j < PF; ++j) {
-                    if (kk + j < k_end) {  // wavefront-uniform
-                        f32x4 cur[MI];
+                for (int f = 0; f < NF; ++f) o[f] = tile4[(16u * f + lo) * (cstride / 4u) + 4u * k + hi];
+            } else {
 #pragma unroll
-                        for (int mi = 0; mi < MI; ++mi) cur[mi] = a[j][mi];
-                        if (kk + j + PF < k_end) {
+                for (int s = 0; s < 4; ++s) o[0][s] = tile[prow(16u * k + 4u * hi + s) * kCols + lo];
+            }
+        };
+        auto k_step = [&](uint32_t i, int j, int refill, bool more) __attribute__((always_inline)) {
+            const uint32_t k = kof(i);
+            if (TILED && more) {
+                read_b(kof(i + 1u), bq[(j + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0);  // ahead of this step's MFMAs, not behind them
+            }
+            if (!TILED) read_b(k, bq[j & 1]);
 #pragma unroll
-                            for (int mi = 0; mi < MI; ++mi)
-                                a[j][mi] = *reinterpret_cast<const f32x4*>(wrow[mi] +
-                                                                           16u * (kk + j + PF));
-                        }
-                        float bv[4];
+            for (int s = 0; s < 4; ++s)
 #pragma unroll
-                        for (int s = 0; s < 4; ++s)
-                            bv[s] = tile[prow(16u * (kk + j) + 4u * hi + s) * kCols + lo];
+                for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-                        for (int s = 0; s < 4; ++s)
+                    for (int f = 0; f < NF; ++f)
+                        acc[mi * NF + f] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                            a[j][mi][s], bq[j & 1][f][s], acc[mi * NF + f], 0, 0, 0);
+            if constexpr (TILED) {
+                // steps 2p and 2p+1 are the halves of a 128-byte line: ask for both together
+                if (refill != 0 && (j & 1)) {
+                    const float* const* src = refill == 1 ? wrow : wnext;  // 2: the next row block
+                    const uint32_t at = refill == 1 ? i + PF : (uint32_t)j;
 #pragma unroll
-                            for (int mi = 0; mi < MI; ++mi)
-                                acc[mi] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur[mi][s], bv[s],
-                                                                               acc[mi], 0, 0, 0);
+                    for (int mi = 0; mi < MI; ++mi) {
+                        a[j - 1][mi] = *reinterpret_cast<const f32x4*>(src[mi] + 16u * kof(at - 1u));
+                        a[j][mi] = *reinterpret_cast<const f32x4*>(src[mi] + 16u * kof(at));
                     }
                 }
+            } else if (refill == 1) {
+#pragma unroll
+                for (int mi = 0; mi < MI; ++mi)
+                    a[j][mi] = *reinterpret_cast<const f32x4*>(wrow[mi] + 16u * kof(i + PF));
+            }
+            // keep every step's loads in the step: left to itself the scheduler gathers the loads
+            // of a round behind its last MFMA and waits for all of them before the next one
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        if constexpr (TILED) {
+            // every wavefront has a whole number of PF-step rounds: all but the last refill the ring
+            read_b(kof(0), bq[0]);
+            for (uint32_t ii = 0; ii + PF < quarter; ii += PF) {
+#pragma unroll
+                for (int j = 0; j < PF; ++j) k_step(ii + j, j, 1, true);
+            }
+            if (has_next) {
+#pragma unroll
+                for (int j = 0; j < PF; ++j) k_step(quarter - PF + j, j, 2, j + 1 < PF);
+#pragma unroll
+                for (int mi = 0; mi < MI; ++mi) wrow[mi] = wnext[mi];
+            } else {
+#pragma unroll
+                for (int j = 0; j < PF; ++j) k_step(quarter - PF + j, j, 0, j + 1 < PF);
+            }
+        } else if (N >= 16u) {
+            for (uint32_t ii = 0; k_begin + ii < k_end; ii += PF) {
+#pragma unroll
+                for (int j = 0; j < PF; ++j)
+                    if (k_begin + ii + j < k_end) k_step(ii + j, j, k_begin + ii + j + PF < k_end ? 1 : 0, false);
             }
         } else if (wave == 0) {
             // N = 2, 4, 8: one partial step, lanes with k >= N contribute zero
@@ -215,49 +423,79 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
         }
 
         // ---- meet the four K quarters in LDS ------------------------------------------------------
+        // Fragment g is finished by wavefront g % 4, which keeps its own partial sum in registers:
+        // only the other three go through LDS (12 KB instead of 16 for 64 rows by 16 columns, which
+        // is what lets two such workgroups with N = 1024 share a compute unit).  The sum is taken in
+        // the order of the wavefronts, whoever holds which part.
         __syncthreads();  // the previous block's sums have been read
 #pragma unroll
-        for (int mi = 0; mi < MI; ++mi) red[(wave * MI + mi) * 64u + lane] = acc[mi];
+        for (int g = 0; g < MI * NF; ++g) {
+            const uint32_t owner = (uint32_t)(g & 3);
+            if (wave != owner) red[((uint32_t)g * 3u + (wave < owner ? wave : wave - 1u)) * 64u + lane] = acc[g];
+        }
         __syncthreads();
         // D[m'][n']: n' = lo is the column, m' = 4*hi + r the row inside the 16-row block
-        for (uint32_t mi = wave; mi < (uint32_t)MI; mi += 4u) {
-            f32x4 sum = red[mi * 64u + lane];
 #pragma unroll
-            for (uint32_t w = 1; w < 4u; ++w) sum += red[(w * MI + mi) * 64u + lane];
-            if (b0 + lo < B) {
+        for (int g = 0; g < MI * NF; ++g) {
+            constexpr int kWaves = kThreads / 64;
+            const int owner = g & 3;
+            if (wave != (uint32_t)owner) continue;
+            f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) {
+                const f32x4 part = w == owner ? acc[g] : red[(g * 3 + (w < owner ? w : w - 1)) * 64 + lane];
+                sum = w == 0 ? part : sum + part;
+            }
+            const uint32_t col = b0 + 16u * (uint32_t)(g % NF) + lo;
+            if (col < B) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const uint32_t m = mb + 16u * mi + 4u * hi + r;
-                    if (m < M) Y[(uint64_t)m * B + b0 + lo] = sum[r];
+                    const uint32_t m = mb + 16u * (uint32_t)(g / NF) + 4u * hi + r;
+                    if (m < M) Y[(uint64_t)m * B + col] = sum[r];
                 }
             }
         }
     }
 }
 
-template <int MI>
-int launch_gemv(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B,
-                float scale, hipStream_t s)
+template <int MI, bool TILED, int NC, int PF = 4>
+int launch_gemv_as(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B,
+                   float scale, hipStream_t s)
 {
-    const size_t lds = (size_t)N * kCols * sizeof(float) + 4u * MI * 64u * sizeof(f32x4);
-    auto kern = fused_ht_gemv_kernel<MI>;
+    const size_t lds = (size_t)(N + (TILED ? kPad : 0u)) * NC * sizeof(float) +
+                       3u * MI * (NC / 16) * 64u * sizeof(f32x4);
+    // the tile transform's two MFMA stages attenuate by a power of two that the scale takes back
+    if (TILED) scale = (float)((double)scale * (double)(1u << tile_stage_shift<4>(9u, false)));
+    auto kern = fused_ht_gemv_kernel<MI, TILED, NC, PF>;
     if (lds > 64u * 1024u) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
             return MI_ERR_LAUNCH;
     }
     // A workgroup keeps its transformed tile for several row blocks once there are more row
-    // blocks than it takes to give every compute unit two workgroups.
+    // blocks than it takes to give every compute unit as many workgroups as fit its LDS (two are
+    // counted on where they fit).
     constexpr uint32_t kBlock = 16u * MI;
-    const uint32_t col_groups = (B + kCols - 1) / kCols;
+    const uint32_t col_groups = (B + NC - 1) / NC;
     const uint32_t row_blocks = (M + kBlock - 1) / kBlock;
-    uint32_t groups_y = (512u + col_groups - 1) / col_groups;
+    uint32_t groups_y = ((lds <= 80u * 1024u ? 512u : 256u) + col_groups - 1) / col_groups;
     if (groups_y > row_blocks) groups_y = row_blocks;
     const uint32_t rows_per_group = ((row_blocks + groups_y - 1) / groups_y) * kBlock;
-    const dim3 grid(col_groups, (M + rows_per_group - 1) / rows_per_group);
-    hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds, s, W, X, Y, M, N, B, ilog2(N), scale,
-                       rows_per_group);
+    const uint32_t row_groups = (M + rows_per_group - 1) / rows_per_group;
+    const uint32_t per_xcd = (col_groups * row_groups + kXcds - 1) / kXcds;
+    hipLaunchKernelGGL(kern, dim3(per_xcd * kXcds), dim3(kThreads), lds, s, W, X, Y, M, N, B,
+                       ilog2(N), scale, rows_per_group, col_groups, row_groups, per_xcd);
     return launch_status();
+}
+
+template <int MI>
+int launch_gemv(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B,
+                float scale, hipStream_t s)
+{
+    if constexpr (MI == 4)
+        if (N == 2048u) return launch_gemv_as<MI, true, kCols, 8>(W, X, Y, M, N, B, scale, s);
+    return N >= 512u ? launch_gemv_as<MI, true, kCols>(W, X, Y, M, N, B, scale, s)
+                     : launch_gemv_as<MI, false, kCols>(W, X, Y, M, N, B, scale, s);
 }
 
 }  // namespace
@@ -279,6 +517,11 @@ extern "C" int mi_fused_ht_gemv(const void* W, const void* X, void* Y, uint32_t 
     // 64-row workgroups once that still gives every compute unit a workgroup; 32-row ones for
     // small problems, where more (shorter) workgroups matter more than the repeated transform,
     // and 16-row ones for the smallest (M = N = 1024, B <= 64: 12.2 -> 11.1 us)
+    // 32 columns per workgroup (W is read half as often, and every read of W comes from the L2)
+    // where the transformed tile still fits the LDS and every compute unit still gets a workgroup
+    const uint64_t groups32x64 = (uint64_t)((B + 31u) / 32u) * ((M + 63u) / 64u);
+    if ((N == 512u || N == 1024u) && groups32x64 >= 256u)
+        return launch_gemv_as<4, true, 32>(w, x, y, M, N, B, scale, s);
     const uint64_t groups64 = (uint64_t)((B + kCols - 1) / kCols) * ((M + 63u) / 64u);
     if (groups64 >= 256u) return launch_gemv<4>(w, x, y, M, N, B, scale, s);
     if (groups64 < 128u) return launch_gemv<1>(w, x, y, M, N, B, scale, s);

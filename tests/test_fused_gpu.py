@@ -50,9 +50,16 @@ def test_gemv_reference_self_check(pkg, oracle, M, N, B):
 # fused_ht/fwht_gemv_fusion.cu:643-653) and a workgroup that walks several row blocks with one
 # transformed tile (more row blocks than workgroup rows in the grid).  (The 32-row variant runs
 # between 128 and 255 such groups: (1024, 1024, 128) here and (256, 256, 512) above; everything
-# smaller runs 16-row workgroups.)
+# smaller runs 16-row workgroups.)  N = 512 and 1024 switch to 32-column workgroups once those
+# still number 256: (1024, 1024, 512) with one row block each, (1024, 1024, 2048) with four (the
+# loads of the next block start in the last steps of the one before), (1000, 512, 700) with a
+# ragged last row block and a last column group of 28, (1100, 1024, 531) with a row length that
+# rules out 16-byte loads of X.  N = 2048 with 64-row workgroups has a deeper load ring:
+# (4100, 2048, 130) and (2048, 2048, 512) walk three and four row blocks with it.
 @pytest.mark.parametrize("M,N,B", [(1024, 1024, 256), (1024, 1024, 512), (1024, 1024, 128),
-                                   (4096, 256, 4096), (2000, 64, 1000), (4100, 2048, 130)])
+                                   (4096, 256, 4096), (2000, 64, 1000), (4100, 2048, 130),
+                                   (1024, 1024, 2048), (1000, 512, 700), (1100, 1024, 531),
+                                   (2048, 2048, 512)])
 def test_gemv_large_launch_paths(pkg, oracle, M, N, B):
     W, X = oracle.inputs_gemv(M, N, B)
     Y = pkg.fused_ht_gemv(W.cuda(), X.cuda())
