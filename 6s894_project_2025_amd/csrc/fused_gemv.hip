@@ -215,7 +215,10 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
             constexpr uint32_t WQ = NC / 16;        // wavefronts side by side along a row
             constexpr uint32_t RP = 16u * 4u / WQ;  // rows per pass of the workgroup
             const uint32_t q4 = (lane & 3u) + 4u * (wave % WQ), r0 = (lane >> 2) + 16u * (wave / WQ);
-            const bool vec_ok = b0 + NC <= B && (B & 3u) == 0;
+            // this thread's four columns: all inside X and 16-byte loadable, some, or none
+            const uint32_t c4 = b0 + 4u * q4;
+            const bool vec_ok = c4 + 4u <= B && (B & 3u) == 0;
+            const bool any = c4 < B;
             // DEPTH rows in flight per thread (DEPTH * RP divides 512): the tile is NC * 4 bytes of
             // each of N rows, from the L2
             constexpr int DEPTH = NC == kCols ? 8 : 16;
@@ -225,13 +228,13 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
                 for (int u = 0; u < DEPTH; ++u) {
                     const uint32_t r = rb + (uint32_t)u * RP;
                     v[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-                    const uint64_t at = (uint64_t)r * B + b0 + 4u * q4;
+                    const uint64_t at = (uint64_t)r * B + c4;
                     if (vec_ok) {
                         v[u] = *reinterpret_cast<const f32x4*>(X + at);
-                    } else {
+                    } else if (any) {
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
-                            if (b0 + 4u * q4 + e < B) v[u][e] = X[at + e];
+                            if (c4 + e < B) v[u][e] = X[at + e];
                     }
                 }
 #pragma unroll
@@ -243,57 +246,78 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
             }
         }
         __syncthreads();
-        // Wavefront w transforms columns (NC/4) w .. (NC/4) (w+1) - 1: its tiles (N / 512 per
-        // column) are taken in pairs whose MFMA chains interleave, the next pair's LDS reads and
-        // three-way splits sitting in the shadow of this pair's MFMAs (one wavefront per SIMD may
-        // be all there is); the tiles of a column are then joined by fp32 butterflies in registers.
+        // Wavefront w transforms columns w, w + 4, w + 8, ... of the tile, those that exist in X
+        // (a last or only column group may hold fewer than NC: with B = 8 every wavefront has two
+        // columns to do, not four for two of them and four columns of zeros for the others).  Its
+        // tiles (N / 512 per column) are taken in pairs whose MFMA chains interleave, the next
+        // pair's LDS reads and three-way splits sitting in the shadow of this pair's MFMAs (one
+        // wavefront per SIMD may be all there is); the tiles of a column are then joined by fp32
+        // butterflies in registers.  Columns past the end of X are left as they are: a column of
+        // the B operand reaches only its own column of the product, which is not stored.
         TileOperands<BF16> ops;
         make_tile_operands<BF16, 4>(9, ops);
         auto transform_columns = [&](auto nt_tag) __attribute__((always_inline)) {
             constexpr int NT = decltype(nt_tag)::value;  // tiles per column
             constexpr int XB = NT == 4 ? 2 : (NT == 2 ? 1 : 0);
-            constexpr int CW = NC / 4;                   // columns per wavefront
-            constexpr int PAIRS = CW * NT / 2;
-            constexpr int HOLD = NT > 2 ? NT : 2;        // tiles held until their column is whole
-            float* const first = tile + (uint32_t)CW * wave * cstride;
-            auto at = [&](int t) { return first + (uint32_t)(t / NT) * cstride + 512u * (uint32_t)(t % NT); };
-            auto fetch = [&](int t, SplitTileF32& o) __attribute__((always_inline)) {
+            constexpr int HOLD = NT > 2 ? NT : 2;        // tiles of a unit: a column, or two of one tile
+            constexpr int UPAIRS = HOLD / 2;             // pairs of tiles per unit
+            const uint32_t ncols = min((uint32_t)NC, B - b0);
+            const uint32_t mine = ncols > wave ? (ncols - wave + 3u) / 4u : 0u;  // columns of this wavefront
+            const uint32_t units = NT == 1 ? (mine + 1u) / 2u : mine;
+            // tile t of unit u: NT > 1: tile t of the wavefront's u-th column; NT = 1: column 2u + t
+            auto at = [&](uint32_t u, int t) {
+                const uint32_t j = NT == 1 ? 2u * u + (uint32_t)t : u;
+                const uint32_t c = min(wave + 4u * j, (uint32_t)NC - 1u);  // (NT = 1, odd count: a spare column)
+                return tile + c * cstride + (NT == 1 ? 0u : 512u * (uint32_t)t);
+            };
+            auto fetch = [&](uint32_t u, int t, SplitTileF32& o) __attribute__((always_inline)) {
                 float in[8];
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
-                    const f32x4 q = *reinterpret_cast<const f32x4*>(at(t) + 256u * h + 4u * lane);
+                    const f32x4 q = *reinterpret_cast<const f32x4*>(at(u, t) + 256u * h + 4u * lane);
 #pragma unroll
                     for (int r = 0; r < 4; ++r) in[4 * h + r] = q[r];
                 }
                 split_tile_f32(in, o);
             };
+            if (units == 0u) return;
             SplitTileF32 cur[2], nxt[2];
-            fetch(0, cur[0]);
-            fetch(1, cur[1]);
-            f32x4 held[HOLD][2];
+            fetch(0u, 0, cur[0]);
+            fetch(0u, 1, cur[1]);
+            auto unit = [&](uint32_t u, bool more) __attribute__((always_inline)) {
+                f32x4 held[HOLD][2];
 #pragma unroll
-            for (int p = 0; p < PAIRS; ++p) {
-                if (p + 1 < PAIRS) {
-                    fetch(2 * p + 2, nxt[0]);
-                    fetch(2 * p + 3, nxt[1]);
+                for (int q = 0; q < UPAIRS; ++q) {
+                    if (q + 1 < UPAIRS) {
+                        fetch(u, 2 * q + 2, nxt[0]);
+                        fetch(u, 2 * q + 3, nxt[1]);
+                    } else if (more) {
+                        fetch(u + 1u, 0, nxt[0]);
+                        fetch(u + 1u, 1, nxt[1]);
+                    }
+                    f32x4 a[2][2];
+                    tile_pair_mfma_f32(cur, ops, a);
+#pragma unroll
+                    for (int c = 0; c < 2; ++c)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) held[2 * q + c][h] = a[c][h];
+                    cur[0] = nxt[0];
+                    cur[1] = nxt[1];
                 }
-                f32x4 a[2][2];
-                tile_pair_mfma_f32(cur, ops, a);
+                if constexpr (NT > 1) cross_tile_butterflies<NT, XB>(held);
 #pragma unroll
-                for (int c = 0; c < 2; ++c)
+                for (int i = 0; i < HOLD; ++i)
 #pragma unroll
-                    for (int h = 0; h < 2; ++h) held[(2 * p + c) % HOLD][h] = a[c][h];
-                if ((2 * p + 2) % HOLD == 0) {
-                    if constexpr (NT > 1) cross_tile_butterflies<NT, XB>(held);
+                    for (int h = 0; h < 2; ++h)
+                        *reinterpret_cast<f32x4*>(at(u, i) + 256u * h + 4u * lane) = held[i][h] * scale;
+            };
+            // a full tile: the same number of units for every wavefront, one straight-line sequence
+            constexpr uint32_t FULL_UNITS = (NC / 4) / (NT == 1 ? 2 : 1);
+            if (ncols == (uint32_t)NC) {
 #pragma unroll
-                    for (int i = 0; i < HOLD; ++i)
-#pragma unroll
-                        for (int h = 0; h < 2; ++h)
-                            *reinterpret_cast<f32x4*>(at(2 * p + 2 - HOLD + i) + 256u * h + 4u * lane) =
-                                held[i][h] * scale;
-                }
-                cur[0] = nxt[0];
-                cur[1] = nxt[1];
+                for (uint32_t u = 0; u < FULL_UNITS; ++u) unit(u, u + 1u < FULL_UNITS);
+            } else {
+                for (uint32_t u = 0; u < units; ++u) unit(u, u + 1u < units);
             }
         };
         if (N == 512u)
