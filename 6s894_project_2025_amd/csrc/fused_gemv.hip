@@ -202,8 +202,9 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
                 }
         }
     };
-    // The first W fragments do not depend on the transform: start them before the prologue.
-    start_block(m_first);
+    // The first W fragments do not depend on the transform.  N < 512: start them before the
+    // prologue; N >= 512: behind the loads of the column tile, which the prologue waits for first.
+    if constexpr (!TILED) start_block(m_first);
 
     // ---- prologue: T = scale * H_N * X[:, b0:b0+16] --------------------------------------------
     const uint32_t cstride = N + kPad;  // TILED: floats per column of TT
@@ -245,6 +246,7 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
                 }
             }
         }
+        start_block(m_first);
         __syncthreads();
         // Wavefront w transforms columns w, w + 4, w + 8, ... of the tile, those that exist in X
         // (a last or only column group may hold fewer than NC: with B = 8 every wavefront has two
