@@ -50,6 +50,18 @@ constexpr uint32_t kXcds = 8;
 // consecutive k of one column.
 constexpr uint32_t kPad = 4;
 
+// Workgroup barrier for data exchanged through LDS only.  __syncthreads() also waits for every
+// outstanding global load (a release at workgroup scope), which would end the flight of the W
+// fragments requested ahead of the prologue and of the next row block at exactly the points
+// where they are meant to overlap other work; nothing here passes data between wavefronts through
+// global memory.
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 // physical row of logical row r in the LDS tile: low two bits mixed with bits 2-3 and 4-5
 __device__ __forceinline__ uint32_t prow(uint32_t r)
 {
@@ -134,14 +146,20 @@ __device__ __forceinline__ void pass_w(int wbits, const float* __restrict__ X, f
 // MI = 16-row blocks of W per workgroup (16, 32 or 64 rows).  The four wavefronts split the K range
 // of the product between them (every wavefront covers all MI row blocks over a quarter of N), so
 // each one streams a short, deeply prefetched run of W, and the partial sums meet in LDS.
-template <int MI, bool TILED, int NC, int PF>
-__global__ void __launch_bounds__(kThreads)
+// WAVES = wavefronts per workgroup.  Every launch uses four: eight (two per SIMD, for the shapes
+// where a compute unit holds one workgroup anyway) measured no faster, since the transform of a
+// column costs a SIMD about 1 400 cycles of MFMA and vector issue whoever issues them (M = N = 1024:
+// B = 64 8.7 instead of 9.2 us, B = 8 8.9 instead of 8.5, B = 2048 59.7 instead of 52.7 with the
+// sums then going through LDS in two phases).
+template <int MI, bool TILED, int NC, int PF, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
 fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
                      float* __restrict__ Y, uint32_t M, uint32_t N, uint32_t B, uint32_t logN,
                      float scale, uint32_t rows_per_group, uint32_t col_groups, uint32_t row_groups,
                      uint32_t per_xcd)
 {
     static_assert(NC == kCols || (TILED && NC == 2 * kCols), "wider tiles only in the column-major form");
+    static_assert(WAVES == kThreads / 64 || (TILED && WAVES == 8), "the register-butterfly prologue is written for 256 threads");
     constexpr int NF = NC / 16;  // 16-column fragments of the product per workgroup
     extern __shared__ __attribute__((aligned(16))) float tile[];  // [N][16] rows swizzled, then sums
     // Workgroups are handed to the eight XCDs in turn, each with an L2 of its own.  Position
@@ -164,7 +182,7 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
     // left the K loop at half the rate of the matrix cores.  (The 32-column workgroups are bound by
     // the matrix cores with four; eight measured slower, 40.7 -> 44.2 us for four row blocks.)
     const uint32_t total = N >> 4;
-    const uint32_t quarter = (total + 3u) / 4u;
+    const uint32_t quarter = (total + (uint32_t)WAVES - 1u) / (uint32_t)WAVES;  // a wavefront's share of the K steps
     const uint32_t k_begin = min(wave * quarter, total), k_end = min(k_begin + quarter, total);
     // The wavefront's i-th K step.  TILED (N >= 512, so the steps divide evenly): steps 2p and
     // 2p+1 of a wavefront are the two 64-byte halves of one 128-byte line of each row of W, asked
@@ -172,7 +190,7 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
     // each, the halves of a line were asked for a step apart, with 256 other lines of rows a
     // multiple of 4 KB apart in between.  Measured: N = 2048, 33.6 -> 31.4 thousand cycles per
     // row block; N = 1024, no change.)
-    auto kof = [&](uint32_t i) { return TILED ? ((i >> 1) << 3) + 2u * wave + (i & 1u) : k_begin + i; };
+    auto kof = [&](uint32_t i) { return TILED ? (i >> 1) * (2u * WAVES) + 2u * wave + (i & 1u) : k_begin + i; };
     const float* wrow[MI];
     f32x4 a[PF][MI];
     auto rows_of = [&](uint32_t mb, const float* (&rows)[MI]) {
@@ -213,8 +231,8 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
         // covers 16 rows by 16 columns, so that its four-byte LDS writes (bank = 16 * (column / 4) +
         // row modulo 64) never meet in a bank.
         {
-            constexpr uint32_t WQ = NC / 16;        // wavefronts side by side along a row
-            constexpr uint32_t RP = 16u * 4u / WQ;  // rows per pass of the workgroup
+            constexpr uint32_t WQ = NC / 16;                     // wavefronts side by side along a row
+            constexpr uint32_t RP = 16u * (uint32_t)WAVES / WQ;  // rows per pass of the workgroup
             const uint32_t q4 = (lane & 3u) + 4u * (wave % WQ), r0 = (lane >> 2) + 16u * (wave / WQ);
             // this thread's four columns: all inside X and 16-byte loadable, some, or none
             const uint32_t c4 = b0 + 4u * q4;
@@ -222,7 +240,8 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
             const bool any = c4 < B;
             // DEPTH rows in flight per thread (DEPTH * RP divides 512): the tile is NC * 4 bytes of
             // each of N rows, from the L2
-            constexpr int DEPTH = NC == kCols ? 8 : 16;
+            constexpr int DEPTH = 512u / RP;
+            static_assert(DEPTH >= 1 && DEPTH <= 16, "a round of DEPTH passes covers 512 rows");
             for (uint32_t rb = r0; rb < N; rb += (uint32_t)DEPTH * RP) {
                 f32x4 v[DEPTH];
 #pragma unroll
@@ -247,7 +266,7 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
             }
         }
         start_block(m_first);
-        __syncthreads();
+        lds_barrier();
         // Wavefront w transforms columns w, w + 4, w + 8, ... of the tile, those that exist in X
         // (a last or only column group may hold fewer than NC: with B = 8 every wavefront has two
         // columns to do, not four for two of them and four columns of zeros for the others).  Its
@@ -264,12 +283,12 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
             constexpr int HOLD = NT > 2 ? NT : 2;        // tiles of a unit: a column, or two of one tile
             constexpr int UPAIRS = HOLD / 2;             // pairs of tiles per unit
             const uint32_t ncols = min((uint32_t)NC, B - b0);
-            const uint32_t mine = ncols > wave ? (ncols - wave + 3u) / 4u : 0u;  // columns of this wavefront
+            const uint32_t mine = ncols > wave ? (ncols - wave + WAVES - 1u) / WAVES : 0u;  // columns of this wavefront
             const uint32_t units = NT == 1 ? (mine + 1u) / 2u : mine;
             // tile t of unit u: NT > 1: tile t of the wavefront's u-th column; NT = 1: column 2u + t
             auto at = [&](uint32_t u, int t) {
                 const uint32_t j = NT == 1 ? 2u * u + (uint32_t)t : u;
-                const uint32_t c = min(wave + 4u * j, (uint32_t)NC - 1u);  // (NT = 1, odd count: a spare column)
+                const uint32_t c = min(wave + (uint32_t)WAVES * j, (uint32_t)NC - 1u);  // (NT = 1, odd count: a spare column)
                 return tile + c * cstride + (NT == 1 ? 0u : 512u * (uint32_t)t);
             };
             auto fetch = [&](uint32_t u, int t, SplitTileF32& o) __attribute__((always_inline)) {
@@ -314,7 +333,7 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
                         *reinterpret_cast<f32x4*>(at(u, i) + 256u * h + 4u * lane) = held[i][h] * scale;
             };
             // a full tile: the same number of units for every wavefront, one straight-line sequence
-            constexpr uint32_t FULL_UNITS = (NC / 4) / (NT == 1 ? 2 : 1);
+            constexpr uint32_t FULL_UNITS = (NC / WAVES) / (NT == 1 ? 2 : 1);
             if (ncols == (uint32_t)NC) {
 #pragma unroll
                 for (uint32_t u = 0; u < FULL_UNITS; ++u) unit(u, u + 1u < FULL_UNITS);
@@ -328,7 +347,7 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
             transform_columns(std::integral_constant<int, 2>{});
         else
             transform_columns(std::integral_constant<int, 4>{});
-        __syncthreads();
+        lds_barrier();
     } else {
         uint32_t done = 0;
         bool first = true;
@@ -448,69 +467,91 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
             }
         }
 
-        // ---- meet the four K quarters in LDS ------------------------------------------------------
-        // Fragment g is finished by wavefront g % 4, which keeps its own partial sum in registers:
-        // only the other three go through LDS (12 KB instead of 16 for 64 rows by 16 columns, which
-        // is what lets two such workgroups with N = 1024 share a compute unit).  The sum is taken in
-        // the order of the wavefronts, whoever holds which part.
-        __syncthreads();  // the previous block's sums have been read
-#pragma unroll
-        for (int g = 0; g < MI * NF; ++g) {
-            const uint32_t owner = (uint32_t)(g & 3);
-            if (wave != owner) red[((uint32_t)g * 3u + (wave < owner ? wave : wave - 1u)) * 64u + lane] = acc[g];
-        }
-        __syncthreads();
+        // ---- meet the wavefronts' K shares in LDS ------------------------------------------------
+        // Fragment g is finished by wavefront g % WAVES, which keeps its own partial sum in
+        // registers: only the others go through LDS (12 KB instead of 16 for 64 rows by 16 columns
+        // and four wavefronts, which is what lets two such workgroups with N = 1024 share a compute
+        // unit).  With eight wavefronts the fragments go in phases of kPhaseFrags, so that the
+        // region stays within what the tile leaves of the LDS.  The sum is taken in the order of
+        // the wavefronts, whoever holds which part.
+        constexpr int G = MI * NF;
+        constexpr int kPhaseFrags = WAVES == 8 && G > 4 ? 4 : G;
         // D[m'][n']: n' = lo is the column, m' = 4*hi + r the row inside the 16-row block
 #pragma unroll
-        for (int g = 0; g < MI * NF; ++g) {
-            constexpr int kWaves = kThreads / 64;
-            const int owner = g & 3;
-            if (wave != (uint32_t)owner) continue;
-            f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+        for (int g0 = 0; g0 < G; g0 += kPhaseFrags) {
+            lds_barrier();  // the sums of the phase (or row block) before have been read
 #pragma unroll
-            for (int w = 0; w < kWaves; ++w) {
-                const f32x4 part = w == owner ? acc[g] : red[(g * 3 + (w < owner ? w : w - 1)) * 64 + lane];
-                sum = w == 0 ? part : sum + part;
+            for (int g = g0; g < g0 + kPhaseFrags; ++g) {
+                const uint32_t owner = (uint32_t)(g % WAVES);
+                if (wave != owner)
+                    red[((uint32_t)(g - g0) * (WAVES - 1) + (wave < owner ? wave : wave - 1u)) * 64u + lane] = acc[g];
             }
-            const uint32_t col = b0 + 16u * (uint32_t)(g % NF) + lo;
-            if (col < B) {
+            lds_barrier();
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const uint32_t m = mb + 16u * (uint32_t)(g / NF) + 4u * hi + r;
-                    if (m < M) Y[(uint64_t)m * B + col] = sum[r];
+            for (int g = g0; g < g0 + kPhaseFrags; ++g) {
+                const int owner = g % WAVES;
+                if (wave != (uint32_t)owner) continue;
+                f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) {
+                    const f32x4 part =
+                        w == owner ? acc[g] : red[((g - g0) * (WAVES - 1) + (w < owner ? w : w - 1)) * 64 + lane];
+                    sum = w == 0 ? part : sum + part;
+                }
+                const uint32_t col = b0 + 16u * (uint32_t)(g % NF) + lo;
+                if (col < B) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const uint32_t m = mb + 16u * (uint32_t)(g / NF) + 4u * hi + r;
+                        if (m < M) Y[(uint64_t)m * B + col] = sum[r];
+                    }
                 }
             }
         }
     }
 }
 
-template <int MI, bool TILED, int NC, int PF = 4>
+// How the tiles of Y are spread: a workgroup keeps its transformed tile for several row blocks once
+// there are more row blocks than it takes to give every compute unit as many workgroups as fit its
+// LDS (two are counted on where they fit).
+struct GemvPlan {
+    uint32_t col_groups, rows_per_group, row_groups;
+    uint32_t workgroups() const { return col_groups * row_groups; }
+};
+inline size_t gemv_lds_bytes(uint32_t N, bool tiled, uint32_t nc, uint32_t mi, uint32_t waves)
+{
+    const uint32_t frags = mi * (nc / 16u), phase = waves == 8u && frags > 4u ? 4u : frags;
+    return (size_t)(N + (tiled ? kPad : 0u)) * nc * sizeof(float) + (size_t)(waves - 1u) * phase * 64u * sizeof(f32x4);
+}
+inline GemvPlan plan_gemv(uint32_t M, uint32_t B, uint32_t nc, uint32_t block_rows, size_t lds)
+{
+    GemvPlan p;
+    p.col_groups = (B + nc - 1u) / nc;
+    const uint32_t row_blocks = (M + block_rows - 1u) / block_rows;
+    uint32_t groups_y = ((lds <= 80u * 1024u ? 512u : 256u) + p.col_groups - 1u) / p.col_groups;
+    if (groups_y > row_blocks) groups_y = row_blocks;
+    p.rows_per_group = ((row_blocks + groups_y - 1u) / groups_y) * block_rows;
+    p.row_groups = (M + p.rows_per_group - 1u) / p.rows_per_group;
+    return p;
+}
+
+template <int MI, bool TILED, int NC, int PF = 4, int WAVES = 4>
 int launch_gemv_as(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B,
                    float scale, hipStream_t s)
 {
-    const size_t lds = (size_t)(N + (TILED ? kPad : 0u)) * NC * sizeof(float) +
-                       3u * MI * (NC / 16) * 64u * sizeof(f32x4);
+    const size_t lds = gemv_lds_bytes(N, TILED, NC, MI, WAVES);
     // the tile transform's two MFMA stages attenuate by a power of two that the scale takes back
     if (TILED) scale = (float)((double)scale * (double)(1u << tile_stage_shift<4>(9u, false)));
-    auto kern = fused_ht_gemv_kernel<MI, TILED, NC, PF>;
+    auto kern = fused_ht_gemv_kernel<MI, TILED, NC, PF, WAVES>;
     if (lds > 64u * 1024u) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
             return MI_ERR_LAUNCH;
     }
-    // A workgroup keeps its transformed tile for several row blocks once there are more row
-    // blocks than it takes to give every compute unit as many workgroups as fit its LDS (two are
-    // counted on where they fit).
-    constexpr uint32_t kBlock = 16u * MI;
-    const uint32_t col_groups = (B + NC - 1) / NC;
-    const uint32_t row_blocks = (M + kBlock - 1) / kBlock;
-    uint32_t groups_y = ((lds <= 80u * 1024u ? 512u : 256u) + col_groups - 1) / col_groups;
-    if (groups_y > row_blocks) groups_y = row_blocks;
-    const uint32_t rows_per_group = ((row_blocks + groups_y - 1) / groups_y) * kBlock;
-    const uint32_t row_groups = (M + rows_per_group - 1) / rows_per_group;
-    const uint32_t per_xcd = (col_groups * row_groups + kXcds - 1) / kXcds;
-    hipLaunchKernelGGL(kern, dim3(per_xcd * kXcds), dim3(kThreads), lds, s, W, X, Y, M, N, B,
-                       ilog2(N), scale, rows_per_group, col_groups, row_groups, per_xcd);
+    const GemvPlan p = plan_gemv(M, B, NC, 16u * MI, lds);
+    const uint32_t per_xcd = (p.workgroups() + kXcds - 1) / kXcds;
+    hipLaunchKernelGGL(kern, dim3(per_xcd * kXcds), dim3(64 * WAVES), lds, s, W, X, Y, M, N, B,
+                       ilog2(N), scale, p.rows_per_group, p.col_groups, p.row_groups, per_xcd);
     return launch_status();
 }
 
@@ -518,10 +559,12 @@ template <int MI>
 int launch_gemv(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B,
                 float scale, hipStream_t s)
 {
+    if (N < 512u) return launch_gemv_as<MI, false, kCols>(W, X, Y, M, N, B, scale, s);
+    // N = 2048 with 64-row blocks: a deeper load ring (one workgroup per compute unit: the tile is
+    // 128 KB)
     if constexpr (MI == 4)
         if (N == 2048u) return launch_gemv_as<MI, true, kCols, 8>(W, X, Y, M, N, B, scale, s);
-    return N >= 512u ? launch_gemv_as<MI, true, kCols>(W, X, Y, M, N, B, scale, s)
-                     : launch_gemv_as<MI, false, kCols>(W, X, Y, M, N, B, scale, s);
+    return launch_gemv_as<MI, true, kCols>(W, X, Y, M, N, B, scale, s);
 }
 
 }  // namespace
