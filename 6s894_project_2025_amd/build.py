@@ -188,6 +188,73 @@ def check_m0_is_the_transfers_alone(asm_text: str, where: str) -> int:
     return writes
 
 
+_LGKM_WAIT = re.compile(r"lgkmcnt\((\d+)\)")
+kLdsReadHorizon = 400  # instructions followed per path; a fragment is used within a few K steps
+
+
+def check_lds_reads_waited_for(asm_text: str, where: str) -> int:
+    """An LDS read written as an opaque statement returns a register that holds nothing until a
+    hand-placed `s_waitcnt lgkmcnt` has covered it.  Raises if, on any path the branches allow, an
+    instruction reads or overwrites the destination of a `ds_read` before a wait that covers it
+    (LDS operations complete in order: a wait for at most as many outstanding operations as were
+    issued after the read); returns the number of reads checked.  Compiler-generated reads are
+    checked alike (the compiler waits before their first use)."""
+    checked = 0
+    lines = asm_text.splitlines()
+    i = 0
+    while i < len(lines):
+        label = _LABEL.match(lines[i])
+        if not label:
+            i += 1
+            continue
+        name = label.group(1)
+        ins, labels = [], {}
+        i += 1
+        while i < len(lines) and not _LABEL.match(lines[i]):
+            text = lines[i].split(";")[0].strip()
+            local = _ANY_LABEL.match(text)
+            if local:
+                labels[local.group(1)] = len(ins)
+            elif text and not text.startswith("."):
+                ins.append(text)
+            i += 1
+        for at, text in enumerate(ins):
+            if not text.startswith("ds_read"):
+                continue
+            checked += 1
+            dest = frozenset(_vregs(text.split(",")[0]))
+            seen = set()
+            todo = [(at + 1, 0, kLdsReadHorizon)]  # position, LDS operations issued since, steps left
+            while todo:
+                k, younger, left = todo.pop()
+                while left > 0 and k < len(ins) and (k, younger) not in seen:
+                    seen.add((k, younger))
+                    t = ins[k]
+                    op = t.split()[0]
+                    if op == "s_endpgm":
+                        break
+                    if op == "s_waitcnt":
+                        m = _LGKM_WAIT.search(t)
+                        if m and int(m.group(1)) <= younger:
+                            break  # covered on this path
+                    elif op == "s_branch":
+                        k = labels.get(t.split()[1], len(ins))
+                        left -= 1
+                        continue
+                    else:
+                        touched = _vregs(t if op.startswith(_NO_DESTINATION) else t.partition(" ")[2])
+                        if touched & dest:
+                            raise RuntimeError(f"{where}: {name}: `{t}` touches the destination of `{text}` "
+                                               f"before an s_waitcnt lgkmcnt that covers it")
+                        if op.startswith("ds_"):
+                            younger += 1
+                        if op.startswith("s_cbranch"):
+                            todo.append((labels.get(t.split()[1], len(ins)), younger, left - 1))
+                    left -= 1
+                    k += 1
+    return checked
+
+
 def sources() -> list[str]:
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
@@ -222,6 +289,8 @@ def _compile(src: str) -> str:
             raise RuntimeError(f"{base}: no register-resident MFMA loop found in the device assembly")
         if check_m0_is_the_transfers_alone(text, base) == 0:
             raise RuntimeError(f"{base}: no global -> LDS transfer found in the device assembly")
+        if check_lds_reads_waited_for(text, base) == 0:
+            raise RuntimeError(f"{base}: no LDS read found in the device assembly")
         for t in temps:
             os.remove(t)
     return obj

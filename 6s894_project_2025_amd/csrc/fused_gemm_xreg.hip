@@ -526,6 +526,13 @@ fused_ht_gemm_xreg_kernel(const typename T16::E* __restrict__ W,
                 }
             }
         }
+        // Control leaves this variant of the block with the fragments of the next block's first
+        // two K steps requested.  The variants need not agree on which registers hold the fragment
+        // ring, so the compiler may copy fragment registers on the edge between two of them, and
+        // a copy reads its source at once: the reads must have landed before the edge (the last
+        // of them was issued NM - 4 MFMAs ago).  The build checks the generated ISA for this
+        // (build.py: check_lds_reads_waited_for).
+        wait_lds();
     };
 
     auto store_block = [&](f32x4 (&acc)[4][NBF], uint64_t base) __attribute__((always_inline)) {

@@ -381,6 +381,11 @@ fused_ht_gemm_xreg_k2048_kernel(const typename T16::E* __restrict__ W, const typ
         // (Nothing here reads the accumulators: the next block's K step 0 hands them over behind its
         // fourth MFMA at the earliest, long after the last MFMA above has retired.  The build checks
         // the generated code for copies the register allocator might put on the loop edge.)
+        // Such copies do get made of the fragment ring, whose registers the variants of this body
+        // need not agree on, and a copy reads its source at once: the fragment reads requested for
+        // the next block's first two K steps must have landed before control leaves this variant
+        // (build.py: check_lds_reads_waited_for).
+        wait_lds();
     };
     // the same meeting of the halves with nothing to hide it behind: the last block of a workgroup,
     // and blocks whose stores need bounds checks

@@ -254,3 +254,42 @@ def test_build_rejects_other_uses_of_m0():
     for other in ("\ts_mov_b32 m0, s9\n", "\ts_mov_b32 s9, m0\n", "\tv_readlane_b32 s4, v3, m0\n"):
         with pytest.raises(RuntimeError, match="uses M0"):
             build.check_m0_is_the_transfers_alone(good.replace("\ts_endpgm\n", other + "\ts_endpgm\n"), "bad")
+
+
+def test_build_rejects_uses_of_an_lds_read_before_its_wait():
+    """An LDS read written as an opaque statement returns a register that holds nothing until a
+    hand-placed s_waitcnt lgkmcnt covers it; the build follows every path from each ds_read and fails
+    on an instruction that reads or overwrites the destination first (a register copy the allocator
+    puts on the edge between two variants of a loop body, say)."""
+    import importlib
+    build = importlib.import_module("6s894_project_2025_amd.build")
+    head = "_Zk: ; @_Zk\n.LBB0_1:\n\tds_read_b128 v[112:115], v128 offset:0\n"
+    tail = "\ts_endpgm\n"
+    mfma = "\tv_mfma_f32_16x16x32_bf16 v[32:35], v[96:99], a[124:127], v[32:35]\n"
+    younger = "\tds_read_b128 v[116:119], v128 offset:0x2000\n"
+
+    def check(body):
+        return build.check_lds_reads_waited_for(head + body + tail, "t")
+
+    # waited for, then used; a wait that allows as many outstanding operations as are younger covers it
+    assert check(mfma * 4 + "\ts_waitcnt lgkmcnt(0)\n\tv_mov_b64_e32 v[76:77], v[112:113]\n") == 1
+    assert check(younger + "\ts_waitcnt lgkmcnt(1)\n\tv_mfma_f32_16x16x32_bf16 v[32:35], v[112:115], a[0:3], v[32:35]\n"
+                 "\ts_waitcnt lgkmcnt(0)\n") == 2
+    assert check("\ts_waitcnt vmcnt(8) lgkmcnt(0)\n\tv_mov_b32_e32 v1, v112\n") == 1
+    # never used on this path: nothing to complain about
+    assert check(mfma * 3) == 1
+    # used, or overwritten, before any wait, or behind one that does not reach back far enough
+    with pytest.raises(RuntimeError, match="touches the destination"):
+        check(mfma * 4 + "\tv_mov_b64_e32 v[76:77], v[112:113]\n")
+    with pytest.raises(RuntimeError, match="touches the destination"):
+        check("\tv_mfma_f32_16x16x32_bf16 v[32:35], v[112:115], a[0:3], v[32:35]\n")
+    with pytest.raises(RuntimeError, match="touches the destination"):
+        check("\tv_mov_b32_e32 v113, v5\n")
+    with pytest.raises(RuntimeError, match="touches the destination"):
+        check(younger + "\ts_waitcnt lgkmcnt(2)\n\tv_mov_b32_e32 v1, v112\n")
+    with pytest.raises(RuntimeError, match="touches the destination"):
+        check("\ts_waitcnt vmcnt(0)\n\tds_write_b128 v7, v[112:115] offset:1024\n")
+    # branches are followed both ways: the copy sits on an edge that skips the wait
+    with pytest.raises(RuntimeError, match="touches the destination"):
+        check("\ts_cbranch_vccnz .LBB0_9\n\ts_waitcnt lgkmcnt(0)\n\ts_endpgm\n.LBB0_9:\n\tv_mov_b64_e32 v[76:77], v[112:113]\n")
+    assert check("\ts_waitcnt lgkmcnt(0)\n\ts_cbranch_vccnz .LBB0_9\n\ts_endpgm\n.LBB0_9:\n\tv_mov_b64_e32 v[76:77], v[112:113]\n") == 1
