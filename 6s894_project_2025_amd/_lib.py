@@ -31,6 +31,7 @@ PROBE_LIB_PATH = os.path.join(HERE, "libmi_probe.so")
 PROBE_SIGNATURES = {
     "mi_probe_mfma_rate": (_i, [_i, _i, _u32, _u32, _vp, _vp, _vp]),
     "mi_probe_issue_rate": (_i, [_i, _i, _i, _u32, _u32, _vp, _vp, _vp, _vp]),
+    "mi_probe_stream_rate": (_i, [_i, _u32, _u32, _u64, _vp, _vp, _vp]),
 }
 
 _lib = None

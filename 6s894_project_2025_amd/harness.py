@@ -344,6 +344,44 @@ def run_issue_probe(reps: int = 1000) -> list[dict[str, Any]]:
     return rows
 
 
+def run_stream_probe(bytes_per_wave: int = 256 * 1024, launches: int = 20) -> list[dict[str, Any]]:
+    """How fast a compute unit takes data in (``mi_probe_stream_rate``): every compute unit streams
+    1 MB (four wavefronts x ``bytes_per_wave``) per launch, through direct global -> LDS transfers or
+    ordinary loads, with 4, 8 or 16 KB requested ahead per wavefront, from regions that are read by
+    one workgroup (everything comes from beyond the L2), by eight (one reader per XCD: the same) or
+    by 32 consecutive ones (four readers per XCD: three of four requests can hit the L2)."""
+    from . import _lib
+
+    lib = _lib.load_probe()
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    src = torch.ones(256 * 4 * bytes_per_wave, dtype=torch.uint8, device=dev)
+    out = torch.zeros(65536, dtype=torch.int32, device=dev)
+    rows = []
+    for share in (1, 8, 32):
+        for mode, name in ((0, "global_load_lds_dwordx4"), (1, "global_load_dwordx4")):
+            for depth in (4, 8, 16):
+                def call():
+                    _lib.check(lib.mi_probe_stream_rate(mode, depth, share, bytes_per_wave, src.data_ptr(),
+                                                        out.data_ptr(), stream), "stream probe")
+                for _ in range(3):
+                    call()
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                for _ in range(launches):
+                    call()
+                b.record()
+                b.synchronize()
+                us = a.elapsed_time(b) * 1e3 / launches
+                per_cu = 4 * bytes_per_wave / us * 1e-3
+                rows.append({"instruction": name, "kb_ahead_per_wave": depth, "readers_per_region": share,
+                             "us_per_launch": us, "gb_per_s_per_cu": per_cu, "tb_per_s_total": per_cu * 256e-3})
+                print(f"{name:24s} {depth:2d} KB ahead per wavefront, {share:2d} reader(s) per region: "
+                      f"{us:7.2f} us per launch (launch gap included), {per_cu:6.1f} GB/s per compute unit, "
+                      f"{per_cu * 256e-3:5.2f} TB/s in all")
+    return rows
+
+
 def _read_power_and_clock() -> dict[str, Any]:
     """Package power (W) and the current shader clock level from the amdgpu sysfs files, which an
     ordinary user may read; empty where the files are absent."""
@@ -552,6 +590,7 @@ def main(argv=None) -> int:
     p4 = sub.add_parser("mfma")
     p4.add_argument("--steps", type=int, default=4096)
     sub.add_parser("issue")
+    sub.add_parser("stream")
     p6 = sub.add_parser("power")
     p6.add_argument("--seconds", type=float, default=1.5)
     p3 = sub.add_parser("plot")
@@ -570,6 +609,9 @@ def main(argv=None) -> int:
         return 0
     if args.cmd == "issue":
         run_issue_probe()
+        return 0
+    if args.cmd == "stream":
+        run_stream_probe()
         return 0
     if args.cmd == "power":
         run_power(args.seconds)

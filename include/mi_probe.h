@@ -43,6 +43,21 @@ int mi_probe_mfma_rate(int shape, int lds_reads, uint32_t waves_per_simd, uint32
 int mi_probe_issue_rate(int mode, int kind, int n, uint32_t waves_per_simd, uint32_t reps,
                         const float* in, float* out, uint64_t* cycles, void* stream);
 
+/*
+ * Streaming-rate probe: 256 workgroups of four wavefronts (one per compute unit); every wavefront
+ * reads bytes_per_wave contiguous bytes, 1 KB per instruction, `depth` (4, 8 or 16) instructions
+ * requested before the older half is waited for; mode 0: global_load_lds_dwordx4 (global -> LDS
+ * directly), mode 1: global_load_dwordx4 into registers.  `share` (a divisor of 256) consecutive
+ * workgroup ids read the same region of 4 x bytes_per_wave bytes at src + (id / share) x that;
+ * consecutive ids run on different XCDs.  The caller times a series of launches; rate per compute
+ * unit = 4 x bytes_per_wave / time.  No counterpart in the reference.
+ *   src : device, 16-byte aligned, (256 / share) x 4 x bytes_per_wave bytes (any contents)
+ *   out : device, 65536 x uint32 (keeps the loads alive)
+ *   bytes_per_wave : a positive multiple of 16 KiB
+ */
+int mi_probe_stream_rate(int mode, uint32_t depth, uint32_t share, uint64_t bytes_per_wave,
+                         const void* src, uint32_t* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

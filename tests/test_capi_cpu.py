@@ -39,7 +39,8 @@ def test_probe_library_is_separate_from_the_product_library(libmod):
     # the matrix-core rate probe is a measurement aid: its own header, its own library, and the
     # product library exports nothing of it
     declared = _declared_symbols(PROBE_HEADER)
-    assert declared == sorted(libmod.PROBE_SIGNATURES) == ["mi_probe_issue_rate", "mi_probe_mfma_rate"]
+    assert declared == sorted(libmod.PROBE_SIGNATURES) == ["mi_probe_issue_rate", "mi_probe_mfma_rate",
+                                                           "mi_probe_stream_rate"]
     probe = libmod.load_probe()
     for name in declared:
         assert hasattr(probe, name)

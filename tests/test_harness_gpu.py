@@ -96,3 +96,15 @@ def test_mfma_probe_structure(harness):
         for key in ("tflops", "ghz", "cycles_per_step_per_simd", "us_per_launch"):
             assert math.isfinite(r[key]) and r[key] > 0.0, r
         assert r["cycles_per_step_per_simd"] > 125.0, r
+
+
+def test_stream_probe_structure(harness):
+    # structural properties only: every configuration reports a positive finite rate, and readers
+    # that share a region inside an XCD are not slower than readers that share nothing
+    import math
+    rows = harness.run_stream_probe(bytes_per_wave=64 * 1024, launches=5)
+    assert len(rows) == 3 * 2 * 3
+    for r in rows:
+        assert math.isfinite(r["gb_per_s_per_cu"]) and r["gb_per_s_per_cu"] > 0.0, r
+    best = lambda share: max(r["gb_per_s_per_cu"] for r in rows if r["readers_per_region"] == share)
+    assert best(32) >= 0.9 * best(1)
