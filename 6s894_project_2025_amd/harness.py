@@ -452,6 +452,12 @@ def run_power(seconds: float = 1.5) -> list[dict[str, Any]]:
     Wb, Xb = W.to(torch.bfloat16), X.to(torch.bfloat16)
     rows.append(watch("fused HT->GEMM bf16 K=1024 M=N=4096", lambda: fused_ht_gemm(Wb, Xb)))
     rows.append(watch("vendor GEMM bf16 K=1024 M=N=4096 (no transform)", lambda: torch.matmul(Wb, Xb.t())))
+    # the same launches on operands that do not toggle the matrix cores' inputs: the instruction
+    # stream and the bytes moved are identical, only the energy per MFMA differs
+    W1, X1 = torch.ones_like(Wb), torch.ones_like(Xb)
+    rows.append(watch("fused HT->GEMM bf16, W constant, X random", lambda: fused_ht_gemm(W1, Xb)))
+    rows.append(watch("fused HT->GEMM bf16, W and X constant", lambda: fused_ht_gemm(W1, X1)))
+    rows.append(watch("vendor GEMM bf16, W and X constant", lambda: torch.matmul(W1, X1.t())))
     rows.append(watch("fused HT->GEMM fp32 K=1024 M=N=4096", lambda: fused_ht_gemm(W, X)))
     W4 = torch.randn(4096, 4096, device=dev, generator=g).to(torch.bfloat16)
     X4 = torch.randn(4096, 4096, device=dev, generator=g).to(torch.bfloat16)
