@@ -145,6 +145,66 @@ def check_mfma_results_not_touched_early(asm_text: str, where: str) -> int:
     return checked
 
 
+kOperandReadSlots = 4  # issue slots during which a 16-pass-or-shorter MFMA may still be reading A
+
+
+def check_mfma_operands_not_overwritten_early(asm_text: str, where: str) -> int:
+    """The matrix core reads the A operand of an MFMA over several cycles after issue, and for an
+    inline-assembly MFMA the compiler inserts no wait states for that: a vector instruction that
+    writes one of those registers right behind the MFMA corrupts the product (observed with a
+    register copy one instruction later).  Raises if, within kOperandReadSlots issue slots of an
+    assembly MFMA (one whose B operand is an accumulation register) and on any path the branches
+    allow, a vector ALU instruction writes a register of its A operand; returns the number of MFMAs
+    checked.  (Loads are left alone: their data arrives far later than that.)"""
+    checked = 0
+    lines = asm_text.splitlines()
+    i = 0
+    while i < len(lines):
+        label = _LABEL.match(lines[i])
+        if not label:
+            i += 1
+            continue
+        name = label.group(1)
+        ins, labels = [], {}
+        i += 1
+        while i < len(lines) and not _LABEL.match(lines[i]):
+            text = lines[i].split(";")[0].strip()
+            local = _ANY_LABEL.match(text)
+            if local:
+                labels[local.group(1)] = len(ins)
+            elif text and not text.startswith("."):
+                ins.append(text)
+            i += 1
+        for at, text in enumerate(ins):
+            if not _MFMA_B_IN_AGPR.match(text):
+                continue
+            checked += 1
+            operand_a = frozenset(_vregs(text.split(",")[1]))
+            todo = [(at + 1, kOperandReadSlots)]
+            seen = set()
+            while todo:
+                k, left = todo.pop()
+                while left > 0 and k < len(ins) and (k, left) not in seen:
+                    seen.add((k, left))
+                    t = ins[k]
+                    op = t.split()[0]
+                    if op == "s_endpgm":
+                        break
+                    if op.startswith("v_") and not op.startswith("v_mfma") and not op.startswith("v_cmp"):
+                        if _vregs(t.partition(" ")[2].split(",")[0]) & operand_a:
+                            raise RuntimeError(f"{where}: {name}: `{t}` overwrites the A operand of `{text}` "
+                                               f"{kOperandReadSlots - left} issue slots after it")
+                    if op == "s_branch":
+                        k = labels.get(t.split()[1], len(ins))
+                        left -= 1
+                        continue
+                    if op.startswith("s_cbranch"):
+                        todo.append((labels.get(t.split()[1], len(ins)), left - 1))
+                    left -= int(t.split()[1], 0) + 1 if op == "s_nop" else 1
+                    k += 1
+    return checked
+
+
 def check_register_resident_isa(asm_text: str, where: str) -> int:
     """Raises if a kernel writes accumulation registers after its first MFMA that reads its B
     operand from them; returns the number of kernels checked."""
@@ -291,6 +351,7 @@ def _compile(src: str) -> str:
             raise RuntimeError(f"{base}: no global -> LDS transfer found in the device assembly")
         if check_lds_reads_waited_for(text, base) == 0:
             raise RuntimeError(f"{base}: no LDS read found in the device assembly")
+        check_mfma_operands_not_overwritten_early(text, base)
         for t in temps:
             os.remove(t)
     return obj

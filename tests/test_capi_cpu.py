@@ -294,3 +294,29 @@ def test_build_rejects_uses_of_an_lds_read_before_its_wait():
     with pytest.raises(RuntimeError, match="touches the destination"):
         check("\ts_cbranch_vccnz .LBB0_9\n\ts_waitcnt lgkmcnt(0)\n\ts_endpgm\n.LBB0_9:\n\tv_mov_b64_e32 v[76:77], v[112:113]\n")
     assert check("\ts_waitcnt lgkmcnt(0)\n\ts_cbranch_vccnz .LBB0_9\n\ts_endpgm\n.LBB0_9:\n\tv_mov_b64_e32 v[76:77], v[112:113]\n") == 1
+
+
+def test_build_rejects_overwriting_an_assembly_mfma_operand_too_soon():
+    """The matrix core reads an MFMA's A operand over several cycles after issue; for an inline-assembly
+    MFMA the compiler adds no wait states, so the build fails on a vector instruction that writes
+    one of those registers within a few issue slots (a register copy right behind the MFMA, say)."""
+    import importlib
+    build = importlib.import_module("6s894_project_2025_amd.build")
+    head = "_Zk: ; @_Zk\n.LBB0_1:\n\tv_mfma_f32_16x16x32_bf16 v[32:35], v[96:99], a[124:127], v[32:35]\n"
+    tail = "\ts_endpgm\n"
+    filler = "\tv_add_u32_e32 v1, v2, v3\n"
+
+    def check(body):
+        return build.check_mfma_operands_not_overwritten_early(head + body + tail, "t")
+
+    # late enough, or not a vector ALU write (a load's data arrives much later; a read is harmless)
+    assert check(filler * build.kOperandReadSlots + "\tv_mov_b32_e32 v97, v5\n") == 1
+    assert check("\tds_read_b128 v[96:99], v128 offset:0\n") == 1
+    assert check("\tv_mov_b32_e32 v5, v97\n") == 1
+    assert check("\ts_nop 3\n\tv_mov_b32_e32 v97, v5\n") == 1
+    with pytest.raises(RuntimeError, match="overwrites the A operand"):
+        check("\tv_mov_b32_e32 v97, v5\n")
+    with pytest.raises(RuntimeError, match="overwrites the A operand"):
+        check(filler * 2 + "\tv_cvt_pk_bf16_f32 v99, v1, v2\n")
+    with pytest.raises(RuntimeError, match="overwrites the A operand"):
+        check("\ts_cbranch_vccnz .LBB0_9\n" + filler * 10 + ".LBB0_9:\n\tv_mov_b64_e32 v[98:99], v[4:5]\n")
