@@ -80,6 +80,24 @@ def test_gemv_large_launch_paths(pkg, oracle, M, N, B):
     assert np.abs(got - colsum).max() / np.abs(colsum).max() <= 1e-5
 
 
+def test_gemv_random_shapes(pkg, oracle):
+    # seeded sweep over the launch logic: every power of two N, row counts around the 16/32/64-row
+    # block sizes, batches around the 16- and 32-column tiles (whole, ragged, not a multiple of four)
+    rng = np.random.default_rng(20251125)
+    for _ in range(48):
+        N = 1 << int(rng.integers(1, 12))
+        M = int(rng.choice([1, 15, 16, 17, 31, 33, 63, 64, 65, 100, 129, 300, 777, 1024, 1500]))
+        B = int(rng.choice([1, 3, 4, 7, 16, 17, 20, 31, 32, 33, 48, 61, 64, 100, 255, 260, 600]))
+        if N >= 1024 and M * B > 400000:
+            M = 129
+        W, X = oracle.inputs_gemv(M, N, B)
+        Y = pkg.fused_ht_gemv(W.cuda(), X.cuda())
+        torch.cuda.synchronize()
+        want = oracle.fused_ht_gemv_f64_blas(W.double().numpy(), X.double().numpy(), 1.0 / math.sqrt(N))
+        assert Y.shape == (M, B)
+        assert _rel(oracle, Y, want) <= 1e-5, (M, N, B)
+
+
 def test_gemv_identity_reduces_to_transform(pkg, oracle):
     N, B = 256, 48
     _, X = oracle.inputs_gemv(N, N, B)
