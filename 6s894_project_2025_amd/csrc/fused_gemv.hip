@@ -156,25 +156,29 @@ __global__ void __launch_bounds__(64 * WAVES)
 fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
                      float* __restrict__ Y, uint32_t M, uint32_t N, uint32_t B, uint32_t logN,
                      float scale, uint32_t rows_per_group, uint32_t col_groups, uint32_t row_groups,
-                     uint32_t per_xcd)
+                     uint32_t per_xcd, bool col_major)
 {
     static_assert(NC == kCols || (TILED && NC == 2 * kCols), "wider tiles only in the column-major form");
     static_assert(WAVES == kThreads / 64 || (TILED && WAVES == 8), "the register-butterfly prologue is written for 256 threads");
     constexpr int NF = NC / 16;  // 16-column fragments of the product per workgroup
     extern __shared__ __attribute__((aligned(16))) float tile[];  // [N][16] rows swizzled, then sums
     // Workgroups are handed to the eight XCDs in turn, each with an L2 of its own.  Position
-    // (XCD, slot) takes place XCD * per_xcd + slot of the row-group-major order of the tiles, so
-    // that the column groups which share a slice of W run side by side on one XCD and read it
-    // from that L2 (W is read once per column group, X once per row group).
+    // (XCD, slot) takes place XCD * per_xcd + slot of an order of the tiles in which neighbours
+    // share data: row-group-major (the column groups that share a slice of W side by side on one
+    // XCD, which reads the slice once from beyond its L2 and all of X it needs) or, col_major,
+    // column-group-major (the row groups that share a column tile side by side: little of X per
+    // XCD, all of W).  The launcher picks the second when the first would have every XCD fetch
+    // more than 2 MB of X at once: the column tiles are wanted all at the same moment, at the
+    // start, while W is streamed over the whole K loop ((1024, 1024, 2048): 52.7 -> 48.7 us).
     const uint32_t place = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
     if (place >= col_groups * row_groups) return;
-    const uint32_t b0 = (place % col_groups) * NC;
+    const uint32_t b0 = (col_major ? place / row_groups : place % col_groups) * NC;
     // the wavefront's index as a scalar: everything derived from it (its K range above all) then
     // steers branches instead of lane masks
     const uint32_t lane = threadIdx.x & 63u, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t lo = lane & 15u, hi = lane >> 4;
     // this workgroup's rows: [m_first, m_last), a multiple of 16 * MI except at the end of W
-    const uint32_t m_first = (place / col_groups) * rows_per_group;
+    const uint32_t m_first = (col_major ? place % row_groups : place / col_groups) * rows_per_group;
     const uint32_t m_last = min(M, m_first + rows_per_group);
 
     // PF = K steps (of 16) in flight per wavefront: four, and eight for N = 2048, where a compute
@@ -550,8 +554,11 @@ int launch_gemv_as(const float* W, const float* X, float* Y, uint32_t M, uint32_
     }
     const GemvPlan p = plan_gemv(M, B, NC, 16u * MI, lds);
     const uint32_t per_xcd = (p.workgroups() + kXcds - 1) / kXcds;
+    // bytes of X an XCD needs under the row-group-major order: its column groups' tiles
+    const uint64_t x_per_xcd = (uint64_t)(p.col_groups < per_xcd ? p.col_groups : per_xcd) * NC * N * sizeof(float);
+    const bool col_major = x_per_xcd > (2ull << 20);
     hipLaunchKernelGGL(kern, dim3(per_xcd * kXcds), dim3(64 * WAVES), lds, s, W, X, Y, M, N, B,
-                       ilog2(N), scale, p.rows_per_group, p.col_groups, p.row_groups, per_xcd);
+                       ilog2(N), scale, p.rows_per_group, p.col_groups, p.row_groups, per_xcd, col_major);
     return launch_status();
 }
 
