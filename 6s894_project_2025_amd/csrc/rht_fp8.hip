@@ -11,11 +11,15 @@
 //   - the result rounded to bf16 as mi_fwht would store it, the row amax taken on the fp32 values
 //     by a lane reduction over the lanes that share a row,
 //   - v_cvt_pk_fp8_f32 for the narrowing (hardware RNE to E4M3FN), 8 codes = one 8-byte store.
-// The kernel is bound by vector-instruction issue, not by memory (the same loads and stores without
-// arithmetic take a third of the time at [8192, 4096]): it is kept at four wavefronts per SIMD
-// (at most 128 registers: simple two-operand instructions then issue every 2.2 cycles per SIMD,
-// conversions and three-operand ones every 4.3; with three wavefronts 2.7 and 5.2) and at as few
-// vector instructions per element as the arithmetic allows.
+// Two costs set the kernel's time at [8192, 4096].  Vector-instruction issue: a SIMD needs about
+// 1.0 us per row of 4096 with two or more wavefronts resident (1.4 us with one), 8 rows per SIMD;
+// hence four wavefronts per SIMD (at most 128 registers: simple two-operand instructions then issue
+// every 2.2 cycles per SIMD, conversions and three-operand ones every 4.3; with three wavefronts
+// 2.7 and 5.2) and as few vector instructions per element as the arithmetic allows.  And the memory
+// system: 100.7 MB per launch at the 6.6 - 7.0 TB/s that a read + write mix of this size reaches on
+// this chip are 14 - 15 us, which is what the span from the first wavefront's start to the last
+// one's end measures (15.4 us); prefetching rows, other workgroup sizes and handing rows out
+// dynamically all moved work between wavefronts without changing that total.
 #include <type_traits>
 
 #include "fwht_device.hpp"
