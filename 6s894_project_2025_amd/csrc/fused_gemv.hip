@@ -33,34 +33,19 @@
 //
 // Behaviour replaced: fused_hadamard_gemv_kernel(_vec), fused_ht/fwht_gemv_fusion.cu:98-244, where
 // every column's block re-reads all of W and reduces with warp shuffles.
-#include <type_traits>
-
-#include "fwht_device.hpp"
+#include "gemv_common.hpp"
 
 namespace mi {
 namespace {
 
 constexpr int kCols = 16;
 constexpr int kThreads = 256;
-constexpr uint32_t kXcds = 8;
 
-// N >= 512: column c of the transformed tile lives at TT + c * (N + kPad) floats.  With a row
-// stride of 16 bytes modulo 128 the 16-byte accesses of eight adjacent lanes (eight columns, the
-// same k) fall into eight different 16-byte columns of the LDS row, as do those of eight lanes on
-// consecutive k of one column.
-constexpr uint32_t kPad = 4;
-
-// Workgroup barrier for data exchanged through LDS only.  __syncthreads() also waits for every
-// outstanding global load (a release at workgroup scope), which would end the flight of the W
-// fragments requested ahead of the prologue and of the next row block at exactly the points
-// where they are meant to overlap other work; nothing here passes data between wavefronts through
-// global memory.
-__device__ __forceinline__ void lds_barrier()
-{
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-}
+using gemv::GemvPlan;
+using gemv::kPad;
+using gemv::kXcds;
+using gemv::lds_barrier;
+using gemv::plan_gemv;
 
 // physical row of logical row r in the LDS tile: low two bits mixed with bits 2-3 and 4-5
 __device__ __forceinline__ uint32_t prow(uint32_t r)
@@ -231,126 +216,10 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
     // ---- prologue: T = scale * H_N * X[:, b0:b0+16] --------------------------------------------
     const uint32_t cstride = N + kPad;  // TILED: floats per column of TT
     if constexpr (TILED) {
-        // X[:, b0 .. b0+NC-1] -> TT: a thread reads four adjacent columns of a row.  A wavefront
-        // covers 16 rows by 16 columns, so that its four-byte LDS writes (bank = 16 * (column / 4) +
-        // row modulo 64) never meet in a bank.
-        {
-            constexpr uint32_t WQ = NC / 16;                     // wavefronts side by side along a row
-            constexpr uint32_t RP = 16u * (uint32_t)WAVES / WQ;  // rows per pass of the workgroup
-            const uint32_t q4 = (lane & 3u) + 4u * (wave % WQ), r0 = (lane >> 2) + 16u * (wave / WQ);
-            // this thread's four columns: all inside X and 16-byte loadable, some, or none
-            const uint32_t c4 = b0 + 4u * q4;
-            const bool vec_ok = c4 + 4u <= B && (B & 3u) == 0;
-            const bool any = c4 < B;
-            // DEPTH rows in flight per thread (DEPTH * RP divides 512): the tile is NC * 4 bytes of
-            // each of N rows, from the L2
-            constexpr int DEPTH = 512u / RP;
-            static_assert(DEPTH >= 1 && DEPTH <= 16, "a round of DEPTH passes covers 512 rows");
-            for (uint32_t rb = r0; rb < N; rb += (uint32_t)DEPTH * RP) {
-                f32x4 v[DEPTH];
-#pragma unroll
-                for (int u = 0; u < DEPTH; ++u) {
-                    const uint32_t r = rb + (uint32_t)u * RP;
-                    v[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-                    const uint64_t at = (uint64_t)r * B + c4;
-                    if (vec_ok) {
-                        v[u] = *reinterpret_cast<const f32x4*>(X + at);
-                    } else if (any) {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (c4 + e < B) v[u][e] = X[at + e];
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < DEPTH; ++u) {
-                    const uint32_t r = rb + (uint32_t)u * RP;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) tile[(4u * q4 + e) * cstride + r] = v[u][e];
-                }
-            }
-        }
+        gemv::stage_column_tile<NC, WAVES>(X, tile, N, B, b0, lane, wave, gemv::first_row_of(blockIdx.x));
         start_block(m_first);
         lds_barrier();
-        // Wavefront w transforms columns w, w + 4, w + 8, ... of the tile, those that exist in X
-        // (a last or only column group may hold fewer than NC: with B = 8 every wavefront has two
-        // columns to do, not four for two of them and four columns of zeros for the others).  Its
-        // tiles (N / 512 per column) are taken in pairs whose MFMA chains interleave, the next
-        // pair's LDS reads and three-way splits sitting in the shadow of this pair's MFMAs (one
-        // wavefront per SIMD may be all there is); the tiles of a column are then joined by fp32
-        // butterflies in registers.  Columns past the end of X are left as they are: a column of
-        // the B operand reaches only its own column of the product, which is not stored.
-        TileOperands<BF16> ops;
-        make_tile_operands<BF16, 4>(9, ops);
-        auto transform_columns = [&](auto nt_tag) __attribute__((always_inline)) {
-            constexpr int NT = decltype(nt_tag)::value;  // tiles per column
-            constexpr int XB = NT == 4 ? 2 : (NT == 2 ? 1 : 0);
-            constexpr int HOLD = NT > 2 ? NT : 2;        // tiles of a unit: a column, or two of one tile
-            constexpr int UPAIRS = HOLD / 2;             // pairs of tiles per unit
-            const uint32_t ncols = min((uint32_t)NC, B - b0);
-            const uint32_t mine = ncols > wave ? (ncols - wave + WAVES - 1u) / WAVES : 0u;  // columns of this wavefront
-            const uint32_t units = NT == 1 ? (mine + 1u) / 2u : mine;
-            // tile t of unit u: NT > 1: tile t of the wavefront's u-th column; NT = 1: column 2u + t
-            auto at = [&](uint32_t u, int t) {
-                const uint32_t j = NT == 1 ? 2u * u + (uint32_t)t : u;
-                const uint32_t c = min(wave + (uint32_t)WAVES * j, (uint32_t)NC - 1u);  // (NT = 1, odd count: a spare column)
-                return tile + c * cstride + (NT == 1 ? 0u : 512u * (uint32_t)t);
-            };
-            auto fetch = [&](uint32_t u, int t, SplitTileF32& o) __attribute__((always_inline)) {
-                float in[8];
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const f32x4 q = *reinterpret_cast<const f32x4*>(at(u, t) + 256u * h + 4u * lane);
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) in[4 * h + r] = q[r];
-                }
-                split_tile_f32(in, o);
-            };
-            if (units == 0u) return;
-            SplitTileF32 cur[2], nxt[2];
-            fetch(0u, 0, cur[0]);
-            fetch(0u, 1, cur[1]);
-            auto unit = [&](uint32_t u, bool more) __attribute__((always_inline)) {
-                f32x4 held[HOLD][2];
-#pragma unroll
-                for (int q = 0; q < UPAIRS; ++q) {
-                    if (q + 1 < UPAIRS) {
-                        fetch(u, 2 * q + 2, nxt[0]);
-                        fetch(u, 2 * q + 3, nxt[1]);
-                    } else if (more) {
-                        fetch(u + 1u, 0, nxt[0]);
-                        fetch(u + 1u, 1, nxt[1]);
-                    }
-                    f32x4 a[2][2];
-                    tile_pair_mfma_f32(cur, ops, a);
-#pragma unroll
-                    for (int c = 0; c < 2; ++c)
-#pragma unroll
-                        for (int h = 0; h < 2; ++h) held[2 * q + c][h] = a[c][h];
-                    cur[0] = nxt[0];
-                    cur[1] = nxt[1];
-                }
-                if constexpr (NT > 1) cross_tile_butterflies<NT, XB>(held);
-#pragma unroll
-                for (int i = 0; i < HOLD; ++i)
-#pragma unroll
-                    for (int h = 0; h < 2; ++h)
-                        *reinterpret_cast<f32x4*>(at(u, i) + 256u * h + 4u * lane) = held[i][h] * scale;
-            };
-            // a full tile: the same number of units for every wavefront, one straight-line sequence
-            constexpr uint32_t FULL_UNITS = (NC / WAVES) / (NT == 1 ? 2 : 1);
-            if (ncols == (uint32_t)NC) {
-#pragma unroll
-                for (uint32_t u = 0; u < FULL_UNITS; ++u) unit(u, u + 1u < FULL_UNITS);
-            } else {
-                for (uint32_t u = 0; u < units; ++u) unit(u, u + 1u < units);
-            }
-        };
-        if (N == 512u)
-            transform_columns(std::integral_constant<int, 1>{});
-        else if (N == 1024u)
-            transform_columns(std::integral_constant<int, 2>{});
-        else
-            transform_columns(std::integral_constant<int, 4>{});
+        gemv::transform_column_tile<NC, WAVES>(tile, N, B, b0, scale, lane, wave);
         lds_barrier();
     } else {
         uint32_t done = 0;
@@ -515,28 +384,10 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
     }
 }
 
-// How the tiles of Y are spread: a workgroup keeps its transformed tile for several row blocks once
-// there are more row blocks than it takes to give every compute unit as many workgroups as fit its
-// LDS (two are counted on where they fit).
-struct GemvPlan {
-    uint32_t col_groups, rows_per_group, row_groups;
-    uint32_t workgroups() const { return col_groups * row_groups; }
-};
 inline size_t gemv_lds_bytes(uint32_t N, bool tiled, uint32_t nc, uint32_t mi, uint32_t waves)
 {
     const uint32_t frags = mi * (nc / 16u), phase = waves == 8u && frags > 4u ? 4u : frags;
     return (size_t)(N + (tiled ? kPad : 0u)) * nc * sizeof(float) + (size_t)(waves - 1u) * phase * 64u * sizeof(f32x4);
-}
-inline GemvPlan plan_gemv(uint32_t M, uint32_t B, uint32_t nc, uint32_t block_rows, size_t lds)
-{
-    GemvPlan p;
-    p.col_groups = (B + nc - 1u) / nc;
-    const uint32_t row_blocks = (M + block_rows - 1u) / block_rows;
-    uint32_t groups_y = ((lds <= 80u * 1024u ? 512u : 256u) + p.col_groups - 1u) / p.col_groups;
-    if (groups_y > row_blocks) groups_y = row_blocks;
-    p.rows_per_group = ((row_blocks + groups_y - 1u) / groups_y) * block_rows;
-    p.row_groups = (M + p.rows_per_group - 1u) / p.rows_per_group;
-    return p;
 }
 
 template <int MI, bool TILED, int NC, int PF = 4, int WAVES = 4>
@@ -599,6 +450,9 @@ extern "C" int mi_fused_ht_gemv(const void* W, const void* X, void* Y, uint32_t 
     if ((N == 512u || N == 1024u) && groups32x64 >= 256u)
         return launch_gemv_as<4, true, 32>(w, x, y, M, N, B, scale, s);
     const uint64_t groups64 = (uint64_t)((B + kCols - 1) / kCols) * ((M + 63u) / 64u);
+    // N = 2048 cannot have 32 columns in LDS: the kernel that holds the transformed columns in
+    // registers and streams W through the LDS in whole lines (fused_gemv_stream.hip)
+    if (N == 2048u && groups64 >= 256u) return gemv::launch_stream_2048(w, x, y, M, B, scale, s);
     if (groups64 >= 256u) return launch_gemv<4>(w, x, y, M, N, B, scale, s);
     if (groups64 < 128u) return launch_gemv<1>(w, x, y, M, N, B, scale, s);
     return launch_gemv<2>(w, x, y, M, N, B, scale, s);
