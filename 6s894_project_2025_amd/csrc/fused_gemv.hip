@@ -1,18 +1,15 @@
 // Fused Hadamard + GEMV-batch (mi_fused_ht_gemv), fp32, gfx950:
 //     Y[M,B] = W[M,N] * (scale * H_N * X[N,B]),  transform down dimension 0 of X.
 //
-// A workgroup owns 16 or 32 columns of X and 16, 32 or 64 rows of W at a time; it keeps its
-// transformed columns in LDS for several row blocks when there are more row blocks than compute
-// units to spread them over.
-//   prologue, N >= 512: the columns are brought into LDS column by column (TT[NC][N + 4]: a
-//              thread reads 16 contiguous bytes of a row of X and scatters them over four
-//              columns), transformed there by the exact fp32 tile transform on the matrix cores
-//              (fwht_device.hpp: 512-element tiles read and written back with 16-byte LDS accesses,
-//              taken in pairs whose MFMA chains interleave, the tiles of a column joined by fp32
-//              butterflies in registers; wavefront w takes columns (NC/4) w ..), and read by the
+// This file: the entry point, and the kernel for every shape but the large ones with N >= 512 (those
+// that give every compute unit a 64-row workgroup go to fused_gemv_stream.hip).  A workgroup owns
+// 16 columns of X and 16, 32 or 64 rows of W at a time; it keeps its transformed columns in LDS for
+// several row blocks when there are more row blocks than compute units to spread them over.
+//   prologue, N >= 512: gemv_common.hpp (the columns are brought into LDS column by column and
+//              transformed there by the exact fp32 tile transform on the matrix cores), read by the
 //              product as 16-byte B fragments.  N = 1024 measured 10.4 us per workgroup for the
 //              register-butterfly prologue below (every LDS access 4 bytes, 128 of them per thread
-//              and pass) against 4 us of loading and 6 us of transform for twice the columns here.
+//              and pass) against 4 us of loading and 6 us of transform for twice the columns there.
 //   prologue, N < 512: the 16 columns are brought into LDS as T[N][16] (a row is 64 bytes, so the 16
 //              column-lanes of a wavefront read global memory contiguously) while radix-16
 //              register butterflies run: each thread owns one column and 16 rows per step, so
@@ -24,12 +21,12 @@
 //              element is read once per workgroup instead of once per column.  The four wavefronts
 //              each take a quarter of the K steps with four steps of loads in flight, the B
 //              fragments of a step read one step early, and their partial sums are added through
-//              LDS.  With 32 columns (N = 512 and 1024, once that still gives every compute unit a
-//              workgroup) the K loop runs at 0.88 of the matrix cores' rate (18.5 thousand cycles
-//              for 512 MFMAs per wavefront); with 16 columns it is bound by the stream of W from
-//              the L2, which is why 32 are taken where the LDS holds them.
+//              LDS.  A load instruction of this form touches 16 rows of W and 64 bytes of each; the
+//              vector cache handles a request per 128-byte line however little of it is asked for,
+//              which bounds this loop at 16 - 17 bytes per clock and compute unit, half of what the
+//              matrix cores could take with 16 columns: fused_gemv_stream.hip is the answer to that.
 //   placement: workgroups are numbered so that the column groups sharing a slice of W run on one
-//              XCD (one L2).
+//              XCD (one L2), or the row groups sharing a column tile.
 //
 // Behaviour replaced: fused_hadamard_gemv_kernel(_vec), fused_ht/fwht_gemv_fusion.cu:98-244, where
 // every column's block re-reads all of W and reduces with warp shuffles.
@@ -131,20 +128,18 @@ __device__ __forceinline__ void pass_w(int wbits, const float* __restrict__ X, f
 // MI = 16-row blocks of W per workgroup (16, 32 or 64 rows).  The four wavefronts split the K range
 // of the product between them (every wavefront covers all MI row blocks over a quarter of N), so
 // each one streams a short, deeply prefetched run of W, and the partial sums meet in LDS.
-// WAVES = wavefronts per workgroup.  Every launch uses four: eight (two per SIMD, for the shapes
-// where a compute unit holds one workgroup anyway) measured no faster, since the transform of a
-// column costs a SIMD about 1 400 cycles of MFMA and vector issue whoever issues them (M = N = 1024:
-// B = 64 8.7 instead of 9.2 us, B = 8 8.9 instead of 8.5, B = 2048 59.7 instead of 52.7 with the
-// sums then going through LDS in two phases).
-template <int MI, bool TILED, int NC, int PF, int WAVES>
-__global__ void __launch_bounds__(64 * WAVES)
+// (Eight wavefronts per workgroup, two per SIMD, measured no faster where a compute unit holds one
+// workgroup anyway: the transform of a column costs a SIMD about 1 400 cycles of MFMA and vector
+// issue whoever issues them.  M = N = 1024: B = 64 8.7 instead of 9.2 us, B = 8 8.9 instead of 8.5.)
+template <int MI, bool TILED>
+__global__ void __launch_bounds__(kThreads)
 fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
                      float* __restrict__ Y, uint32_t M, uint32_t N, uint32_t B, uint32_t logN,
                      float scale, uint32_t rows_per_group, uint32_t col_groups, uint32_t row_groups,
                      uint32_t per_xcd, bool col_major)
 {
-    static_assert(NC == kCols || (TILED && NC == 2 * kCols), "wider tiles only in the column-major form");
-    static_assert(WAVES == kThreads / 64 || (TILED && WAVES == 8), "the register-butterfly prologue is written for 256 threads");
+    constexpr int NC = kCols, WAVES = kThreads / 64;
+    constexpr int PF = 4;        // K steps (of 16) in flight per wavefront
     constexpr int NF = NC / 16;  // 16-column fragments of the product per workgroup
     extern __shared__ __attribute__((aligned(16))) float tile[];  // [N][16] rows swizzled, then sums
     // Workgroups are handed to the eight XCDs in turn, each with an L2 of its own.  Position
@@ -166,10 +161,6 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
     const uint32_t m_first = (col_major ? place % row_groups : place / col_groups) * rows_per_group;
     const uint32_t m_last = min(M, m_first + rows_per_group);
 
-    // PF = K steps (of 16) in flight per wavefront: four, and eight for N = 2048, where a compute
-    // unit holds one workgroup (four wavefronts) whose 64 KB on the way at the latency of the L2
-    // left the K loop at half the rate of the matrix cores.  (The 32-column workgroups are bound by
-    // the matrix cores with four; eight measured slower, 40.7 -> 44.2 us for four row blocks.)
     const uint32_t total = N >> 4;
     const uint32_t quarter = (total + (uint32_t)WAVES - 1u) / (uint32_t)WAVES;  // a wavefront's share of the K steps
     const uint32_t k_begin = min(wave * quarter, total), k_end = min(k_begin + quarter, total);
@@ -344,40 +335,32 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
         // Fragment g is finished by wavefront g % WAVES, which keeps its own partial sum in
         // registers: only the others go through LDS (12 KB instead of 16 for 64 rows by 16 columns
         // and four wavefronts, which is what lets two such workgroups with N = 1024 share a compute
-        // unit).  With eight wavefronts the fragments go in phases of kPhaseFrags, so that the
-        // region stays within what the tile leaves of the LDS.  The sum is taken in the order of
-        // the wavefronts, whoever holds which part.
+        // unit).  The sum is taken in the order of the wavefronts, whoever holds which part.
         constexpr int G = MI * NF;
-        constexpr int kPhaseFrags = WAVES == 8 && G > 4 ? 4 : G;
         // D[m'][n']: n' = lo is the column, m' = 4*hi + r the row inside the 16-row block
+        lds_barrier();  // the sums of the row block before have been read
 #pragma unroll
-        for (int g0 = 0; g0 < G; g0 += kPhaseFrags) {
-            lds_barrier();  // the sums of the phase (or row block) before have been read
+        for (int g = 0; g < G; ++g) {
+            const uint32_t owner = (uint32_t)(g % WAVES);
+            if (wave != owner) red[((uint32_t)g * (WAVES - 1) + (wave < owner ? wave : wave - 1u)) * 64u + lane] = acc[g];
+        }
+        lds_barrier();
 #pragma unroll
-            for (int g = g0; g < g0 + kPhaseFrags; ++g) {
-                const uint32_t owner = (uint32_t)(g % WAVES);
-                if (wave != owner)
-                    red[((uint32_t)(g - g0) * (WAVES - 1) + (wave < owner ? wave : wave - 1u)) * 64u + lane] = acc[g];
+        for (int g = 0; g < G; ++g) {
+            const int owner = g % WAVES;
+            if (wave != (uint32_t)owner) continue;
+            f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) {
+                const f32x4 part = w == owner ? acc[g] : red[(g * (WAVES - 1) + (w < owner ? w : w - 1)) * 64 + lane];
+                sum = w == 0 ? part : sum + part;
             }
-            lds_barrier();
+            const uint32_t col = b0 + 16u * (uint32_t)(g % NF) + lo;
+            if (col < B) {
 #pragma unroll
-            for (int g = g0; g < g0 + kPhaseFrags; ++g) {
-                const int owner = g % WAVES;
-                if (wave != (uint32_t)owner) continue;
-                f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int w = 0; w < WAVES; ++w) {
-                    const f32x4 part =
-                        w == owner ? acc[g] : red[((g - g0) * (WAVES - 1) + (w < owner ? w : w - 1)) * 64 + lane];
-                    sum = w == 0 ? part : sum + part;
-                }
-                const uint32_t col = b0 + 16u * (uint32_t)(g % NF) + lo;
-                if (col < B) {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const uint32_t m = mb + 16u * (uint32_t)(g / NF) + 4u * hi + r;
-                        if (m < M) Y[(uint64_t)m * B + col] = sum[r];
-                    }
+                for (int r = 0; r < 4; ++r) {
+                    const uint32_t m = mb + 16u * (uint32_t)(g / NF) + 4u * hi + r;
+                    if (m < M) Y[(uint64_t)m * B + col] = sum[r];
                 }
             }
         }
@@ -386,18 +369,18 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
 
 inline size_t gemv_lds_bytes(uint32_t N, bool tiled, uint32_t nc, uint32_t mi, uint32_t waves)
 {
-    const uint32_t frags = mi * (nc / 16u), phase = waves == 8u && frags > 4u ? 4u : frags;
-    return (size_t)(N + (tiled ? kPad : 0u)) * nc * sizeof(float) + (size_t)(waves - 1u) * phase * 64u * sizeof(f32x4);
+    return (size_t)(N + (tiled ? kPad : 0u)) * nc * sizeof(float) + (size_t)(waves - 1u) * mi * (nc / 16u) * 64u * sizeof(f32x4);
 }
 
-template <int MI, bool TILED, int NC, int PF = 4, int WAVES = 4>
+template <int MI, bool TILED>
 int launch_gemv_as(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B,
                    float scale, hipStream_t s)
 {
+    constexpr uint32_t NC = kCols, WAVES = kThreads / 64;
     const size_t lds = gemv_lds_bytes(N, TILED, NC, MI, WAVES);
     // the tile transform's two MFMA stages attenuate by a power of two that the scale takes back
     if (TILED) scale = (float)((double)scale * (double)(1u << tile_stage_shift<4>(9u, false)));
-    auto kern = fused_ht_gemv_kernel<MI, TILED, NC, PF, WAVES>;
+    auto kern = fused_ht_gemv_kernel<MI, TILED>;
     if (lds > 64u * 1024u) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -417,12 +400,8 @@ template <int MI>
 int launch_gemv(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B,
                 float scale, hipStream_t s)
 {
-    if (N < 512u) return launch_gemv_as<MI, false, kCols>(W, X, Y, M, N, B, scale, s);
-    // N = 2048 with 64-row blocks: a deeper load ring (one workgroup per compute unit: the tile is
-    // 128 KB)
-    if constexpr (MI == 4)
-        if (N == 2048u) return launch_gemv_as<MI, true, kCols, 8>(W, X, Y, M, N, B, scale, s);
-    return launch_gemv_as<MI, true, kCols>(W, X, Y, M, N, B, scale, s);
+    if (N < 512u) return launch_gemv_as<MI, false>(W, X, Y, M, N, B, scale, s);
+    return launch_gemv_as<MI, true>(W, X, Y, M, N, B, scale, s);
 }
 
 }  // namespace
@@ -441,18 +420,19 @@ extern "C" int mi_fused_ht_gemv(const void* W, const void* X, void* Y, uint32_t 
     const float* w = static_cast<const float*>(W);
     const float* x = static_cast<const float*>(X);
     float* y = static_cast<float*>(Y);
-    // 64-row workgroups once that still gives every compute unit a workgroup; 32-row ones for
-    // small problems, where more (shorter) workgroups matter more than the repeated transform,
-    // and 16-row ones for the smallest (M = N = 1024, B <= 64: 12.2 -> 11.1 us)
-    // 32 columns per workgroup (W is read half as often, and every read of W comes from the L2)
-    // where the transformed tile still fits the LDS and every compute unit still gets a workgroup
+    // N >= 512 on shapes that give every compute unit a 64-row workgroup (of 32 columns; of 16 for
+    // N = 2048, whose transformed tile fills the LDS with 16): the kernel of fused_gemv_stream.hip,
+    // which holds the transformed columns in registers and streams W through the LDS in whole lines
+    // (measured against the 32-column, LDS-resident form of this file's kernel, which it replaced:
+    // (1024, 1024, 2048) 48.0 -> 44.3 us, (4096, 1024, 4096) 300 -> 269, (4096, 512, 4096) 171 -> 154,
+    // (512, 512, 1024) 12.0 -> 11.5; N = 2048 with 16 columns from LDS: (2048, 2048, 512) 73 -> 46)
     const uint64_t groups32x64 = (uint64_t)((B + 31u) / 32u) * ((M + 63u) / 64u);
-    if ((N == 512u || N == 1024u) && groups32x64 >= 256u)
-        return launch_gemv_as<4, true, 32>(w, x, y, M, N, B, scale, s);
+    if ((N == 512u || N == 1024u) && groups32x64 >= 256u) return gemv::launch_stream(w, x, y, M, N, B, scale, s);
+    // otherwise 64-row workgroups once that still gives every compute unit a workgroup; 32-row ones
+    // for small problems, where more (shorter) workgroups matter more than the repeated transform,
+    // and 16-row ones for the smallest (M = N = 1024, B <= 64: 12.2 -> 11.1 us)
     const uint64_t groups64 = (uint64_t)((B + kCols - 1) / kCols) * ((M + 63u) / 64u);
-    // N = 2048 cannot have 32 columns in LDS: the kernel that holds the transformed columns in
-    // registers and streams W through the LDS in whole lines (fused_gemv_stream.hip)
-    if (N == 2048u && groups64 >= 256u) return gemv::launch_stream_2048(w, x, y, M, B, scale, s);
+    if (N == 2048u && groups64 >= 256u) return gemv::launch_stream(w, x, y, M, N, B, scale, s);
     if (groups64 >= 256u) return launch_gemv<4>(w, x, y, M, N, B, scale, s);
     if (groups64 < 128u) return launch_gemv<1>(w, x, y, M, N, B, scale, s);
     return launch_gemv<2>(w, x, y, M, N, B, scale, s);

@@ -246,11 +246,11 @@ fused_ht_gemv_stream_kernel(const float* __restrict__ W, const float* __restrict
 
 namespace gemv {
 
-// N = 2048, launched by mi_fused_ht_gemv (fused_gemv.hip) for the shapes that give every compute
-// unit a 64-row, 16-column workgroup.
-int launch_stream_2048(const float* W, const float* X, float* Y, uint32_t M, uint32_t B, float scale, hipStream_t s)
+namespace {
+
+template <int N, int NC>
+int launch_stream_as(const float* W, const float* X, float* Y, uint32_t M, uint32_t B, float scale, hipStream_t s)
 {
-    constexpr int N = 2048, NC = 16;
     using Geo = StreamGeom<N, NC>;
     // the tile transform's two MFMA stages attenuate by a power of two that the scale takes back
     scale = (float)((double)scale * (double)(1u << tile_stage_shift<4>(9u, false)));
@@ -266,6 +266,19 @@ int launch_stream_2048(const float* W, const float* X, float* Y, uint32_t M, uin
     hipLaunchKernelGGL(kern, dim3(per_xcd * kXcds), dim3(64 * kWaves), Geo::kLdsBytes, s, W, X, Y, M, B, scale,
                        p.rows_per_group, p.col_groups, p.row_groups, per_xcd, col_major);
     return launch_status();
+}
+
+}  // namespace
+
+// Launched by mi_fused_ht_gemv (fused_gemv.hip) for the shapes that give every compute unit a 64-row
+// workgroup: N = 2048 with 16 columns per workgroup, N = 1024 with 32.
+int launch_stream(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B, float scale,
+                  hipStream_t s)
+{
+    if (N == 2048u) return launch_stream_as<2048, 16>(W, X, Y, M, B, scale, s);
+    if (N == 1024u) return launch_stream_as<1024, 32>(W, X, Y, M, B, scale, s);
+    if (N == 512u) return launch_stream_as<512, 32>(W, X, Y, M, B, scale, s);
+    return MI_ERR_SIZE;
 }
 
 }  // namespace gemv

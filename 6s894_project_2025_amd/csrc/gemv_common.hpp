@@ -199,9 +199,10 @@ inline GemvPlan plan_gemv(uint32_t M, uint32_t B, uint32_t nc, uint32_t block_ro
     return p;
 }
 
-// N = 2048 with W streamed through LDS and the transformed columns in registers
+// N = 1024 and 2048 with W streamed through LDS and the transformed columns in registers
 // (fused_gemv_stream.hip); same contract as the kernels of fused_gemv.hip.
-int launch_stream_2048(const float* W, const float* X, float* Y, uint32_t M, uint32_t B, float scale, hipStream_t s);
+int launch_stream(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B, float scale,
+                  hipStream_t s);
 
 }  // namespace gemv
 }  // namespace mi

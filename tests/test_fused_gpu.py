@@ -50,16 +50,22 @@ def test_gemv_reference_self_check(pkg, oracle, M, N, B):
 # fused_ht/fwht_gemv_fusion.cu:643-653) and a workgroup that walks several row blocks with one
 # transformed tile (more row blocks than workgroup rows in the grid).  (The 32-row variant runs
 # between 128 and 255 such groups: (1024, 1024, 128) here and (256, 256, 512) above; everything
-# smaller runs 16-row workgroups.)  N = 512 and 1024 switch to 32-column workgroups once those
-# still number 256: (1024, 1024, 512) with one row block each, (1024, 1024, 2048) with four (the
-# loads of the next block start in the last steps of the one before), (1000, 512, 700) with a
-# ragged last row block and a last column group of 28, (1100, 1024, 531) with a row length that
-# rules out 16-byte loads of X.  N = 2048 with 64-row workgroups has a deeper load ring:
-# (4100, 2048, 130) and (2048, 2048, 512) walk three and four row blocks with it.
+# smaller runs 16-row workgroups.)
+# N >= 512 on shapes with a 64-row workgroup for every compute unit run the kernel that keeps the
+# transformed columns in registers and streams W through LDS (32 columns per workgroup for N = 512
+# and 1024, 16 for N = 2048): (1024, 1024, 512) with one row block per workgroup (the stream ends
+# with its first block), (1024, 1024, 2048) and (2048, 2048, 512) with four (each block requests the
+# first stages of the next), (1000, 512, 700) with a ragged last row block and a last column group of
+# 28, (1100, 1024, 531) and (1100, 2048, 531) with a row length that rules out 16-byte loads of X,
+# (4100, 2048, 130) with a last column group of two and a last block of four rows, (300, 2048, 1024)
+# with more column groups than a round of workgroups, (20000, 2048, 24) and (8192, 512, 40) with long
+# walks over row blocks, (16384, 2048, 16) with one column group.
 @pytest.mark.parametrize("M,N,B", [(1024, 1024, 256), (1024, 1024, 512), (1024, 1024, 128),
                                    (4096, 256, 4096), (2000, 64, 1000), (4100, 2048, 130),
                                    (1024, 1024, 2048), (1000, 512, 700), (1100, 1024, 531),
-                                   (2048, 2048, 512)])
+                                   (2048, 2048, 512), (1100, 2048, 531), (300, 2048, 1024),
+                                   (20000, 2048, 24), (8192, 512, 40), (16384, 2048, 16),
+                                   (512, 512, 1024)])
 def test_gemv_large_launch_paths(pkg, oracle, M, N, B):
     W, X = oracle.inputs_gemv(M, N, B)
     Y = pkg.fused_ht_gemv(W.cuda(), X.cuda())
