@@ -42,6 +42,7 @@ PER_FILE_FLAGS = {
     "fused_gemm_xreg.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "fused_gemm_xreg_f32.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "fused_gemm_xreg_k2048.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "fused_gemv_rows.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
 }
 
 
@@ -57,7 +58,7 @@ PER_FILE_FLAGS = {
 # the allocator puts on a loop edge, say) would see the old value, where for its own MFMAs the
 # compiler inserts the wait states.  The build fails when anything but another MFMA reads an
 # assembly MFMA's destination within kResultWaitStates issue slots on any path.
-ISA_CHECKED = {"fused_gemm_xreg.hip", "fused_gemm_xreg_f32.hip", "fused_gemm_xreg_k2048.hip"}
+ISA_CHECKED = {"fused_gemm_xreg.hip", "fused_gemm_xreg_f32.hip", "fused_gemm_xreg_k2048.hip", "fused_gemv_rows.hip"}
 # Files whose MFMAs are the compiler's own but which use the direct global -> LDS transfers (M0 is
 # theirs alone) and wait for them by hand before ordinary LDS reads: the M0 and LDS-read checks only.
 TRANSFER_CHECKED = {"fused_gemv_stream.hip"}

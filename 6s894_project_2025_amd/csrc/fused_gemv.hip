@@ -420,19 +420,21 @@ extern "C" int mi_fused_ht_gemv(const void* W, const void* X, void* Y, uint32_t 
     const float* w = static_cast<const float*>(W);
     const float* x = static_cast<const float*>(X);
     float* y = static_cast<float*>(Y);
-    // N >= 512 on shapes that give every compute unit a 64-row workgroup (of 32 columns; of 16 for
-    // N = 2048, whose transformed tile fills the LDS with 16): the kernel of fused_gemv_stream.hip,
-    // which holds the transformed columns in registers and streams W through the LDS in whole lines
-    // (measured against the 32-column, LDS-resident form of this file's kernel, which it replaced:
-    // (1024, 1024, 2048) 48.0 -> 44.3 us, (4096, 1024, 4096) 300 -> 269, (4096, 512, 4096) 171 -> 154,
-    // (512, 512, 1024) 12.0 -> 11.5; N = 2048 with 16 columns from LDS: (2048, 2048, 512) 73 -> 46)
-    const uint64_t groups32x64 = (uint64_t)((B + 31u) / 32u) * ((M + 63u) / 64u);
-    if ((N == 512u || N == 1024u) && groups32x64 >= 256u) return gemv::launch_stream(w, x, y, M, N, B, scale, s);
+    // N >= 512 on shapes that give every compute unit a 64-row, 16-column workgroup: the kernels that
+    // hold the transformed columns in registers and stream W through the LDS in whole lines.
+    //   N = 512, 1024 (fused_gemv_rows.hip: every wavefront holds all of K, the wavefronts split the
+    //   rows): (1024, 1024, 256) 14.4 -> 11.7 us, (1024, 1024, 512) 19.1 -> 16.1, (1024, 1024, 2048)
+    //   48.0 -> 40.3, (4096, 1024, 4096) 300 -> 257, (512, 512, 1024) 11.6 -> 10.0, (4096, 512, 4096)
+    //   171 -> 139 against this file's kernel with 16 or 32 columns in LDS;
+    //   N = 2048 (fused_gemv_stream.hip: the wavefronts split K): (2048, 2048, 512) 73 -> 46.
+    const uint64_t groups64 = (uint64_t)((B + kCols - 1) / kCols) * ((M + 63u) / 64u);
+    if (groups64 >= 256u) {
+        if (N == 512u || N == 1024u) return gemv::launch_rows(w, x, y, M, N, B, scale, s);
+        if (N == 2048u) return gemv::launch_stream_2048(w, x, y, M, B, scale, s);
+    }
     // otherwise 64-row workgroups once that still gives every compute unit a workgroup; 32-row ones
     // for small problems, where more (shorter) workgroups matter more than the repeated transform,
     // and 16-row ones for the smallest (M = N = 1024, B <= 64: 12.2 -> 11.1 us)
-    const uint64_t groups64 = (uint64_t)((B + kCols - 1) / kCols) * ((M + 63u) / 64u);
-    if (N == 2048u && groups64 >= 256u) return gemv::launch_stream(w, x, y, M, N, B, scale, s);
     if (groups64 >= 256u) return launch_gemv<4>(w, x, y, M, N, B, scale, s);
     if (groups64 < 128u) return launch_gemv<1>(w, x, y, M, N, B, scale, s);
     return launch_gemv<2>(w, x, y, M, N, B, scale, s);

@@ -258,7 +258,7 @@ int launch_stream_as(const float* W, const float* X, float* Y, uint32_t M, uint3
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)Geo::kLdsBytes) != hipSuccess)
         return MI_ERR_LAUNCH;
-    const GemvPlan p = plan_gemv(M, B, NC, kBlockRows, Geo::kLdsBytes);
+    const GemvPlan p = plan_gemv_rounds(M, B, NC, kBlockRows);
     const uint32_t per_xcd = (p.workgroups() + kXcds - 1) / kXcds;
     // bytes of X an XCD needs under the row-group-major order: its column groups' tiles
     const uint64_t x_per_xcd = (uint64_t)(p.col_groups < per_xcd ? p.col_groups : per_xcd) * NC * N * sizeof(float);
@@ -270,15 +270,11 @@ int launch_stream_as(const float* W, const float* X, float* Y, uint32_t M, uint3
 
 }  // namespace
 
-// Launched by mi_fused_ht_gemv (fused_gemv.hip) for the shapes that give every compute unit a 64-row
-// workgroup: N = 2048 with 16 columns per workgroup, N = 1024 with 32.
-int launch_stream(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B, float scale,
-                  hipStream_t s)
+// Launched by mi_fused_ht_gemv (fused_gemv.hip) for N = 2048 on the shapes that give every compute
+// unit a 64-row workgroup.
+int launch_stream_2048(const float* W, const float* X, float* Y, uint32_t M, uint32_t B, float scale, hipStream_t s)
 {
-    if (N == 2048u) return launch_stream_as<2048, 16>(W, X, Y, M, B, scale, s);
-    if (N == 1024u) return launch_stream_as<1024, 32>(W, X, Y, M, B, scale, s);
-    if (N == 512u) return launch_stream_as<512, 32>(W, X, Y, M, B, scale, s);
-    return MI_ERR_SIZE;
+    return launch_stream_as<2048, 16>(W, X, Y, M, B, scale, s);
 }
 
 }  // namespace gemv

@@ -199,10 +199,42 @@ inline GemvPlan plan_gemv(uint32_t M, uint32_t B, uint32_t nc, uint32_t block_ro
     return p;
 }
 
-// N = 1024 and 2048 with W streamed through LDS and the transformed columns in registers
-// (fused_gemv_stream.hip); same contract as the kernels of fused_gemv.hip.
-int launch_stream(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B, float scale,
-                  hipStream_t s);
+// The same for a kernel of which a compute unit holds one workgroup (fused_gemv_stream.hip): the
+// launch runs in rounds of 256 workgroups, each costing one prologue plus a time per 64-row block
+// (measured about 12 us and 9 us: 4 : 3), so the number of row groups is the one that minimises
+// rounds x (prologue + row blocks per group).  33 column groups over 32 row blocks: seven row groups
+// of five blocks (231 workgroups, one round) instead of eight of four (264: a second round for eight
+// workgroups, 104 us instead of 60 for M = N = 2048, B = 528).
+inline GemvPlan plan_gemv_rounds(uint32_t M, uint32_t B, uint32_t nc, uint32_t block_rows)
+{
+    GemvPlan p;
+    p.col_groups = (B + nc - 1u) / nc;
+    const uint32_t row_blocks = (M + block_rows - 1u) / block_rows;
+    uint64_t best = ~0ull;
+    uint32_t best_per_group = row_blocks;
+    for (uint32_t per_group = 1; per_group <= row_blocks; ++per_group) {
+        const uint64_t groups = (row_blocks + per_group - 1u) / per_group;
+        const uint64_t rounds = (groups * p.col_groups + 255u) / 256u;
+        const uint64_t cost = rounds * (4u + 3ull * per_group);
+        if (cost < best) {
+            best = cost;
+            best_per_group = per_group;
+        }
+        if (rounds == 1u) break;  // longer groups only cost more from here on
+    }
+    p.rows_per_group = best_per_group * block_rows;
+    p.row_groups = (M + p.rows_per_group - 1u) / p.rows_per_group;
+    return p;
+}
+
+// N = 2048 with W streamed through LDS and each wavefront's quarter of the transformed columns in its
+// registers (fused_gemv_stream.hip); same contract as the kernels of fused_gemv.hip.
+int launch_stream_2048(const float* W, const float* X, float* Y, uint32_t M, uint32_t B, float scale, hipStream_t s);
+
+// N = 512 and 1024 with the whole B operand in every wavefront's registers, the wavefronts splitting
+// the rows (fused_gemv_rows.hip); same contract.
+int launch_rows(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B, float scale,
+                hipStream_t s);
 
 }  // namespace gemv
 }  // namespace mi

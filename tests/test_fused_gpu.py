@@ -51,21 +51,23 @@ def test_gemv_reference_self_check(pkg, oracle, M, N, B):
 # transformed tile (more row blocks than workgroup rows in the grid).  (The 32-row variant runs
 # between 128 and 255 such groups: (1024, 1024, 128) here and (256, 256, 512) above; everything
 # smaller runs 16-row workgroups.)
-# N >= 512 on shapes with a 64-row workgroup for every compute unit run the kernel that keeps the
-# transformed columns in registers and streams W through LDS (32 columns per workgroup for N = 512
-# and 1024, 16 for N = 2048): (1024, 1024, 512) with one row block per workgroup (the stream ends
-# with its first block), (1024, 1024, 2048) and (2048, 2048, 512) with four (each block requests the
-# first stages of the next), (1000, 512, 700) with a ragged last row block and a last column group of
-# 28, (1100, 1024, 531) and (1100, 2048, 531) with a row length that rules out 16-byte loads of X,
-# (4100, 2048, 130) with a last column group of two and a last block of four rows, (300, 2048, 1024)
-# with more column groups than a round of workgroups, (20000, 2048, 24) and (8192, 512, 40) with long
-# walks over row blocks, (16384, 2048, 16) with one column group.
+# N >= 512 on shapes with a 64-row, 16-column workgroup for every compute unit run the kernels that
+# keep the transformed columns in registers and stream W through LDS.  N = 512 and 1024 (every
+# wavefront all of K, 16 rows of a block each): (1024, 1024, 256) and (64, 1024, 4096) with one row
+# block per workgroup (the stream ends with its first block), (1024, 1024, 512), (1024, 1024, 2048)
+# and (512, 512, 1024) with two to eight (each block requests the first stages of the next),
+# (1000, 512, 700) with a ragged last row block and a last column group of 12, (1100, 1024, 531) with
+# a row length that rules out 16-byte loads of X, (4100, 1024, 130) with a last column group of two
+# and a last block of four rows, (8192, 512, 40) with a long walk over row blocks.  N = 2048 (the
+# wavefronts split K, sums meet in LDS): (2048, 2048, 512), (1100, 2048, 531), (4100, 2048, 130),
+# (300, 2048, 1024) with a second row block that is the last and ragged, (20000, 2048, 24) with three
+# blocks per workgroup, (16384, 2048, 16) with one column group.
 @pytest.mark.parametrize("M,N,B", [(1024, 1024, 256), (1024, 1024, 512), (1024, 1024, 128),
                                    (4096, 256, 4096), (2000, 64, 1000), (4100, 2048, 130),
                                    (1024, 1024, 2048), (1000, 512, 700), (1100, 1024, 531),
                                    (2048, 2048, 512), (1100, 2048, 531), (300, 2048, 1024),
                                    (20000, 2048, 24), (8192, 512, 40), (16384, 2048, 16),
-                                   (512, 512, 1024)])
+                                   (512, 512, 1024), (64, 1024, 4096), (4100, 1024, 130)])
 def test_gemv_large_launch_paths(pkg, oracle, M, N, B):
     W, X = oracle.inputs_gemv(M, N, B)
     Y = pkg.fused_ht_gemv(W.cuda(), X.cuda())
