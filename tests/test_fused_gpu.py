@@ -106,6 +106,32 @@ def test_gemv_random_shapes(pkg, oracle):
         assert _rel(oracle, Y, want) <= 1e-5, (M, N, B)
 
 
+def test_gemv_random_large_shapes(pkg, oracle):
+    # seeded sweep over the kernels that serve N >= 512 once column groups x 64-row blocks reach 256
+    # (rows split over the wavefronts for N = 512 and 1024, K split for N = 2048) and over the launch
+    # plan around that threshold: ragged row and column counts, one to many row blocks per workgroup,
+    # more column groups than one round of workgroups.  Checked on sampled rows and by column sums.
+    rng = np.random.default_rng(20251126)
+    g = torch.Generator().manual_seed(11)
+    for _ in range(24):
+        N = int(rng.choice([512, 1024, 2048]))
+        M = int(rng.choice([64, 65, 127, 200, 256, 300, 513, 1000, 1024, 1500, 2048, 3000, 5000]))
+        B = int(rng.choice([16, 17, 33, 64, 100, 255, 256, 260, 511, 528, 1000, 1024, 2049, 4100]))
+        if M * B > 6_000_000:
+            B = 528
+        W, X = oracle.inputs_gemv(M, N, B)
+        Y = pkg.fused_ht_gemv(W.cuda(), X.cuda())
+        torch.cuda.synchronize()
+        assert Y.shape == (M, B)
+        rows = torch.unique(torch.cat([torch.tensor([0, M // 2, M - 1]), torch.randint(0, M, (29,), generator=g)]))
+        want = oracle.fused_ht_gemv_f64_blas(W[rows].double().numpy(), X.double().numpy(), 1.0 / math.sqrt(N))
+        assert _rel(oracle, Y[rows.cuda()], want) <= 1e-5, (M, N, B)
+        colsum = oracle.fused_ht_gemv_f64_blas(W.double().sum(0, keepdim=True).numpy(), X.double().numpy(),
+                                               1.0 / math.sqrt(N))
+        got = Y.double().sum(0, keepdim=True).cpu().numpy()
+        assert np.abs(got - colsum).max() / np.abs(colsum).max() <= 1e-5, (M, N, B)
+
+
 def test_gemv_identity_reduces_to_transform(pkg, oracle):
     N, B = 256, 48
     _, X = oracle.inputs_gemv(N, N, B)
