@@ -17,6 +17,13 @@ namespace mi {
 int fused_gemm_f32_xreg(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, uint32_t K,
                         float scale, hipStream_t s);
 
+// The GEMV kernels (fused_gemv.hip and the files it names) on X given column by column: the same
+// product with 16 columns per workgroup.
+namespace gemv {
+int launch_any(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B, float scale,
+               bool columns_contiguous, hipStream_t s);
+}  // namespace gemv
+
 namespace {
 
 constexpr int kThreads = 512;
@@ -199,6 +206,28 @@ int launch(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, ui
 int fused_gemm_f32(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, uint32_t K,
                    float scale, hipStream_t s)
 {
+    // Small and medium outputs: the GEMV kernels, 16 columns per workgroup.  The GEMM kernels give a
+    // workgroup 64 columns or more (256 at K = 256), which pays once every workgroup walks many row
+    // blocks; below that their prologue and their few, long workgroups cost more than they save.
+    // Measured, GEMV route against GEMM kernel, us:
+    //   K = 64: 512^2 11.3 / 15.1, 2048^2 17.8 / 20.0;  K = 128: 1024^2 11.4 / 19.5, 2048^2 26.3 / 23.6;
+    //   K = 256: 512^2 11.7 / 29.9, 1024^2 16.1 / 30.5, 2048^2 46.5 / 31.9;
+    //   K = 512: 512^2 9.4 / 30.0, 1024^2 14.2 / 30.5, 2048^2 39.6 / 45.1, 3072^2 87.2 / 88.8, 4096^2 134.9 /
+    //   133.8, 8192 x 1024 71.9 / 74.8, 1024 x 8192 77.2 / 74.4;  K = 1024: 512^2 12.1 / 30.5, 1024^2 23.6 /
+    //   30.6, 2048^2 71.2 / 76.0, 3072^2 157.9 / 162.6, 4096^2 255.5 / 246.9;
+    //   K = 2048: 512^2 19.2 / 32.5, 1024^2 43.9 / 47.6, 2048^2 136.5 / 136.5, 4096^2 509 / 492.
+    {
+        const uint64_t groups = (uint64_t)((N + 15u) / 16u) * ((M + 63u) / 64u);  // >= 256: the large-shape GEMV kernels
+        const uint64_t outputs = (uint64_t)M * N;
+        bool by_gemv = false;
+        if (K <= 256u)
+            by_gemv = outputs <= 1536ull * 1024ull;
+        else if (K <= 1024u)
+            by_gemv = groups >= 256u && N <= 4096u && outputs <= 3072ull * 3072ull;
+        else if (K == 2048u)
+            by_gemv = groups >= 256u && N <= 4096u && outputs < 2048ull * 2048ull;
+        if (by_gemv) return gemv::launch_any(W, Xt, C, M, K, N, scale, true, s);
+    }
     switch (K) {
         case 32:
         case 64:

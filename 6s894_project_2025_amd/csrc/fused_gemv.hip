@@ -64,14 +64,16 @@ __device__ __forceinline__ void butterfly_regs(float (&v)[32])
         }
 }
 
-// One radix-2^WBITS pass over index bits [shift, shift + WBITS).  FROM_GLOBAL: read X, else LDS.
+// One radix-2^WBITS pass over index bits [shift, shift + WBITS).  FROM: 0 the LDS tile, 1 X[N][B] in
+// global memory, 2 X given column by column (Xt[B][N], the layout of mi_fused_ht_gemm).
 // Each thread owns one column and works on SETS butterfly sets at a time, all of their loads
 // issued before any arithmetic (the pass from global memory is latency-bound otherwise).
-template <int WBITS, bool FROM_GLOBAL>
+template <int WBITS, int FROM>
 __device__ __forceinline__ void pass(const float* __restrict__ X, float* tile, uint32_t N,
                                      uint32_t B, uint32_t b0, uint32_t shift, float mul)
 {
     constexpr int R = 1 << WBITS;
+    constexpr bool FROM_GLOBAL = FROM != 0;
     constexpr int SETS = (FROM_GLOBAL ? 4 : 2) / (WBITS == 5 ? 2 : 1);
     const uint32_t c = threadIdx.x & 15u, g = threadIdx.x >> 4;
     const uint32_t stride = 1u << shift;
@@ -89,8 +91,10 @@ __device__ __forceinline__ void pass(const float* __restrict__ X, float* tile, u
 #pragma unroll
                 for (int i = 0; i < R; ++i) {
                     const uint32_t r = base[u] + (uint32_t)i * stride;
-                    if (FROM_GLOBAL)
+                    if (FROM == 1)
                         v[u][i] = col_ok ? X[(uint64_t)r * B + b0 + c] : 0.0f;
+                    else if (FROM == 2)
+                        v[u][i] = col_ok ? X[(uint64_t)(b0 + c) * N + r] : 0.0f;
                     else
                         v[u][i] = tile[prow(r) * kCols + c];
                 }
@@ -111,17 +115,17 @@ __device__ __forceinline__ void pass(const float* __restrict__ X, float* tile, u
     }
 }
 
-template <bool FROM_GLOBAL>
+template <int FROM>
 __device__ __forceinline__ void pass_w(int wbits, const float* __restrict__ X, float* tile,
                                        uint32_t N, uint32_t B, uint32_t b0, uint32_t shift,
                                        float mul)
 {
     switch (wbits) {
-        case 1: pass<1, FROM_GLOBAL>(X, tile, N, B, b0, shift, mul); break;
-        case 2: pass<2, FROM_GLOBAL>(X, tile, N, B, b0, shift, mul); break;
-        case 3: pass<3, FROM_GLOBAL>(X, tile, N, B, b0, shift, mul); break;
-        case 4: pass<4, FROM_GLOBAL>(X, tile, N, B, b0, shift, mul); break;
-        default: pass<5, FROM_GLOBAL>(X, tile, N, B, b0, shift, mul); break;
+        case 1: pass<1, FROM>(X, tile, N, B, b0, shift, mul); break;
+        case 2: pass<2, FROM>(X, tile, N, B, b0, shift, mul); break;
+        case 3: pass<3, FROM>(X, tile, N, B, b0, shift, mul); break;
+        case 4: pass<4, FROM>(X, tile, N, B, b0, shift, mul); break;
+        default: pass<5, FROM>(X, tile, N, B, b0, shift, mul); break;
     }
 }
 
@@ -131,13 +135,15 @@ __device__ __forceinline__ void pass_w(int wbits, const float* __restrict__ X, f
 // (Eight wavefronts per workgroup, two per SIMD, measured no faster where a compute unit holds one
 // workgroup anyway: the transform of a column costs a SIMD about 1 400 cycles of MFMA and vector
 // issue whoever issues them.  M = N = 1024: B = 64 8.7 instead of 9.2 us, B = 8 8.9 instead of 8.5.)
-template <int MI, bool TILED>
+// XT: X is given column by column (Xt[B][N]); the register-butterfly prologue only.
+template <int MI, bool TILED, bool XT>
 __global__ void __launch_bounds__(kThreads)
 fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
                      float* __restrict__ Y, uint32_t M, uint32_t N, uint32_t B, uint32_t logN,
                      float scale, uint32_t rows_per_group, uint32_t col_groups, uint32_t row_groups,
                      uint32_t per_xcd, bool col_major)
 {
+    static_assert(!(TILED && XT), "the column-major staging reads X[N][B]");
     constexpr int NC = kCols, WAVES = kThreads / 64;
     constexpr int PF = 4;        // K steps (of 16) in flight per wavefront
     constexpr int NF = NC / 16;  // 16-column fragments of the product per workgroup
@@ -221,9 +227,9 @@ fused_ht_gemv_kernel(const float* __restrict__ W, const float* __restrict__ X,
             --passes_left;
             const float mul = (done + wbits == logN) ? scale : 1.0f;
             if (first)
-                pass_w<true>(wbits, X, tile, N, B, b0, done, mul);
+                pass_w<XT ? 2 : 1>(wbits, X, tile, N, B, b0, done, mul);
             else
-                pass_w<false>(wbits, X, tile, N, B, b0, done, mul);
+                pass_w<0>(wbits, X, tile, N, B, b0, done, mul);
             first = false;
             done += wbits;
             __syncthreads();
@@ -372,7 +378,7 @@ inline size_t gemv_lds_bytes(uint32_t N, bool tiled, uint32_t nc, uint32_t mi, u
     return (size_t)(N + (tiled ? kPad : 0u)) * nc * sizeof(float) + (size_t)(waves - 1u) * mi * (nc / 16u) * 64u * sizeof(f32x4);
 }
 
-template <int MI, bool TILED>
+template <int MI, bool TILED, bool XT>
 int launch_gemv_as(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B,
                    float scale, hipStream_t s)
 {
@@ -380,7 +386,7 @@ int launch_gemv_as(const float* W, const float* X, float* Y, uint32_t M, uint32_
     const size_t lds = gemv_lds_bytes(N, TILED, NC, MI, WAVES);
     // the tile transform's two MFMA stages attenuate by a power of two that the scale takes back
     if (TILED) scale = (float)((double)scale * (double)(1u << tile_stage_shift<4>(9u, false)));
-    auto kern = fused_ht_gemv_kernel<MI, TILED>;
+    auto kern = fused_ht_gemv_kernel<MI, TILED, XT>;
     if (lds > 64u * 1024u) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -398,13 +404,45 @@ int launch_gemv_as(const float* W, const float* X, float* Y, uint32_t M, uint32_
 
 template <int MI>
 int launch_gemv(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B,
-                float scale, hipStream_t s)
+                float scale, bool xt, hipStream_t s)
 {
-    if (N < 512u) return launch_gemv_as<MI, false>(W, X, Y, M, N, B, scale, s);
-    return launch_gemv_as<MI, true>(W, X, Y, M, N, B, scale, s);
+    if (N < 512u)
+        return xt ? launch_gemv_as<MI, false, true>(W, X, Y, M, N, B, scale, s)
+                  : launch_gemv_as<MI, false, false>(W, X, Y, M, N, B, scale, s);
+    if (xt) return MI_ERR_SIZE;  // (no caller: mi_fused_ht_gemm sends N >= 512 here only on large shapes)
+    return launch_gemv_as<MI, true, false>(W, X, Y, M, N, B, scale, s);
 }
 
 }  // namespace
+
+namespace gemv {
+
+// The kernel for a shape; arguments already validated.  `columns_contiguous`: X is given as Xt[B][N]
+// (mi_fused_ht_gemm's layout) instead of X[N][B].
+int launch_any(const float* w, const float* x, float* y, uint32_t M, uint32_t N, uint32_t B, float scale,
+               bool columns_contiguous, hipStream_t s)
+{
+    // N >= 512 on shapes that give every compute unit a 64-row, 16-column workgroup: the kernels that
+    // hold the transformed columns in registers and stream W through the LDS in whole lines.
+    //   N = 512, 1024 (fused_gemv_rows.hip: every wavefront holds all of K, the wavefronts split the
+    //   rows): (1024, 1024, 256) 14.4 -> 11.7 us, (1024, 1024, 512) 19.1 -> 16.1, (1024, 1024, 2048)
+    //   48.0 -> 40.3, (4096, 1024, 4096) 300 -> 257, (512, 512, 1024) 11.6 -> 10.0, (4096, 512, 4096)
+    //   171 -> 139 against this file's kernel with 16 or 32 columns in LDS;
+    //   N = 2048 (fused_gemv_stream.hip: the wavefronts split K): (2048, 2048, 512) 73 -> 46.
+    const uint64_t groups64 = (uint64_t)((B + kCols - 1) / kCols) * ((M + 63u) / 64u);
+    if (groups64 >= 256u) {
+        if (N == 512u || N == 1024u) return launch_rows(w, x, y, M, N, B, scale, columns_contiguous, s);
+        if (N == 2048u) return launch_stream_2048(w, x, y, M, B, scale, columns_contiguous, s);
+    }
+    // otherwise 64-row workgroups once that still gives every compute unit a workgroup; 32-row ones
+    // for small problems, where more (shorter) workgroups matter more than the repeated transform,
+    // and 16-row ones for the smallest (M = N = 1024, B <= 64: 12.2 -> 11.1 us)
+    if (groups64 >= 256u) return launch_gemv<4>(w, x, y, M, N, B, scale, columns_contiguous, s);
+    if (groups64 < 128u) return launch_gemv<1>(w, x, y, M, N, B, scale, columns_contiguous, s);
+    return launch_gemv<2>(w, x, y, M, N, B, scale, columns_contiguous, s);
+}
+
+}  // namespace gemv
 }  // namespace mi
 
 extern "C" int mi_fused_ht_gemv(const void* W, const void* X, void* Y, uint32_t M, uint32_t N,
@@ -420,22 +458,5 @@ extern "C" int mi_fused_ht_gemv(const void* W, const void* X, void* Y, uint32_t 
     const float* w = static_cast<const float*>(W);
     const float* x = static_cast<const float*>(X);
     float* y = static_cast<float*>(Y);
-    // N >= 512 on shapes that give every compute unit a 64-row, 16-column workgroup: the kernels that
-    // hold the transformed columns in registers and stream W through the LDS in whole lines.
-    //   N = 512, 1024 (fused_gemv_rows.hip: every wavefront holds all of K, the wavefronts split the
-    //   rows): (1024, 1024, 256) 14.4 -> 11.7 us, (1024, 1024, 512) 19.1 -> 16.1, (1024, 1024, 2048)
-    //   48.0 -> 40.3, (4096, 1024, 4096) 300 -> 257, (512, 512, 1024) 11.6 -> 10.0, (4096, 512, 4096)
-    //   171 -> 139 against this file's kernel with 16 or 32 columns in LDS;
-    //   N = 2048 (fused_gemv_stream.hip: the wavefronts split K): (2048, 2048, 512) 73 -> 46.
-    const uint64_t groups64 = (uint64_t)((B + kCols - 1) / kCols) * ((M + 63u) / 64u);
-    if (groups64 >= 256u) {
-        if (N == 512u || N == 1024u) return gemv::launch_rows(w, x, y, M, N, B, scale, s);
-        if (N == 2048u) return gemv::launch_stream_2048(w, x, y, M, B, scale, s);
-    }
-    // otherwise 64-row workgroups once that still gives every compute unit a workgroup; 32-row ones
-    // for small problems, where more (shorter) workgroups matter more than the repeated transform,
-    // and 16-row ones for the smallest (M = N = 1024, B <= 64: 12.2 -> 11.1 us)
-    if (groups64 >= 256u) return launch_gemv<4>(w, x, y, M, N, B, scale, s);
-    if (groups64 < 128u) return launch_gemv<1>(w, x, y, M, N, B, scale, s);
-    return launch_gemv<2>(w, x, y, M, N, B, scale, s);
+    return gemv::launch_any(w, x, y, M, N, B, scale, false, s);
 }

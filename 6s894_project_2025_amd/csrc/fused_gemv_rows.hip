@@ -88,7 +88,8 @@ struct RowsGeom {
     static_assert(STEPS * NF * 4 <= 256, "the B operand of a wavefront fits its registers");
 };
 
-template <int N, int NC>
+// XT: X is given column by column (Xt[B][N]).
+template <int N, int NC, bool XT>
 __global__ void __launch_bounds__(64 * kWaves)
 fused_ht_gemv_rows_kernel(const float* __restrict__ W, const float* __restrict__ X, float* __restrict__ Y,
                           uint32_t M, uint32_t B, float scale, uint32_t rows_per_group, uint32_t col_groups,
@@ -139,8 +140,11 @@ fused_ht_gemv_rows_kernel(const float* __restrict__ W, const float* __restrict__
 
     // ---- prologue: TT = scale * H_N * X[:, b0 .. b0 + NC - 1] in LDS ------------------------------
     // (all N rows of the tile requested before the first is waited for)
-    gemv::stage_column_tile<NC, kWaves, N / (16 * kWaves / (NC / 16))>(X, tile, N, B, b0, lane, wave,
-                                                                      gemv::first_row_of(blockIdx.x));
+    if constexpr (XT)
+        gemv::stage_column_tile_xt<NC, kWaves, N>(X, tile, B, b0, threadIdx.x);
+    else
+        gemv::stage_column_tile<NC, kWaves, N / (16 * kWaves / (NC / 16))>(X, tile, N, B, b0, lane, wave,
+                                                                          gemv::first_row_of(blockIdx.x));
     lds_barrier();
     gemv::transform_column_tile<NC, kWaves>(tile, N, B, b0, scale, lane, wave);
     lds_barrier();
@@ -267,13 +271,13 @@ fused_ht_gemv_rows_kernel(const float* __restrict__ W, const float* __restrict__
     }
 }
 
-template <int N, int NC>
+template <int N, int NC, bool XT>
 int launch_rows_as(const float* W, const float* X, float* Y, uint32_t M, uint32_t B, float scale, hipStream_t s)
 {
     using Geo = RowsGeom<N, NC>;
     // the tile transform's two MFMA stages attenuate by a power of two that the scale takes back
     scale = (float)((double)scale * (double)(1u << tile_stage_shift<4>(9u, false)));
-    auto kern = fused_ht_gemv_rows_kernel<N, NC>;
+    auto kern = fused_ht_gemv_rows_kernel<N, NC, XT>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)Geo::kLdsBytes) != hipSuccess)
         return MI_ERR_LAUNCH;
@@ -292,10 +296,14 @@ int launch_rows_as(const float* W, const float* X, float* Y, uint32_t M, uint32_
 namespace gemv {
 
 int launch_rows(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B, float scale,
-                hipStream_t s)
+                bool columns_contiguous, hipStream_t s)
 {
-    if (N == 1024u) return launch_rows_as<1024, 16>(W, X, Y, M, B, scale, s);
-    if (N == 512u) return launch_rows_as<512, 16>(W, X, Y, M, B, scale, s);
+    if (N == 1024u)
+        return columns_contiguous ? launch_rows_as<1024, 16, true>(W, X, Y, M, B, scale, s)
+                                  : launch_rows_as<1024, 16, false>(W, X, Y, M, B, scale, s);
+    if (N == 512u)
+        return columns_contiguous ? launch_rows_as<512, 16, true>(W, X, Y, M, B, scale, s)
+                                  : launch_rows_as<512, 16, false>(W, X, Y, M, B, scale, s);
     return MI_ERR_SIZE;
 }
 

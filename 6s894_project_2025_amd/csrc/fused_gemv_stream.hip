@@ -74,7 +74,8 @@ struct StreamGeom {
     static_assert(STEPS * NF * 4 <= 256, "the B fragments of a wavefront fit its registers");
 };
 
-template <int N, int NC>
+// XT: X is given column by column (Xt[B][N]).
+template <int N, int NC, bool XT>
 __global__ void __launch_bounds__(64 * kWaves)
 fused_ht_gemv_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, float* __restrict__ Y,
                             uint32_t M, uint32_t B, float scale, uint32_t rows_per_group, uint32_t col_groups,
@@ -97,7 +98,11 @@ fused_ht_gemv_stream_kernel(const float* __restrict__ W, const float* __restrict
     // ---- prologue: TT = scale * H_N * X[:, b0 .. b0 + NC - 1] in LDS ------------------------------
     // (all N rows of the tile requested before the first is waited for: 128 registers per lane that
     // nothing else needs yet)
-    gemv::stage_column_tile<NC, kWaves, N / (16 * kWaves / (NC / 16))>(X, tile, N, B, b0, lane, wave, gemv::first_row_of(blockIdx.x));
+    if constexpr (XT)
+        gemv::stage_column_tile_xt<NC, kWaves, N>(X, tile, B, b0, threadIdx.x);
+    else
+        gemv::stage_column_tile<NC, kWaves, N / (16 * kWaves / (NC / 16))>(X, tile, N, B, b0, lane, wave,
+                                                                          gemv::first_row_of(blockIdx.x));
     lds_barrier();
     gemv::transform_column_tile<NC, kWaves>(tile, N, B, b0, scale, lane, wave);
     lds_barrier();
@@ -248,13 +253,13 @@ namespace gemv {
 
 namespace {
 
-template <int N, int NC>
+template <int N, int NC, bool XT>
 int launch_stream_as(const float* W, const float* X, float* Y, uint32_t M, uint32_t B, float scale, hipStream_t s)
 {
     using Geo = StreamGeom<N, NC>;
     // the tile transform's two MFMA stages attenuate by a power of two that the scale takes back
     scale = (float)((double)scale * (double)(1u << tile_stage_shift<4>(9u, false)));
-    auto kern = fused_ht_gemv_stream_kernel<N, NC>;
+    auto kern = fused_ht_gemv_stream_kernel<N, NC, XT>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)Geo::kLdsBytes) != hipSuccess)
         return MI_ERR_LAUNCH;
@@ -272,9 +277,11 @@ int launch_stream_as(const float* W, const float* X, float* Y, uint32_t M, uint3
 
 // Launched by mi_fused_ht_gemv (fused_gemv.hip) for N = 2048 on the shapes that give every compute
 // unit a 64-row workgroup.
-int launch_stream_2048(const float* W, const float* X, float* Y, uint32_t M, uint32_t B, float scale, hipStream_t s)
+int launch_stream_2048(const float* W, const float* X, float* Y, uint32_t M, uint32_t B, float scale,
+                       bool columns_contiguous, hipStream_t s)
 {
-    return launch_stream_as<2048, 16>(W, X, Y, M, B, scale, s);
+    return columns_contiguous ? launch_stream_as<2048, 16, true>(W, X, Y, M, B, scale, s)
+                              : launch_stream_as<2048, 16, false>(W, X, Y, M, B, scale, s);
 }
 
 }  // namespace gemv

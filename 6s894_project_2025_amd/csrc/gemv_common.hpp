@@ -88,6 +88,29 @@ __device__ __forceinline__ void stage_column_tile(const float* __restrict__ X, f
     }
 }
 
+// The same tile from X given column by column (Xt[B][N], each column of X contiguous: the layout of
+// mi_fused_ht_gemm): a straight copy, 16 bytes per thread and access, every load of the tile in
+// flight at once.  Columns past the end of X are filled with zeros.
+template <int NC, int WAVES, int N>
+__device__ __forceinline__ void stage_column_tile_xt(const float* __restrict__ Xt, float* tile, uint32_t B, uint32_t b0,
+                                                     uint32_t tid)
+{
+    constexpr uint32_t cstride = N + kPad, kPerColumn = N / 4u;     // 16-byte chunks per column
+    constexpr int PER_THREAD = NC * (int)kPerColumn / (64 * WAVES);  // chunks per thread
+    static_assert(PER_THREAD >= 1 && PER_THREAD <= 32 && NC * kPerColumn % (64u * WAVES) == 0u, "whole rounds of the workgroup");
+    f32x4 v[PER_THREAD];
+#pragma unroll
+    for (int u = 0; u < PER_THREAD; ++u) {
+        const uint32_t at = tid + (uint32_t)u * 64u * WAVES, c = at / kPerColumn, q = at % kPerColumn;
+        v[u] = b0 + c < B ? *reinterpret_cast<const f32x4*>(Xt + ((uint64_t)(b0 + c) * N + 4u * q)) : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int u = 0; u < PER_THREAD; ++u) {
+        const uint32_t at = tid + (uint32_t)u * 64u * WAVES, c = at / kPerColumn, q = at % kPerColumn;
+        *reinterpret_cast<f32x4*>(tile + c * cstride + 4u * q) = v[u];
+    }
+}
+
 // Wavefront w transforms columns w, w + WAVES, w + 2 WAVES, ... of the tile, those that exist in X
 // (a last or only column group may hold fewer than NC: with B = 8 every wavefront has two columns
 // to do, not four for two of them and four columns of zeros for the others).  Its tiles (NT = N /
@@ -229,12 +252,19 @@ inline GemvPlan plan_gemv_rounds(uint32_t M, uint32_t B, uint32_t nc, uint32_t b
 
 // N = 2048 with W streamed through LDS and each wavefront's quarter of the transformed columns in its
 // registers (fused_gemv_stream.hip); same contract as the kernels of fused_gemv.hip.
-int launch_stream_2048(const float* W, const float* X, float* Y, uint32_t M, uint32_t B, float scale, hipStream_t s);
+// `columns_contiguous`: X is given as Xt[B][N] (the layout of mi_fused_ht_gemm) instead of X[N][B].
+int launch_stream_2048(const float* W, const float* X, float* Y, uint32_t M, uint32_t B, float scale,
+                       bool columns_contiguous, hipStream_t s);
 
 // N = 512 and 1024 with the whole B operand in every wavefront's registers, the wavefronts splitting
 // the rows (fused_gemv_rows.hip); same contract.
 int launch_rows(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B, float scale,
-                hipStream_t s);
+                bool columns_contiguous, hipStream_t s);
+
+// The GEMV kernel for a shape (fused_gemv.hip), arguments already validated; `columns_contiguous` as
+// above (supported for N < 512 and for the shapes the two kernels above take).
+int launch_any(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B, float scale,
+               bool columns_contiguous, hipStream_t s);
 
 }  // namespace gemv
 }  // namespace mi

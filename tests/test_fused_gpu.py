@@ -304,6 +304,58 @@ def test_gemm_f32_xreg_launch_plans(pkg, oracle, M, N, K):
     assert _rel(oracle, C[idx], want) <= 1e-5
 
 
+# fp32, K = 512 ... 2048 on small and medium outputs (at least 256 pairs of 16 columns x 64 rows, N <=
+# 4096, up to 3072^2 outputs, below 2048^2 for K = 2048) runs the GEMV kernels on X given column by
+# column: ragged rows and columns, one to many row blocks per workgroup, the shapes just inside and
+# just outside the route's limits.
+@pytest.mark.parametrize("K", [1024, 512, 2048])
+@pytest.mark.parametrize("M,N", [(512, 512), (1024, 1024), (700, 1023), (4100, 130), (64, 4096), (2047, 2048),
+                                 (3072, 3072), (8192, 1024), (1000, 4100)])
+def test_gemm_f32_through_gemv_kernels(pkg, oracle, M, N, K):
+    g = torch.Generator(device="cuda").manual_seed(M + N + K)
+    Wd = torch.randn(M, K, generator=g, device="cuda")
+    Xd = torch.randn(N, K, generator=g, device="cuda")
+    Y = pkg.hadamard_transform(Xd, 1.0 / 32.0)
+    for _ in range(2):
+        C = pkg.fused_ht_gemm(Wd, Xd, 1.0 / 32.0)
+    torch.cuda.synchronize()
+    assert C.shape == (M, N) and torch.isfinite(C).all()
+    worst = 0.0
+    for r0 in range(0, M, 1024):                             # fp64 product in slices (memory)
+        ref = Wd[r0:r0 + 1024].double() @ Y.double().t()
+        worst = max(worst, (C[r0:r0 + 1024].double() - ref).abs().max().item())
+    assert worst / (K / 32.0) <= 1e-5, worst
+    idx = torch.unique(torch.tensor([0, 63, 64, M // 2, M - 1]).clamp(0, M - 1))   # (M = 64 has no row 64)
+    want = oracle.fused_ht_gemm_f64_blas(Wd[idx].cpu().double().numpy(), Xd.cpu().double().numpy(), 1.0 / 32.0)
+    assert _rel(oracle, C[idx], want) <= 1e-5
+
+
+# fp32, K <= 256: outputs up to 1536 x 1024 run the GEMV kernel (register-butterfly prologue reading
+# X column by column), larger ones the GEMM kernels (LDS tile for K <= 128, register-resident for
+# K = 256).  Shapes on both sides of the limit, ragged in both directions, and the smallest.
+@pytest.mark.parametrize("K", [32, 64, 128, 256])
+@pytest.mark.parametrize("M,N", [(1, 1), (33, 7), (512, 512), (700, 1023), (1024, 1536), (1025, 1536), (2048, 1024),
+                                 (130, 4100)])
+def test_gemm_f32_small_k_both_routes(pkg, oracle, M, N, K):
+    g = torch.Generator(device="cuda").manual_seed(M + N + K)
+    Wd = torch.randn(M, K, generator=g, device="cuda")
+    Xd = torch.randn(N, K, generator=g, device="cuda")
+    scale = 1.0 / math.sqrt(K)
+    Y = pkg.hadamard_transform(Xd, scale)
+    for _ in range(2):
+        C = pkg.fused_ht_gemm(Wd, Xd, scale)
+    torch.cuda.synchronize()
+    assert C.shape == (M, N) and torch.isfinite(C).all()
+    ref = Wd.double() @ Y.double().t()
+    assert (C.double() - ref).abs().max().item() / math.sqrt(K) <= 1e-5
+    idx = torch.unique(torch.tensor([0, 63, 64, M // 2, M - 1]).clamp(0, M - 1))
+    want = oracle.fused_ht_gemm_f64_blas(Wd[idx].cpu().double().numpy(), Xd.cpu().double().numpy(), scale)
+    # against the typical magnitude of an output (sqrt(K) for these inputs), not the largest of a
+    # handful that may all be sums that nearly cancel (M = N = 1)
+    err = np.abs(C[idx].cpu().double().numpy() - want).max() / max(np.abs(want).max(), math.sqrt(K))
+    assert err <= 1e-5, err
+
+
 def test_gemm_small_bruteforce(pkg, oracle):
     # triple-loop oracle (no BLAS), fp32
     M, N, K = 16, 20, 64
