@@ -132,6 +132,30 @@ def test_gemv_random_large_shapes(pkg, oracle):
         assert np.abs(got - colsum).max() / np.abs(colsum).max() <= 1e-5, (M, N, B)
 
 
+@pytest.mark.parametrize("M,N", [(1_100_000, 1024), (550_000, 2048)])
+def test_gemv_w_beyond_4_gib(pkg, oracle, M, N):
+    # W of 4.5 GB: byte offsets into W pass 2^32 (the streaming kernels address a row block with a
+    # 64-bit base and 32-bit offsets inside it); rows on both sides of the 4 GiB line and the last ones
+    B = 16
+    g = torch.Generator(device="cuda").manual_seed(3)
+    W = torch.randn(M, N, generator=g, device="cuda")
+    X = torch.randn(N, B, generator=g, device="cuda")
+    Y = pkg.fused_ht_gemv(W, X)
+    torch.cuda.synchronize()
+    line = (1 << 32) // (4 * N)                      # the first row that starts at or beyond 4 GiB
+    rows = torch.tensor([0, 1, 63, 64, line - 65, line - 1, line, line + 1, line + 64, M - 65, M - 64, M - 1])
+    want = oracle.fused_ht_gemv_f64_blas(W[rows.cuda()].cpu().double().numpy(), X.cpu().double().numpy(),
+                                         1.0 / math.sqrt(N))
+    assert _rel(oracle, Y[rows.cuda()], want) <= 1e-5
+    # every row: Y against the product with the library's own transform, in slices
+    T = pkg.hadamard_transform(X.t().contiguous()).t().contiguous()
+    worst = 0.0
+    for r0 in range(0, M, 200_000):
+        ref = W[r0:r0 + 200_000] @ T
+        worst = max(worst, (Y[r0:r0 + 200_000] - ref).abs().max().item())
+    assert worst / math.sqrt(N) <= 1e-4, worst          # (fp32 against fp32: summation orders differ)
+
+
 def test_gemv_identity_reduces_to_transform(pkg, oracle):
     N, B = 256, 48
     _, X = oracle.inputs_gemv(N, N, B)
