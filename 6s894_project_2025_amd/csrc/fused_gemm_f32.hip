@@ -1,6 +1,6 @@
 // fp32 variant of the fused Hadamard -> GEMM for short transforms, K = 32, 64, 128 (see
-// fused_gemm.hip for the structure; K >= 256 runs the register-resident kernels of
-// fused_gemm_xreg_f32.hip).
+// fused_gemm.hip for the structure; K = 256 runs the GEMV kernels, K >= 512 those or the
+// register-resident kernels of fused_gemm_xreg_f32.hip: see fused_gemm_f32 below).
 //
 // The transformed tile Y[BN][K] is kept in LDS as fp32; the prologue runs the fp32 transform on
 // the bf16 matrix cores with exact three-piece operands (tile_transform_f32), and the
@@ -13,7 +13,7 @@
 
 namespace mi {
 
-// K = 256 ... 4096 with the transformed operand in registers: fused_gemm_xreg_f32.hip
+// K = 512 ... 4096 with the transformed operand in registers: fused_gemm_xreg_f32.hip
 int fused_gemm_f32_xreg(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, uint32_t K,
                         float scale, hipStream_t s);
 
@@ -211,7 +211,8 @@ int fused_gemm_f32(const float* W, const float* Xt, float* C, uint32_t M, uint32
     // blocks; below that their prologue and their few, long workgroups cost more than they save.
     // Measured, GEMV route against GEMM kernel, us:
     //   K = 64: 512^2 11.3 / 15.1, 2048^2 17.8 / 20.0;  K = 128: 1024^2 11.4 / 19.5, 2048^2 26.3 / 23.6;
-    //   K = 256: 512^2 11.7 / 29.9, 1024^2 16.1 / 30.5, 2048^2 46.5 / 31.9;
+    //   K = 256 (64 columns per workgroup from 128 pairs of 64 columns x 64 rows on): 512^2 11.7 / 29.9,
+    //   1024^2 11.3 / 30.5, 2048^2 24.7 / 31.9, 4096^2 72.0 / 79.7, 8192^2 255.8 / 258.0: every shape;
     //   K = 512: 512^2 9.4 / 30.0, 1024^2 14.2 / 30.5, 2048^2 39.6 / 45.1, 3072^2 87.2 / 88.8, 4096^2 134.9 /
     //   133.8, 8192 x 1024 71.9 / 74.8, 1024 x 8192 77.2 / 74.4;  K = 1024: 512^2 12.1 / 30.5, 1024^2 23.6 /
     //   30.6, 2048^2 71.2 / 76.0, 3072^2 157.9 / 162.6, 4096^2 255.5 / 246.9;
@@ -220,7 +221,9 @@ int fused_gemm_f32(const float* W, const float* Xt, float* C, uint32_t M, uint32
         const uint64_t groups = (uint64_t)((N + 15u) / 16u) * ((M + 63u) / 64u);  // >= 256: the large-shape GEMV kernels
         const uint64_t outputs = (uint64_t)M * N;
         bool by_gemv = false;
-        if (K <= 256u)
+        if (K == 256u)
+            by_gemv = true;
+        else if (K < 256u)
             by_gemv = outputs <= 1536ull * 1024ull;
         else if (K <= 1024u)
             by_gemv = groups >= 256u && N <= 4096u && outputs <= 3072ull * 3072ull;
@@ -232,7 +235,6 @@ int fused_gemm_f32(const float* W, const float* Xt, float* C, uint32_t M, uint32
         case 32:
         case 64:
         case 128: return launch<32>(W, Xt, C, M, N, K, scale, s);
-        case 256:
         case 512:
         case 1024:
         case 2048:

@@ -1,6 +1,7 @@
 // Fused Hadamard -> GEMM in fp32 (the reference's precision) with the transformed operand held in
 // registers, gfx950:
-//     C[M,N] = W[M,K] * (scale * H_K * X[K,N]),  X given as Xt[N,K],  K = 1024, fp32 in and out.
+//     C[M,N] = W[M,K] * (scale * H_K * X[K,N]),  X given as Xt[N,K],  K = 512 ... 4096, fp32 in and out
+// (described for K = 1024).
 //
 // Same structure as the 16-bit kernel of fused_gemm_xreg.hip (one wavefront per SIMD, W streamed
 // global -> LDS directly through a ring of four 32 KB stages, fragments broadcast to the four
@@ -37,7 +38,9 @@ __device__ __forceinline__ void xmfma_f32_next(f32x4& c, float a, float b)
 // Geometry by K: a wavefront's 256 accumulation registers hold 16 NBF columns x K values.
 template <int K>
 struct GeomF32 {
-    static_assert(K == 256 || K == 512 || K == 1024, "16 NBF columns x K fp32 values = 256 registers per lane");
+    // (K = 256 would be 64 columns per wavefront; mi_fused_ht_gemm sends it to the GEMV kernels instead,
+    // which are faster on every shape: fused_gemm_f32.hip)
+    static_assert(K == 512 || K == 1024, "16 NBF columns x K fp32 values = 256 registers per lane");
     static constexpr int NBF = 1024 / K;      // 16-column fragments per wavefront
     static constexpr int CPW = 16 * NBF;      // columns per wavefront
     static constexpr int COLS = 4 * CPW;      // columns per workgroup
@@ -74,7 +77,7 @@ constexpr bool area_f32_conflict_free()
                     return false;
     return true;
 }
-static_assert(area_f32_conflict_free<256>() && area_f32_conflict_free<512>() && area_f32_conflict_free<1024>(),
+static_assert(area_f32_conflict_free<512>() && area_f32_conflict_free<1024>(),
               "an LDS access pattern of the fp32 prologue would serialise");
 
 template <int K>
@@ -126,7 +129,7 @@ fused_ht_gemm_xreg_f32_kernel(const float* __restrict__ W, const float* __restri
     // ---- prologue: column f of lane (., lo) = column n0 + CPW w + NBF lo + f ------------------------
     // The wavefront's columns pass through its LDS area in four rounds of 4 NBF columns = eight
     // 512-element tiles (K = 1024: two tiles and one butterfly per column; K = 512: a tile per
-    // column; K = 256: two columns per tile, the tile's high index bit left alone).
+    // column).
     // (yf is an array of scalars, not of 4-vectors: an MFMA names one register, and the compiler
     // keeps a vector's elements in the accumulation-register file only as a whole; with vectors
     // it copied every element into one scratch register right before use, while the previous MFMA
@@ -135,7 +138,7 @@ fused_ht_gemm_xreg_f32_kernel(const float* __restrict__ W, const float* __restri
     {
         unsigned char* area = lds + kAreaBase + wave * kAreaBytes;
         TileOperands<BF16> ops;
-        make_tile_operands<BF16, 4>(K >= 512 ? 9 : 8, ops);
+        make_tile_operands<BF16, 4>(9, ops);
         float in[8][8];
         auto load_tile = [&](int p4, int i) {
 #pragma unroll
@@ -191,14 +194,10 @@ fused_ht_gemm_xreg_f32_kernel(const float* __restrict__ W, const float* __restri
                         // column p: element 512 half + 256 t + 4 lane + r = chunk 128 half + 64 t + lane
                         put(p, 64u * t + lane, a[0][t] + a[1][t]);
                         put(p, 128u + 64u * t + lane, a[0][t] - a[1][t]);
-                    } else if constexpr (K == 512) {
+                    } else {
                         // columns 2 p, 2 p + 1: element 256 t + 4 lane + r
                         put(2 * p, 64u * t + lane, a[0][t]);
                         put(2 * p + 1, 64u * t + lane, a[1][t]);
-                    } else {
-                        // columns 4 p + 2 c + t: element 4 lane + r
-                        put(4 * p + t, lane, a[0][t]);
-                        put(4 * p + 2 + t, lane, a[1][t]);
                     }
                 }
                 cur[0] = nxt[0];
@@ -245,14 +244,9 @@ fused_ht_gemm_xreg_f32_kernel(const float* __restrict__ W, const float* __restri
         const float v0 = acc[mb][0][r];
         if constexpr (NBF == 1) {
             stream_store4(lane_off, __float_as_uint(v0), row_ptr);
-        } else if constexpr (NBF == 2) {
+        } else {
             const float v1 = acc[mb][1][r];
             stream_store8(lane_off, u32x2{__float_as_uint(v0), __float_as_uint(v1)}, row_ptr);
-        } else {
-            const float v1 = acc[mb][1][r], v2 = acc[mb][2][r], v3 = acc[mb][3][r];
-            stream_store16(lane_off,
-                           u32x4{__float_as_uint(v0), __float_as_uint(v1), __float_as_uint(v2), __float_as_uint(v3)},
-                           row_ptr);
         }
     };
     auto store_edge = [&](const f32x4 (&acc)[4][NBF], uint32_t row_base) __attribute__((always_inline)) {
@@ -347,7 +341,7 @@ fused_ht_gemm_xreg_f32_kernel(const float* __restrict__ W, const float* __restri
             store_edge(acc, row_base);
         }
     };
-    if constexpr (NBF <= 2) {
+    {
         // two accumulator sets: a finished block is stored behind the MFMAs of the next one
         f32x4 accA[4][NBF], accB[4][NBF];
         bool pend = false;        // accB holds a finished full row block that is not stored yet
@@ -374,21 +368,6 @@ fused_ht_gemm_xreg_f32_kernel(const float* __restrict__ W, const float* __restri
             }
         }
         if (pend) store_block(accB, pend_base);
-    } else {
-        // one accumulator set (the registers do not hold two): stored right after its block
-        f32x4 acc[4][NBF];
-        auto one = [&](auto second_tag, uint32_t rbi) __attribute__((always_inline)) {
-            row_block_body(std::false_type{}, second_tag, acc, acc, 0, rbi);
-            bool full;
-            uint64_t base;
-            finish(acc, rbi, full, base);
-            if (full) store_block(acc, base);
-        };
-#pragma unroll 1
-        for (uint32_t rbi = 0; rbi < nrb; rbi += 2u) {
-            one(std::false_type{}, rbi);
-            if (rbi + 1u < nrb) one(std::true_type{}, rbi + 1u);
-        }
     }
 }
 
@@ -755,7 +734,7 @@ template <int K>
 int launch_xreg_f32(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, float scale, hipStream_t s)
 {
     using namespace xreg;
-    constexpr uint32_t log2k = K == 256 ? 8 : K == 512 ? 9 : 10;
+    constexpr uint32_t log2k = K == 512 ? 9 : 10;
     const int shift = tile_stage_shift<4>(log2k, false);
     const float fscale = (float)((double)scale * (double)(1u << shift));
     const Plan p = plan(M, N, (uint32_t)GeomF32<K>::COLS, 8u, 9u, 8u);
@@ -784,7 +763,7 @@ int launch_ksplit_f32(const float* W, const float* Xt, float* C, uint32_t M, uin
 }
 }  // namespace
 
-// Called by the fp32 dispatcher of mi_fused_ht_gemm for K = 256 ... 4096 (arguments already
+// Called by the fp32 dispatcher of mi_fused_ht_gemm for K = 512 ... 4096 (arguments already
 // validated).
 int fused_gemm_f32_xreg(const float* W, const float* Xt, float* C, uint32_t M, uint32_t N, uint32_t K,
                         float scale, hipStream_t s)
@@ -792,7 +771,6 @@ int fused_gemm_f32_xreg(const float* W, const float* Xt, float* C, uint32_t M, u
     // W and a row block of C are addressed with 32-bit byte offsets
     if ((uint64_t)M * K * 4u > 0xffffffffull || (uint64_t)N * 4u * 64u > 0xffffffffull) return MI_ERR_SHAPE;
     switch (K) {
-        case 256: return launch_xreg_f32<256>(W, Xt, C, M, N, scale, s);
         case 512: return launch_xreg_f32<512>(W, Xt, C, M, N, scale, s);
         case 1024: return launch_xreg_f32<1024>(W, Xt, C, M, N, scale, s);
         case 2048: return launch_ksplit_f32<2048>(W, Xt, C, M, N, scale, s);

@@ -430,6 +430,12 @@ int launch_any(const float* w, const float* x, float* y, uint32_t M, uint32_t N,
     //   171 -> 139 against this file's kernel with 16 or 32 columns in LDS;
     //   N = 2048 (fused_gemv_stream.hip: the wavefronts split K): (2048, 2048, 512) 73 -> 46.
     const uint64_t groups64 = (uint64_t)((B + kCols - 1) / kCols) * ((M + 63u) / 64u);
+    //   N = 256 (the same kernel with 64 columns per workgroup, which is what 256 registers hold of
+    //   such columns) from 128 pairs of 64 columns x 64 rows on: (1024, 256, 1024) 15.5 -> 11.3 us,
+    //   (2048, 256, 2048) 46.4 -> 24.7, (4096, 256, 4096) 153 -> 72, (1024, 256, 512) 13.6 -> 11.1,
+    //   (512, 256, 1024) 11.0 -> 11.1, (512, 256, 512) 10.7 -> 10.9.
+    if (N == 256u && (uint64_t)((B + 63u) / 64u) * ((M + 63u) / 64u) >= 128u)
+        return launch_rows(w, x, y, M, N, B, scale, columns_contiguous, s);
     if (groups64 >= 256u) {
         if (N == 512u || N == 1024u) return launch_rows(w, x, y, M, N, B, scale, columns_contiguous, s);
         if (N == 2048u) return launch_stream_2048(w, x, y, M, B, scale, columns_contiguous, s);

@@ -27,38 +27,45 @@ using gemv::kXcds;
 using gemv::lds_barrier;
 
 constexpr int kWaves = 4;
-constexpr uint32_t kBlockRows = 64;                // rows of W per row block: 16 per wavefront
-constexpr uint32_t kStageRowBytes = 512;           // eight K steps (8 x 16 floats) of a row
-constexpr uint32_t kStageBytes = 16 * kStageRowBytes;  // 8 KB: a wavefront's 16 rows
-constexpr int kStageSteps = 8;
-constexpr int kSlots = 4;                          // stages in a wavefront's ring
-constexpr int kAhead = 3;                          // stages requested ahead of the MFMAs
-constexpr int kPieces = kStageBytes / 1024;        // transfers (64 lanes x 16 bytes) per stage
-constexpr uint32_t kSlotBytes = kWaves * kStageBytes;       // ring slot s of wavefront w: s * 32 KB + w * 8 KB
-constexpr uint32_t kRingBytes = kSlots * kSlotBytes;        // 128 KB
-constexpr uint32_t kTileBase = 2 * kSlotBytes;              // the column tile lives on top of slots 2 and 3
+constexpr uint32_t kBlockRows = 64;  // rows of W per row block: 16 per wavefront
+constexpr int kSlots = 4;            // stages in a wavefront's ring
+constexpr int kAhead = 3;            // stages requested ahead of the MFMAs
 
-// LDS image of a stage: [16 rows][512 bytes], the 16-byte chunk q of row r stored at q ^ (r & 7).
-// A transfer puts lane l's bytes at 16 l of its kilobyte, so lane l asks for row l / 32 of the
-// transfer's two rows and chunk (l % 32) ^ (row & 7); a fragment read (lane (hi, lo): row lo, chunk
-// 4 ks + hi) then finds eight different 16-byte columns under eight adjacent lanes.
-__host__ __device__ constexpr uint32_t stage_chunk_offset(uint32_t row, uint32_t q)
-{
-    return row * kStageRowBytes + ((q ^ (row & 7u)) << 4);
-}
-constexpr bool stage_patterns_ok()
-{
-    for (uint32_t i = 0; i < (uint32_t)kPieces; ++i)  // the transfers fill every slot of the stage exactly once
-        for (uint32_t l = 0; l < 64; ++l) {
-            const uint32_t row = 2u * i + l / 32u;
-            if (stage_chunk_offset(row, (l % 32u) ^ (row & 7u)) != 1024u * i + 16u * l) return false;
-        }
-    for (uint32_t ks = 0; ks < (uint32_t)kStageSteps; ++ks)
-        if (!lds::conflict_free_b128([=](uint32_t lane) { return stage_chunk_offset(lane & 15u, 4u * ks + (lane >> 4)); }))
-            return false;
-    return true;
-}
-static_assert(stage_patterns_ok(), "the W stage layout does not match its transfers or its reads would serialise");
+// A wavefront's stage: its 16 rows x SS K steps (64 SS bytes of each row: 512 for N >= 512, 256 for
+// N = 256, so that a row block is a multiple of four stages).
+// LDS image: [16 rows][64 SS bytes], the 16-byte chunk q of row r stored at q ^ (r & 7).  A transfer
+// puts lane l's bytes at 16 l of its kilobyte, so lane l asks for row l / (4 SS) of the transfer's
+// rows and chunk (l % (4 SS)) ^ (row & 7): whole 128-byte lines of W.  A fragment read (lane (hi, lo):
+// row lo, chunk 4 ks + hi) then finds eight different 16-byte columns under eight adjacent lanes.
+template <int SS>
+struct Stage {
+    static constexpr uint32_t kRowBytes = 64u * SS;
+    static constexpr uint32_t kBytes = 16u * kRowBytes;
+    static constexpr int kPieces = kBytes / 1024;            // transfers (64 lanes x 16 bytes) per stage
+    static constexpr uint32_t kRowsPerPiece = 1024u / kRowBytes;
+    static constexpr uint32_t kSlotBytes = kWaves * kBytes;  // ring slot s of wavefront w: s * kSlotBytes + w * kBytes
+    static constexpr uint32_t kRingBytes = kSlots * kSlotBytes;
+    static constexpr uint32_t kTileBase = 2 * kSlotBytes;    // the column tile lives on top of slots 2 and 3
+    static_assert(kPieces <= SS, "one transfer of the stage three ahead per K step");
+    static __host__ __device__ constexpr uint32_t chunk_offset(uint32_t row, uint32_t q)
+    {
+        return row * kRowBytes + ((q ^ (row & 7u)) << 4);
+    }
+    static constexpr bool patterns_ok()
+    {
+        for (uint32_t i = 0; i < (uint32_t)kPieces; ++i)  // the transfers fill every slot of the stage exactly once
+            for (uint32_t l = 0; l < 64; ++l) {
+                const uint32_t row = kRowsPerPiece * i + l / (4u * SS);
+                if (chunk_offset(row, (l % (4u * SS)) ^ (row & 7u)) != 1024u * i + 16u * l) return false;
+            }
+        for (uint32_t ks = 0; ks < (uint32_t)SS; ++ks)
+            if (!lds::conflict_free_b128([=](uint32_t lane) { return chunk_offset(lane & 15u, 4u * ks + (lane >> 4)); }))
+                return false;
+        return true;
+    }
+};
+static_assert(Stage<8>::patterns_ok() && Stage<4>::patterns_ok(),
+              "the W stage layout does not match its transfers or its reads would serialise");
 
 // acc (+)= A(16 x 4) * B(4 x 16) with B straight from the accumulation-register file.  Opaque
 // statements: the compiler would otherwise copy every B value into an ordinary register right before
@@ -77,12 +84,14 @@ __device__ __forceinline__ void xmfma_next(f32x4& c, float a, float b)
 
 template <int N, int NC>
 struct RowsGeom {
-    static_assert(N % 512 == 0 && NC % 16 == 0, "whole tiles, whole fragments");
+    static_assert(N % 256 == 0 && NC % 16 == 0, "whole half tiles, whole fragments");
+    static constexpr int SS = N >= 512 ? 8 : 4;           // K steps per stage
+    using St = Stage<SS>;
     static constexpr int NF = NC / 16;                    // 16-column fragments
     static constexpr int STEPS = N / 16;                  // K steps (of 16) per row block
-    static constexpr int STAGES = STEPS / kStageSteps;
+    static constexpr int STAGES = STEPS / SS;
     static constexpr uint32_t kTileBytes = (uint32_t)NC * (N + kPad) * 4u;
-    static constexpr uint32_t kLdsBytes = kTileBase + kTileBytes > kRingBytes ? kTileBase + kTileBytes : kRingBytes;
+    static constexpr uint32_t kLdsBytes = St::kTileBase + kTileBytes > St::kRingBytes ? St::kTileBase + kTileBytes : St::kRingBytes;
     static_assert(STAGES % kSlots == 0, "stage g of every row block lives in ring slot g % 4");
     static_assert(kLdsBytes <= 160u * 1024u, "the tile on top of the last two ring slots fits the LDS");
     static_assert(STEPS * NF * 4 <= 256, "the B operand of a wavefront fits its registers");
@@ -96,9 +105,11 @@ fused_ht_gemv_rows_kernel(const float* __restrict__ W, const float* __restrict__
                           uint32_t row_groups, uint32_t per_xcd, bool col_major)
 {
     using Geo = RowsGeom<N, NC>;
-    constexpr int NF = Geo::NF, STEPS = Geo::STEPS, STAGES = Geo::STAGES;
+    using St = typename Geo::St;
+    constexpr int NF = Geo::NF, STEPS = Geo::STEPS, STAGES = Geo::STAGES, kStageSteps = Geo::SS, kPieces = St::kPieces;
+    constexpr uint32_t kStageBytes = St::kBytes, kSlotBytes = St::kSlotBytes, kStageRowBytes = St::kRowBytes;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    float* const tile = reinterpret_cast<float*>(lds + kTileBase);
+    float* const tile = reinterpret_cast<float*>(lds + St::kTileBase);
     // placement as in fused_gemv.hip: (XCD, slot) takes place XCD * per_xcd + slot of an order of the
     // tiles in which neighbours share a slice of W or, col_major, a column tile
     const uint32_t place = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
@@ -112,13 +123,15 @@ fused_ht_gemv_rows_kernel(const float* __restrict__ W, const float* __restrict__
     // ---- W stream -----------------------------------------------------------------------------------
     const uint32_t ring = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(xreg::lptr_t)lds) + wave * kStageBytes;
     const unsigned char* const ring_ptr = lds + wave * kStageBytes;
-    const uint32_t trow = lane >> 5;
+    constexpr uint32_t kLanesPerRow = 4u * kStageSteps;  // 16-byte chunks of a row in a stage
+    const uint32_t trow = lane / kLanesPerRow;
     uint32_t voff[kPieces];  // lane part of a transfer's address inside the row block being requested
     auto aim = [&](uint32_t mb) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < kPieces; ++i) {
-            const uint32_t row = 2u * i + trow;  // of the wavefront's 16
-            voff[i] = (min(mb + 16u * wave + row, M - 1u) - mb) * (uint32_t)(N * 4) + (((lane & 31u) ^ (row & 7u)) << 4);
+            const uint32_t row = St::kRowsPerPiece * i + trow;  // of the wavefront's 16
+            voff[i] = (min(mb + 16u * wave + row, M - 1u) - mb) * (uint32_t)(N * 4) +
+                      (((lane % kLanesPerRow) ^ (row & 7u)) << 4);
         }
     };
     // the first 512 bytes of a row block's first row (derived from the block's first row every time,
@@ -146,7 +159,10 @@ fused_ht_gemv_rows_kernel(const float* __restrict__ W, const float* __restrict__
         gemv::stage_column_tile<NC, kWaves, N / (16 * kWaves / (NC / 16))>(X, tile, N, B, b0, lane, wave,
                                                                           gemv::first_row_of(blockIdx.x));
     lds_barrier();
-    gemv::transform_column_tile<NC, kWaves>(tile, N, B, b0, scale, lane, wave);
+    if constexpr (N == 256)
+        gemv::transform_column_pairs_256<NC, kWaves>(tile, scale, lane, wave);
+    else
+        gemv::transform_column_tile<NC, kWaves>(tile, N, B, b0, scale, lane, wave);
     lds_barrier();
     // Lane (hi, lo) holds k = 16 step + 4 hi + s of column 16 f + lo for the MFMA with index s.
     float bf[STEPS][NF][4];
@@ -169,7 +185,7 @@ fused_ht_gemv_rows_kernel(const float* __restrict__ W, const float* __restrict__
     // lane part of a fragment read, by parity of the K step inside its stage
     uint32_t frag_at[2];
 #pragma unroll
-    for (int p = 0; p < 2; ++p) frag_at[p] = stage_chunk_offset(lo, 4u * p + hi);
+    for (int p = 0; p < 2; ++p) frag_at[p] = St::chunk_offset(lo, 4u * p + hi);
     auto read_frag = [&](int step) __attribute__((always_inline)) {
         const int ks = step % kStageSteps, stage = step / kStageSteps;
         return *reinterpret_cast<const f32x4*>(ring_ptr + frag_at[ks & 1] + (stage % kSlots) * kSlotBytes + (ks >> 1) * 128u);
@@ -228,7 +244,7 @@ fused_ht_gemv_rows_kernel(const float* __restrict__ W, const float* __restrict__
                         xmfma_first(acc[f][s & 1], fr[t % kFragRing][s], bf[t][f][s]);
                     else
                         xmfma_next(acc[f][s & 1], fr[t % kFragRing][s], bf[t][f][s]);
-            if (ask < STAGES || !LAST) request(ask < STAGES ? block : next_block, ask % STAGES, ks);
+            if (ks < kPieces && (ask < STAGES || !LAST)) request(ask < STAGES ? block : next_block, ask % STAGES, ks);
             __builtin_amdgcn_sched_barrier(0);
         }
         // D[m'][n']: n' = lo is the column, m' = 4 hi + r the row inside the wavefront's 16
@@ -276,7 +292,7 @@ int launch_rows_as(const float* W, const float* X, float* Y, uint32_t M, uint32_
 {
     using Geo = RowsGeom<N, NC>;
     // the tile transform's two MFMA stages attenuate by a power of two that the scale takes back
-    scale = (float)((double)scale * (double)(1u << tile_stage_shift<4>(9u, false)));
+    scale = (float)((double)scale * (double)(1u << tile_stage_shift<4>(N >= 512 ? 9u : 8u, false)));
     auto kern = fused_ht_gemv_rows_kernel<N, NC, XT>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)Geo::kLdsBytes) != hipSuccess)
@@ -304,6 +320,9 @@ int launch_rows(const float* W, const float* X, float* Y, uint32_t M, uint32_t N
     if (N == 512u)
         return columns_contiguous ? launch_rows_as<512, 16, true>(W, X, Y, M, B, scale, s)
                                   : launch_rows_as<512, 16, false>(W, X, Y, M, B, scale, s);
+    if (N == 256u)
+        return columns_contiguous ? launch_rows_as<256, 64, true>(W, X, Y, M, B, scale, s)
+                                  : launch_rows_as<256, 64, false>(W, X, Y, M, B, scale, s);
     return MI_ERR_SIZE;
 }
 

@@ -63,7 +63,7 @@ __device__ __forceinline__ void stage_column_tile(const float* __restrict__ X, f
     // DEPTH rows in flight per thread (DEPTH * RP divides N): the tile is NC * 4 bytes of each of N
     // rows, from the L2
     constexpr int DEPTH = ROWS_AHEAD ? ROWS_AHEAD : 512u / RP;
-    static_assert(DEPTH >= 1 && DEPTH <= 32 && (DEPTH * RP) % 512u == 0, "a round of DEPTH passes covers whole tiles of 512 rows");
+    static_assert(DEPTH >= 1 && DEPTH <= 32 && (DEPTH * RP) % 256u == 0, "a round of DEPTH passes covers whole (half) tiles of rows");
     for (uint32_t rb = r0; rb < N; rb += (uint32_t)DEPTH * RP) {
         f32x4 v[DEPTH];
 #pragma unroll
@@ -190,6 +190,48 @@ __device__ __forceinline__ void transform_column_tile_as(float* tile, uint32_t N
     }
 }
 
+// N = 256: a 512-element tile is two adjacent columns (the operands leave the tile's upper index bit
+// alone).  Wavefront w takes the column pairs w, w + WAVES, ..., two pairs at a time; every column of
+// the tile is transformed, present in X or not (a tile this narrow is only used on large batches).
+template <int NC, int WAVES>
+__device__ __forceinline__ void transform_column_pairs_256(float* tile, float scale, uint32_t lane, uint32_t wave)
+{
+    constexpr uint32_t cstride = 256u + kPad;
+    constexpr int PER_WAVE = NC / 2 / WAVES;  // column pairs per wavefront
+    static_assert(PER_WAVE >= 2 && PER_WAVE % 2 == 0, "pairs are taken two at a time");
+    TileOperands<BF16> ops;
+    make_tile_operands<BF16, 4>(8, ops);
+    auto column = [&](int j, int h) { return tile + (2u * (wave + (uint32_t)WAVES * j) + h) * cstride + 4u * lane; };
+    auto fetch = [&](int j, SplitTileF32& o) __attribute__((always_inline)) {
+        float in[8];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const f32x4 q = *reinterpret_cast<const f32x4*>(column(j, h));
+#pragma unroll
+            for (int r = 0; r < 4; ++r) in[4 * h + r] = q[r];
+        }
+        split_tile_f32(in, o);
+    };
+    SplitTileF32 cur[2], nxt[2];
+    fetch(0, cur[0]);
+    fetch(1, cur[1]);
+#pragma unroll
+    for (int u = 0; u < PER_WAVE / 2; ++u) {
+        if (u + 1 < PER_WAVE / 2) {
+            fetch(2 * u + 2, nxt[0]);
+            fetch(2 * u + 3, nxt[1]);
+        }
+        f32x4 a[2][2];
+        tile_pair_mfma_f32(cur, ops, a);
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) *reinterpret_cast<f32x4*>(column(2 * u + c, h)) = a[c][h] * scale;
+        cur[0] = nxt[0];
+        cur[1] = nxt[1];
+    }
+}
+
 // N = 512, 1024 or 2048
 template <int NC, int WAVES>
 __device__ __forceinline__ void transform_column_tile(float* tile, uint32_t N, uint32_t B, uint32_t b0, float scale,
@@ -256,8 +298,9 @@ inline GemvPlan plan_gemv_rounds(uint32_t M, uint32_t B, uint32_t nc, uint32_t b
 int launch_stream_2048(const float* W, const float* X, float* Y, uint32_t M, uint32_t B, float scale,
                        bool columns_contiguous, hipStream_t s);
 
-// N = 512 and 1024 with the whole B operand in every wavefront's registers, the wavefronts splitting
-// the rows (fused_gemv_rows.hip); same contract.
+// N = 256, 512 and 1024 with the whole B operand in every wavefront's registers, the wavefronts
+// splitting the rows (fused_gemv_rows.hip: 64 columns per workgroup for N = 256, 16 otherwise); same
+// contract.
 int launch_rows(const float* W, const float* X, float* Y, uint32_t M, uint32_t N, uint32_t B, float scale,
                 bool columns_contiguous, hipStream_t s);
 

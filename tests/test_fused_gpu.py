@@ -61,13 +61,18 @@ def test_gemv_reference_self_check(pkg, oracle, M, N, B):
 # and a last block of four rows, (8192, 512, 40) with a long walk over row blocks.  N = 2048 (the
 # wavefronts split K, sums meet in LDS): (2048, 2048, 512), (1100, 2048, 531), (4100, 2048, 130),
 # (300, 2048, 1024) with a second row block that is the last and ragged, (20000, 2048, 24) with three
-# blocks per workgroup, (16384, 2048, 16) with one column group.
+# blocks per workgroup, (16384, 2048, 16) with one column group.  N = 256 from 128 pairs of 64 columns
+# x 64 rows on runs the row-split kernel with 64 columns per workgroup (two columns per 512-element
+# tile of the transform): (4096, 256, 4096), (1000, 256, 1100) ragged both ways, (130, 256, 9000) with
+# more column groups than row blocks, (8192, 256, 100) with two column groups, the second of 36
+# columns, (512, 256, 1024) right at the threshold.
 @pytest.mark.parametrize("M,N,B", [(1024, 1024, 256), (1024, 1024, 512), (1024, 1024, 128),
                                    (4096, 256, 4096), (2000, 64, 1000), (4100, 2048, 130),
                                    (1024, 1024, 2048), (1000, 512, 700), (1100, 1024, 531),
                                    (2048, 2048, 512), (1100, 2048, 531), (300, 2048, 1024),
                                    (20000, 2048, 24), (8192, 512, 40), (16384, 2048, 16),
-                                   (512, 512, 1024), (64, 1024, 4096), (4100, 1024, 130)])
+                                   (512, 512, 1024), (64, 1024, 4096), (4100, 1024, 130),
+                                   (1000, 256, 1100), (130, 256, 9000), (8192, 256, 100), (512, 256, 1024)])
 def test_gemv_large_launch_paths(pkg, oracle, M, N, B):
     W, X = oracle.inputs_gemv(M, N, B)
     Y = pkg.fused_ht_gemv(W.cuda(), X.cuda())
@@ -113,8 +118,8 @@ def test_gemv_random_large_shapes(pkg, oracle):
     # more column groups than one round of workgroups.  Checked on sampled rows and by column sums.
     rng = np.random.default_rng(20251126)
     g = torch.Generator().manual_seed(11)
-    for _ in range(24):
-        N = int(rng.choice([512, 1024, 2048]))
+    for _ in range(32):
+        N = int(rng.choice([256, 512, 1024, 2048]))
         M = int(rng.choice([64, 65, 127, 200, 256, 300, 513, 1000, 1024, 1500, 2048, 3000, 5000]))
         B = int(rng.choice([16, 17, 33, 64, 100, 255, 256, 260, 511, 528, 1000, 1024, 2049, 4100]))
         if M * B > 6_000_000:
@@ -283,8 +288,10 @@ def test_gemm_k1024_launch_plans(pkg, oracle, M, N, K):
     assert _rel(oracle, C[idx], want) <= 2e-2
 
 
-# fp32 at K = 256, 512, 1024 runs the register-resident fp32 kernel: groups of 65536 / K columns,
-# 64-row blocks, one store of 1024 / K adjacent columns per lane and row; K = 2048 and 4096 its
+# fp32 at K = 512 and 1024 runs the register-resident fp32 kernel on these shapes (too few 16-column
+# x 64-row pairs for the GEMV route, all but (700, 1023)): groups of 65536 / K columns, 64-row
+# blocks, one store of 1024 / K adjacent columns per lane and row; K = 256 runs the GEMV kernels
+# (test_gemm_f32_small_k_both_routes has more of those); K = 2048 and 4096 the register-resident
 # variant with the K range split over pairs of wavefronts (groups of 32 columns; K = 4096 in two
 # phases, the second adding to what the first stored).  Shapes around every tile
 # boundary (edge store path, N that rules out vector stores, one row block, odd and even numbers of
@@ -354,9 +361,10 @@ def test_gemm_f32_through_gemv_kernels(pkg, oracle, M, N, K):
     assert _rel(oracle, C[idx], want) <= 1e-5
 
 
-# fp32, K <= 256: outputs up to 1536 x 1024 run the GEMV kernel (register-butterfly prologue reading
-# X column by column), larger ones the GEMM kernels (LDS tile for K <= 128, register-resident for
-# K = 256).  Shapes on both sides of the limit, ragged in both directions, and the smallest.
+# fp32, K <= 128: outputs up to 1536 x 1024 run the GEMV kernel (register-butterfly prologue reading
+# X column by column), larger ones the LDS-tile GEMM kernel; K = 256 runs the GEMV kernels on every
+# shape (the row-split one with 64 columns per workgroup from 128 pairs of 64 columns x 64 rows on).
+# Shapes on both sides of the limits, ragged in both directions, and the smallest.
 @pytest.mark.parametrize("K", [32, 64, 128, 256])
 @pytest.mark.parametrize("M,N", [(1, 1), (33, 7), (512, 512), (700, 1023), (1024, 1536), (1025, 1536), (2048, 1024),
                                  (130, 4100)])
