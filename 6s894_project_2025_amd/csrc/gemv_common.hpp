@@ -120,6 +120,10 @@ __device__ __forceinline__ void stage_column_tile_xt(const float* __restrict__ X
 // the end of X are left as they are: a column of the B operand reaches only its own column of the
 // product, which is not stored.  `scale` carries the power of two that the two MFMA stages take
 // out (tile_stage_shift<4>(9, false)).
+// (A pair of tiles is 28 MFMAs and about 136 other instructions, and a wavefront that has its SIMD
+// to itself issues one instruction per eight cycles: 1 300 cycles of issue before any wait, whatever
+// the order.  Handing the next pair's split out evenly between the MFMAs with scheduling groups,
+// three vector instructions behind each bf16 MFMA and five behind each fp32 one, changed nothing.)
 template <int NT, int NC, int WAVES>
 __device__ __forceinline__ void transform_column_tile_as(float* tile, uint32_t N, uint32_t B, uint32_t b0,
                                                          float scale, uint32_t lane, uint32_t wave)
