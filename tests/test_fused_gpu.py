@@ -161,6 +161,18 @@ def test_gemv_w_beyond_4_gib(pkg, oracle, M, N):
     assert worst / math.sqrt(N) <= 1e-4, worst          # (fp32 against fp32: summation orders differ)
 
 
+@pytest.mark.parametrize("M,N,B", [(1, 1024, 4096), (1, 2048, 4096), (1, 256, 8192), (3, 512, 4100), (17, 2048, 4097)])
+def test_gemv_few_rows_many_columns(pkg, oracle, M, N, B):
+    # the large-shape kernels with less than one 16-row fragment of W: every wavefront's rows past
+    # the end are clamped to the last row for the loads and masked at the store
+    W, X = oracle.inputs_gemv(M, N, B)
+    Y = pkg.fused_ht_gemv(W.cuda(), X.cuda())
+    torch.cuda.synchronize()
+    want = oracle.fused_ht_gemv_f64_blas(W.double().numpy(), X.double().numpy(), 1.0 / math.sqrt(N))
+    assert Y.shape == (M, B)
+    assert _rel(oracle, Y, want) <= 1e-5
+
+
 def test_gemv_identity_reduces_to_transform(pkg, oracle):
     N, B = 256, 48
     _, X = oracle.inputs_gemv(N, N, B)
