@@ -125,7 +125,10 @@ __device__ __forceinline__ void stage_column_tile_xt(const float* __restrict__ X
 // the order.  Handing the next pair's split out evenly between the MFMAs with scheduling groups,
 // three vector instructions behind each bf16 MFMA and five behind each fp32 one, changed nothing;
 // nor did stage 1 on the fp32 matrix cores, eight MFMAs of 32 cycles on the unsplit data instead of
-// three of 16 on the pieces: 48 MFMAs a pair, 1 536 cycles, the same 0.8 us.)
+// three of 16 on the pieces: 48 MFMAs a pair, 1 536 cycles, the same 0.8 us; with a column's
+// butterflies, scale and write-back handed out between the next column's MFMAs as well, N = 1024
+// went from 3.2 to 2.9 us per four columns and N = 2048 from 6.5 to 7.2; one tile of a pair in each
+// form, 1 120 cycles of matrix core beside a hundred other instructions, measured 3.2 and 6.8.)
 template <int NT, int NC, int WAVES>
 __device__ __forceinline__ void transform_column_tile_as(float* tile, uint32_t N, uint32_t B, uint32_t b0,
                                                          float scale, uint32_t lane, uint32_t wave)
